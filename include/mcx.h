@@ -1,0 +1,174 @@
+/*
+ * mcx.h -- C ABI of the MI355X (gfx950) mapped-convolution backend.
+ *
+ * One shared library, libmcx_hip.so, exports the functions below.  They are
+ * what the reference's Python layers reach through its pybind modules
+ * (`_mapped_convolution_ext._*`), re-cut as plain C: device pointers, sizes and
+ * an explicit stream; no tensor types.  Citations name the reference interface
+ * each entry point replaces (paths relative to package/ext_modules/).
+ *
+ * Conventions
+ *   - All pointers are DEVICE pointers to contiguous row-major buffers, laid
+ *     out exactly like the reference's tensors (NCHW data, [H,W,K,(P,)2] maps).
+ *   - `stream` is a hipStream_t passed as void*; NULL is the default stream.
+ *     Calls only enqueue work; they never synchronise or allocate.
+ *   - `dtype` selects the data scalar: MCX_F32, MCX_F64, or MCX_BF16
+ *     (convolution entry points only; accumulation is fp32).  sample_map and
+ *     interp_weights have the data's type for F32/F64 and are float for BF16.
+ *   - `interp`: 0 nearest (also any other value), 1 bilinear, 2 bispherical
+ *     (include/core/resample.h:62-90).
+ *   - `P` is the number of interpolation points per tap: 0 means "no
+ *     interp_weights" (iw must be NULL, map is [..,K,2]); P >= 1 selects the
+ *     weighted form (map [..,K,P,2], iw [..,K,P]).
+ *   - Scatter-type outputs (gx, tconv y, resample_to_map out, unpool gin) are
+ *     fully overwritten: the library clears them itself before accumulating.
+ *   - Return value: 0 on success; a positive hipError_t if a launch failed; a
+ *     negative MCX_E_* for rejected arguments.  Nothing aborts the process.
+ *   - Thread safety: no global mutable state; concurrent calls on different
+ *     streams are independent as long as their output buffers are.
+ */
+#ifndef MCX_H_
+#define MCX_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { MCX_F32 = 0, MCX_F64 = 1, MCX_BF16 = 2 };
+
+enum {
+  MCX_OK = 0,
+  MCX_E_DTYPE = -1,     /* dtype not supported by this entry point */
+  MCX_E_SHAPE = -2,     /* a size is negative, zero where it may not be, or too large */
+  MCX_E_NULL = -3,      /* a required pointer is NULL (or iw/P disagree) */
+  MCX_E_WORKSPACE = -4  /* workspace missing or too small */
+};
+
+/* Library identification; bumps when a signature changes. */
+int mcx_abi_version(void);
+/* Human-readable text for a return code of any function below. */
+const char *mcx_error_string(int code);
+
+/* ---- Resample / Unresample ------------------------------------------------ */
+
+/* resample_from_map (+ weighted_resample_from_map):
+ * include/nn/layers/resample_layer.h:60-61,85 and weighted_resample_layer.h:78-81;
+ * kernels include/nn/cuda/resample.cuh:49-61,124-139.
+ * dst[b,c,i,j] = sample(src[b,c,:,:], map[i,j]);  src [B,C,SH,SW], map [MH,MW,(P,)2],
+ * iw [MH,MW,P] or NULL, dst [B,C,MH,MW]. */
+int mcx_resample_from_map(const void *src, const void *map, const void *iw, void *dst,
+                          int64_t B, int64_t C, int64_t SH, int64_t SW, int64_t MH, int64_t MW,
+                          int64_t P, int interp, int dtype, void *stream);
+
+/* resample_to_map (+ weighted_resample_to_map):
+ * include/nn/layers/resample_layer.h:38-40,83 and weighted_resample_layer.h:49-54;
+ * kernels include/nn/cuda/resample.cuh:14-26,85-99.
+ * out (cleared here) accumulates every input pixel at map[y_in,x_in];
+ * in [B,C,IH,IW], map [IH,IW,(P,)2], out [B,C,OH,OW]. */
+int mcx_resample_to_map(const void *in, const void *map, const void *iw, void *out,
+                        int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t OH, int64_t OW,
+                        int64_t P, int interp, int dtype, void *stream);
+
+/* ---- Pooling --------------------------------------------------------------- */
+
+/* mapped_max_pool (+ weighted): include/nn/layers/mapped_max_pooling_layer.h:46-49,101,
+ * weighted_mapped_max_pooling_layer.h:42-44; kernels include/nn/cuda/mapped_max_pool.cuh:15-31,99-117.
+ * in [B,C,IH,IW], map [OH,OW,K,(P,)2] -> out [B,C,OH,OW], idx int64 [B,C,OH,OW]
+ * (element offset of the winning tap inside the flattened map; -1 if none). */
+int mcx_max_pool(const void *in, const void *map, const void *iw, void *out, int64_t *idx,
+                 int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t OH, int64_t OW,
+                 int64_t K, int64_t P, int interp, int dtype, void *stream);
+
+/* mapped_max_unpool (+ weighted): mapped_max_pooling_layer.h:69-73,103,
+ * weighted_mapped_max_pooling_layer.h:67-70; kernels mapped_max_pool.cuh:56-70,144-159.
+ * gout, idx [B,C,OH,OW] -> gin [B,C,IH,IW] (cleared here). */
+int mcx_max_unpool(const void *gout, const int64_t *idx, const void *map, const void *iw,
+                   void *gin, int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t OH,
+                   int64_t OW, int64_t K, int64_t P, int interp, int dtype, void *stream);
+
+/* mapped_avg_pool (+ weighted): include/nn/layers/mapped_avg_pooling_layer.h:42-44,91-94,
+ * weighted_mapped_avg_pooling_layer.h:48-52; kernels include/nn/cuda/mapped_avg_pool.cuh:15-27,91-106. */
+int mcx_avg_pool(const void *in, const void *map, const void *iw, void *out, int64_t B,
+                 int64_t C, int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
+                 int64_t P, int interp, int dtype, void *stream);
+
+/* mapped_avg_unpool (+ weighted): mapped_avg_pooling_layer.h:64-67,
+ * weighted_mapped_avg_pooling_layer.h:75-78; kernels mapped_avg_pool.cuh:50-63,131-145. */
+int mcx_avg_unpool(const void *gout, const void *map, const void *iw, void *gin, int64_t B,
+                   int64_t C, int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
+                   int64_t P, int interp, int dtype, void *stream);
+
+/* ---- Mapped convolution ---------------------------------------------------- */
+
+/* mapped_conv_forward (+ weighted_mapped_conv_forward):
+ * include/nn/layers/mapped_convolution_layer.h:64-66,141,
+ * weighted_mapped_convolution_layer.h:65-68,153; host driver
+ * src/nn/cuda/mapped_convolution_layer.cu:16-73.
+ * x [B,Ci,IH,IW], map [OH,OW,K,(P,)2], w [Co,Ci,K], bias [Co] -> y [B,Co,OH,OW].
+ * The gather, the product with w and the bias are one fused kernel; no column
+ * buffer exists. */
+int mcx_conv_forward(const void *x, const void *map, const void *iw, const void *w,
+                     const void *bias, void *y, int64_t B, int64_t Ci, int64_t Co, int64_t IH,
+                     int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
+                     int dtype, void *stream);
+
+/* Bytes of scratch mcx_conv_backward needs for these sizes (may be 0). */
+size_t mcx_conv_backward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t IH, int64_t IW,
+                                   int64_t OH, int64_t OW, int64_t K, int64_t P, int dtype);
+
+/* mapped_conv_backward (+ weighted): mapped_convolution_layer.h:90-135,143,
+ * weighted_mapped_convolution_layer.h:97-100,156; host drivers
+ * src/nn/cuda/mapped_convolution_layer.cu:75-193.
+ * gy [B,Co,OH,OW], x, w as above -> gx [B,Ci,IH,IW] (cleared here),
+ * gw [Co,Ci,K], gb [Co] (= gy summed over b,h,w).  Any of gx, gw, gb may be
+ * NULL to skip that gradient.  workspace: device scratch of at least
+ * mcx_conv_backward_workspace(...) bytes, 256-byte aligned. */
+int mcx_conv_backward(const void *gy, const void *map, const void *iw, const void *x,
+                      const void *w, void *gx, void *gw, void *gb, void *workspace,
+                      size_t workspace_bytes, int64_t B, int64_t Ci, int64_t Co, int64_t IH,
+                      int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
+                      int dtype, void *stream);
+
+/* mapped_transposed_conv_forward (+ weighted):
+ * include/nn/layers/mapped_transposed_convolution_layer.h:64-69,148,
+ * weighted_mapped_transposed_convolution_layer.h:64-67; host driver
+ * src/nn/cuda/mapped_transposed_convolution_layer.cu:53-110.
+ * x [B,Ci,IH,IW], map [IH,IW,K,(P,)2] pointing into the OUTPUT, w [Ci,Co,K],
+ * bias [Co] -> y [B,Co,OH,OW] (initialised to the bias here, then accumulated). */
+int mcx_tconv_forward(const void *x, const void *map, const void *iw, const void *w,
+                      const void *bias, void *y, int64_t B, int64_t Ci, int64_t Co, int64_t IH,
+                      int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
+                      int dtype, void *stream);
+
+size_t mcx_tconv_backward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t IH, int64_t IW,
+                                    int64_t OH, int64_t OW, int64_t K, int64_t P, int dtype);
+
+/* mapped_transposed_conv_backward (+ weighted):
+ * mapped_transposed_convolution_layer.h:97-100,150,
+ * weighted_mapped_transposed_convolution_layer.h:98-100; host drivers
+ * src/nn/cuda/mapped_transposed_convolution_layer.cu:112-220.
+ * gy [B,Co,OH,OW] -> gx [B,Ci,IH,IW], gw [Ci,Co,K], gb [Co]; NULL skips. */
+int mcx_tconv_backward(const void *gy, const void *map, const void *iw, const void *x,
+                       const void *w, void *gx, void *gw, void *gb, void *workspace,
+                       size_t workspace_bytes, int64_t B, int64_t Ci, int64_t Co, int64_t IH,
+                       int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
+                       int dtype, void *stream);
+
+/* ---- KNN -------------------------------------------------------------------- */
+
+/* knn_forward: include/util/layers/knn_layer.h:25-35,41; kernels
+ * include/util/cuda/knn.cuh:43-275; host src/util/cuda/knn_layer.cu:13-32.
+ * ref [B,D,R], query [B,D,Q] (points are columns) -> idx int64 [B,k,Q]
+ * (1-based reference index, row j = j-th nearest, ties keep the lower index),
+ * dist [B,k,Q] (Euclidean).  k <= 64; F32 and F64.  The R x Q distance matrix
+ * of the reference is never formed. */
+int mcx_knn(const void *ref, const void *query, int64_t *idx, void *dist, int64_t B, int64_t D,
+            int64_t R, int64_t Q, int64_t k, int dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MCX_H_ */

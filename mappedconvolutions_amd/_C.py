@@ -1,0 +1,437 @@
+"""The extension-op boundary of the mapped-convolution backend.
+
+Same op names, argument order and return values as the reference's pybind
+modules under `_mapped_convolution_ext` (one module per op family there, one
+namespace here); each function checks its tensors like the reference's
+include/nn/layers/*.h wrappers do, allocates the outputs with torch, and calls
+the C ABI of libmcx_hip.so on the current HIP stream.  Tensors must live on the
+GPU: there is no CPU implementation behind these names.
+"""
+import torch
+
+from . import _lib
+from ._lib import MCX_BF16, MCX_F32, MCX_F64
+
+_DTYPES = {torch.float32: MCX_F32, torch.float64: MCX_F64, torch.bfloat16: MCX_BF16}
+
+
+def _contig(**tensors):
+    for name, t in tensors.items():
+        if t is not None and not t.is_contiguous():
+            raise RuntimeError("%s must be contiguous" % name)
+
+
+def _on_gpu(ref_name, ref, **tensors):
+    if not ref.is_cuda:
+        raise RuntimeError(
+            "%s must be a GPU tensor: this backend has no CPU implementation" % ref_name)
+    for name, t in tensors.items():
+        if t is not None and t.device != ref.device:
+            raise RuntimeError("%s must be on the same device as %s" % (name, ref_name))
+
+
+def _dtype(data, maps=(), same=()):
+    """Data dtype code.  Maps share the data's dtype (the reference's rule,
+    layers/nn/layer_utils.py:21-30), except bf16 data which takes fp32 maps
+    because bf16 cannot hold pixel coordinates above 256 exactly."""
+    if data.dtype not in _DTYPES:
+        raise RuntimeError("unsupported dtype %s" % data.dtype)
+    want_map = torch.float32 if data.dtype == torch.bfloat16 else data.dtype
+    for m in maps:
+        if m is not None and m.dtype != want_map:
+            raise RuntimeError("sample_map / interp_weights must be %s for %s data (got %s)" %
+                               (want_map, data.dtype, m.dtype))
+    for t in same:
+        if t is not None and t.dtype != data.dtype:
+            raise RuntimeError("tensor dtypes differ: %s vs %s" % (t.dtype, data.dtype))
+    return _DTYPES[data.dtype]
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _stream(t):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _weighted_dims(sample_map, interp_weights, kernel):
+    """Number of interpolation points P (0 = unweighted) after a shape check."""
+    want = (4 if kernel else 3) + (0 if interp_weights is None else 1)
+    if sample_map.dim() != want or sample_map.shape[-1] != 2:
+        raise RuntimeError("sample_map has shape %s, expected %d dims ending in 2" %
+                           (tuple(sample_map.shape), want))
+    if interp_weights is None:
+        return 0
+    if tuple(interp_weights.shape) != tuple(sample_map.shape[:-1]):
+        raise RuntimeError("interp_weights shape %s does not match sample_map %s" %
+                           (tuple(interp_weights.shape), tuple(sample_map.shape)))
+    return int(interp_weights.shape[-1])
+
+
+# --------------------------------------------------------------------------- conv
+def _conv_forward(input, sample_map, interp_weights, weight, bias, kernel_size, interpolation):
+    _contig(input=input, sample_map=sample_map, interp_weights=interp_weights, weight=weight,
+            bias=bias)
+    _on_gpu("input", input, sample_map=sample_map, interp_weights=interp_weights, weight=weight,
+            bias=bias)
+    dt = _dtype(input, maps=(sample_map, interp_weights), same=(weight, bias))
+    P = _weighted_dims(sample_map, interp_weights, True)
+    B, Ci, IH, IW = input.shape
+    Co = weight.shape[0]
+    OH, OW, K = sample_map.shape[0], sample_map.shape[1], int(kernel_size)
+    if weight.dim() != 3 or weight.shape[1] != Ci or weight.shape[2] != K or sample_map.shape[2] != K:
+        raise RuntimeError("weight %s / sample_map %s do not match input channels %d, kernel %d" %
+                           (tuple(weight.shape), tuple(sample_map.shape), Ci, K))
+    if bias.numel() != Co:
+        raise RuntimeError("bias must have %d elements" % Co)
+    out = torch.empty((B, Co, OH, OW), dtype=input.dtype, device=input.device)
+    with torch.cuda.device(input.device):
+        rc = _lib.load().mcx_conv_forward(_ptr(input), _ptr(sample_map), _ptr(interp_weights),
+                                          _ptr(weight), _ptr(bias), _ptr(out), B, Ci, Co, IH, IW,
+                                          OH, OW, K, P, int(interpolation), dt, _stream(input))
+    _lib.check(rc, "mapped_conv_forward")
+    return out
+
+
+def _conv_backward(grad_output, sample_map, interp_weights, input, weight, bias, kernel_size,
+                   interpolation):
+    _contig(input=input, sample_map=sample_map, interp_weights=interp_weights, weight=weight,
+            bias=bias)
+    grad_output = grad_output.contiguous()  # the reference reads it raw without a check
+    _on_gpu("grad_output", grad_output, input=input, sample_map=sample_map,
+            interp_weights=interp_weights, weight=weight, bias=bias)
+    dt = _dtype(input, maps=(sample_map, interp_weights), same=(weight, grad_output))
+    P = _weighted_dims(sample_map, interp_weights, True)
+    B, Ci, IH, IW = input.shape
+    Co, OH, OW = grad_output.shape[1], grad_output.shape[2], grad_output.shape[3]
+    K = int(kernel_size)
+    if tuple(weight.shape) != (Co, Ci, K) or tuple(sample_map.shape[:3]) != (OH, OW, K):
+        raise RuntimeError("shape mismatch in mapped_conv_backward")
+    grad_input = torch.empty_like(input)
+    grad_weight = torch.empty_like(weight)
+    grad_bias = torch.empty((Co,), dtype=input.dtype, device=input.device)
+    lib = _lib.load()
+    ws_bytes = lib.mcx_conv_backward_workspace(B, Ci, Co, IH, IW, OH, OW, K, P, dt)
+    ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=input.device)
+    with torch.cuda.device(input.device):
+        rc = lib.mcx_conv_backward(_ptr(grad_output), _ptr(sample_map), _ptr(interp_weights),
+                                   _ptr(input), _ptr(weight), _ptr(grad_input), _ptr(grad_weight),
+                                   _ptr(grad_bias), _ptr(ws), ws_bytes, B, Ci, Co, IH, IW, OH, OW,
+                                   K, P, int(interpolation), dt, _stream(input))
+    _lib.check(rc, "mapped_conv_backward")
+    return [grad_input, grad_weight, grad_bias]
+
+
+def mapped_conv_forward(input, sample_map, weight, bias, kernel_size, interpolation):
+    """include/nn/layers/mapped_convolution_layer.h:64-66."""
+    return _conv_forward(input, sample_map, None, weight, bias, kernel_size, interpolation)
+
+
+def mapped_conv_backward(grad_output, sample_map, input, weight, bias, kernel_size, interpolation):
+    """include/nn/layers/mapped_convolution_layer.h:90-93 -> [grad_input, grad_weight, grad_bias]."""
+    return _conv_backward(grad_output, sample_map, None, input, weight, bias, kernel_size,
+                          interpolation)
+
+
+def weighted_mapped_conv_forward(input, sample_map, interp_weights, weight, bias, kernel_size,
+                                 interpolation):
+    """include/nn/layers/weighted_mapped_convolution_layer.h:65-68."""
+    return _conv_forward(input, sample_map, interp_weights, weight, bias, kernel_size,
+                         interpolation)
+
+
+def weighted_mapped_conv_backward(grad_output, sample_map, interp_weights, input, weight, bias,
+                                  kernel_size, interpolation):
+    """include/nn/layers/weighted_mapped_convolution_layer.h:97-100."""
+    return _conv_backward(grad_output, sample_map, interp_weights, input, weight, bias,
+                          kernel_size, interpolation)
+
+
+# ---------------------------------------------------------------- transposed conv
+def _tconv_forward(input, sample_map, interp_weights, weight, bias, output_height, output_width,
+                   kernel_size, interpolation):
+    _contig(input=input, sample_map=sample_map, interp_weights=interp_weights, weight=weight,
+            bias=bias)
+    _on_gpu("input", input, sample_map=sample_map, interp_weights=interp_weights, weight=weight,
+            bias=bias)
+    dt = _dtype(input, maps=(sample_map, interp_weights), same=(weight, bias))
+    P = _weighted_dims(sample_map, interp_weights, True)
+    B, Ci, IH, IW = input.shape
+    Co, K = weight.shape[1], int(kernel_size)
+    OH, OW = int(output_height), int(output_width)
+    if tuple(weight.shape) != (Ci, Co, K) or tuple(sample_map.shape[:3]) != (IH, IW, K):
+        raise RuntimeError("shape mismatch in mapped_transposed_conv_forward")
+    out = torch.empty((B, Co, OH, OW), dtype=input.dtype, device=input.device)
+    with torch.cuda.device(input.device):
+        rc = _lib.load().mcx_tconv_forward(_ptr(input), _ptr(sample_map), _ptr(interp_weights),
+                                           _ptr(weight), _ptr(bias), _ptr(out), B, Ci, Co, IH, IW,
+                                           OH, OW, K, P, int(interpolation), dt, _stream(input))
+    _lib.check(rc, "mapped_transposed_conv_forward")
+    return out
+
+
+def _tconv_backward(grad_output, sample_map, interp_weights, input, weight, bias, kernel_size,
+                    interpolation):
+    _contig(input=input, sample_map=sample_map, interp_weights=interp_weights, weight=weight,
+            bias=bias)
+    grad_output = grad_output.contiguous()
+    _on_gpu("grad_output", grad_output, input=input, sample_map=sample_map,
+            interp_weights=interp_weights, weight=weight, bias=bias)
+    dt = _dtype(input, maps=(sample_map, interp_weights), same=(weight, grad_output))
+    P = _weighted_dims(sample_map, interp_weights, True)
+    B, Ci, IH, IW = input.shape
+    Co, OH, OW = grad_output.shape[1], grad_output.shape[2], grad_output.shape[3]
+    K = int(kernel_size)
+    if tuple(weight.shape) != (Ci, Co, K) or tuple(sample_map.shape[:3]) != (IH, IW, K):
+        raise RuntimeError("shape mismatch in mapped_transposed_conv_backward")
+    grad_input = torch.empty_like(input)
+    grad_weight = torch.empty_like(weight)
+    grad_bias = torch.empty((Co,), dtype=input.dtype, device=input.device)
+    lib = _lib.load()
+    ws_bytes = lib.mcx_tconv_backward_workspace(B, Ci, Co, IH, IW, OH, OW, K, P, dt)
+    ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=input.device)
+    with torch.cuda.device(input.device):
+        rc = lib.mcx_tconv_backward(_ptr(grad_output), _ptr(sample_map), _ptr(interp_weights),
+                                    _ptr(input), _ptr(weight), _ptr(grad_input), _ptr(grad_weight),
+                                    _ptr(grad_bias), _ptr(ws), ws_bytes, B, Ci, Co, IH, IW, OH, OW,
+                                    K, P, int(interpolation), dt, _stream(input))
+    _lib.check(rc, "mapped_transposed_conv_backward")
+    return [grad_input, grad_weight, grad_bias]
+
+
+def mapped_transposed_conv_forward(input, sample_map, weight, bias, output_height, output_width,
+                                   kernel_size, interpolation):
+    """include/nn/layers/mapped_transposed_convolution_layer.h:64-69."""
+    return _tconv_forward(input, sample_map, None, weight, bias, output_height, output_width,
+                          kernel_size, interpolation)
+
+
+def mapped_transposed_conv_backward(grad_output, sample_map, input, weight, bias, kernel_size,
+                                    interpolation):
+    """include/nn/layers/mapped_transposed_convolution_layer.h:97-100."""
+    return _tconv_backward(grad_output, sample_map, None, input, weight, bias, kernel_size,
+                           interpolation)
+
+
+def weighted_mapped_transposed_conv_forward(input, sample_map, interp_weights, weight, bias,
+                                            output_height, output_width, kernel_size,
+                                            interpolation):
+    """include/nn/layers/weighted_mapped_transposed_convolution_layer.h:64-67."""
+    return _tconv_forward(input, sample_map, interp_weights, weight, bias, output_height,
+                          output_width, kernel_size, interpolation)
+
+
+def weighted_mapped_transposed_conv_backward(grad_output, sample_map, interp_weights, input,
+                                             weight, bias, kernel_size, interpolation):
+    """include/nn/layers/weighted_mapped_transposed_convolution_layer.h:98-100."""
+    return _tconv_backward(grad_output, sample_map, interp_weights, input, weight, bias,
+                           kernel_size, interpolation)
+
+
+# ------------------------------------------------------------------------ pooling
+def _pool_dims(input, sample_map, interp_weights, kernel_size):
+    P = _weighted_dims(sample_map, interp_weights, True)
+    K = int(kernel_size)
+    if sample_map.shape[2] != K:
+        raise RuntimeError("sample_map kernel dimension %d != kernel_size %d" %
+                           (sample_map.shape[2], K))
+    return P, K
+
+
+def _max_pool(input, sample_map, interp_weights, kernel_size, interpolation):
+    _contig(input=input, sample_map=sample_map, interp_weights=interp_weights)
+    _on_gpu("input", input, sample_map=sample_map, interp_weights=interp_weights)
+    dt = _dtype(input, maps=(sample_map, interp_weights))
+    P, K = _pool_dims(input, sample_map, interp_weights, kernel_size)
+    B, C, IH, IW = input.shape
+    OH, OW = sample_map.shape[0], sample_map.shape[1]
+    out = torch.empty((B, C, OH, OW), dtype=input.dtype, device=input.device)
+    idx = torch.empty((B, C, OH, OW), dtype=torch.int64, device=input.device)
+    with torch.cuda.device(input.device):
+        rc = _lib.load().mcx_max_pool(_ptr(input), _ptr(sample_map), _ptr(interp_weights),
+                                      _ptr(out), _ptr(idx), B, C, IH, IW, OH, OW, K, P,
+                                      int(interpolation), dt, _stream(input))
+    _lib.check(rc, "mapped_max_pool")
+    return [out, idx]
+
+
+def _max_unpool(grad_output, idx_mask, sample_map, interp_weights, input_height, input_width,
+                kernel_size, interpolation):
+    _contig(grad_output=grad_output, idx_mask=idx_mask, sample_map=sample_map,
+            interp_weights=interp_weights)
+    _on_gpu("grad_output", grad_output, idx_mask=idx_mask, sample_map=sample_map,
+            interp_weights=interp_weights)
+    dt = _dtype(grad_output, maps=(sample_map, interp_weights))
+    if idx_mask.dtype != torch.int64 or idx_mask.shape != grad_output.shape:
+        raise RuntimeError("idx_mask must be int64 with grad_output's shape")
+    P, K = _pool_dims(grad_output, sample_map, interp_weights, kernel_size)
+    B, C, OH, OW = grad_output.shape
+    IH, IW = int(input_height), int(input_width)
+    gin = torch.empty((B, C, IH, IW), dtype=grad_output.dtype, device=grad_output.device)
+    with torch.cuda.device(grad_output.device):
+        rc = _lib.load().mcx_max_unpool(_ptr(grad_output), _ptr(idx_mask), _ptr(sample_map),
+                                        _ptr(interp_weights), _ptr(gin), B, C, IH, IW, OH, OW, K,
+                                        P, int(interpolation), dt, _stream(grad_output))
+    _lib.check(rc, "mapped_max_unpool")
+    return gin
+
+
+def _avg_pool(input, sample_map, interp_weights, kernel_size, interpolation):
+    _contig(input=input, sample_map=sample_map, interp_weights=interp_weights)
+    _on_gpu("input", input, sample_map=sample_map, interp_weights=interp_weights)
+    dt = _dtype(input, maps=(sample_map, interp_weights))
+    P, K = _pool_dims(input, sample_map, interp_weights, kernel_size)
+    B, C, IH, IW = input.shape
+    OH, OW = sample_map.shape[0], sample_map.shape[1]
+    out = torch.empty((B, C, OH, OW), dtype=input.dtype, device=input.device)
+    with torch.cuda.device(input.device):
+        rc = _lib.load().mcx_avg_pool(_ptr(input), _ptr(sample_map), _ptr(interp_weights),
+                                      _ptr(out), B, C, IH, IW, OH, OW, K, P, int(interpolation),
+                                      dt, _stream(input))
+    _lib.check(rc, "mapped_avg_pool")
+    return out
+
+
+def _avg_unpool(grad_output, sample_map, interp_weights, input_height, input_width, kernel_size,
+                interpolation):
+    _contig(grad_output=grad_output, sample_map=sample_map, interp_weights=interp_weights)
+    _on_gpu("grad_output", grad_output, sample_map=sample_map, interp_weights=interp_weights)
+    dt = _dtype(grad_output, maps=(sample_map, interp_weights))
+    P, K = _pool_dims(grad_output, sample_map, interp_weights, kernel_size)
+    B, C, OH, OW = grad_output.shape
+    if tuple(sample_map.shape[:2]) != (OH, OW):
+        raise RuntimeError("sample_map spatial size must match grad_output")
+    IH, IW = int(input_height), int(input_width)
+    gin = torch.empty((B, C, IH, IW), dtype=grad_output.dtype, device=grad_output.device)
+    with torch.cuda.device(grad_output.device):
+        rc = _lib.load().mcx_avg_unpool(_ptr(grad_output), _ptr(sample_map), _ptr(interp_weights),
+                                        _ptr(gin), B, C, IH, IW, OH, OW, K, P, int(interpolation),
+                                        dt, _stream(grad_output))
+    _lib.check(rc, "mapped_avg_unpool")
+    return gin
+
+
+def mapped_max_pool(input, sample_map, kernel_size, interpolation):
+    """include/nn/layers/mapped_max_pooling_layer.h:46-49 -> [pooled, idx_mask]."""
+    return _max_pool(input, sample_map, None, kernel_size, interpolation)
+
+
+def mapped_max_unpool(grad_output, idx_mask, sample_map, input_height, input_width, kernel_size,
+                      interpolation):
+    """include/nn/layers/mapped_max_pooling_layer.h:69-73."""
+    return _max_unpool(grad_output, idx_mask, sample_map, None, input_height, input_width,
+                       kernel_size, interpolation)
+
+
+def weighted_mapped_max_pool(input, sample_map, interp_weights, kernel_size, interpolation):
+    """include/nn/layers/weighted_mapped_max_pooling_layer.h:42-44."""
+    return _max_pool(input, sample_map, interp_weights, kernel_size, interpolation)
+
+
+def weighted_mapped_max_unpool(grad_output, idx_mask, sample_map, interp_weights, input_height,
+                               input_width, kernel_size, interpolation):
+    """include/nn/layers/weighted_mapped_max_pooling_layer.h:67-70."""
+    return _max_unpool(grad_output, idx_mask, sample_map, interp_weights, input_height,
+                       input_width, kernel_size, interpolation)
+
+
+def mapped_avg_pool(input, sample_map, kernel_size, interpolation):
+    """include/nn/layers/mapped_avg_pooling_layer.h:42-44."""
+    return _avg_pool(input, sample_map, None, kernel_size, interpolation)
+
+
+def mapped_avg_unpool(grad_output, sample_map, input_height, input_width, kernel_size,
+                      interpolation):
+    """include/nn/layers/mapped_avg_pooling_layer.h:64-67."""
+    return _avg_unpool(grad_output, sample_map, None, input_height, input_width, kernel_size,
+                       interpolation)
+
+
+def weighted_mapped_avg_pool(input, sample_map, interp_weights, kernel_size, interpolation):
+    """include/nn/layers/weighted_mapped_avg_pooling_layer.h:48-52."""
+    return _avg_pool(input, sample_map, interp_weights, kernel_size, interpolation)
+
+
+def weighted_mapped_avg_unpool(grad_output, sample_map, interp_weights, input_height, input_width,
+                               kernel_size, interpolation):
+    """include/nn/layers/weighted_mapped_avg_pooling_layer.h:75-78."""
+    return _avg_unpool(grad_output, sample_map, interp_weights, input_height, input_width,
+                       kernel_size, interpolation)
+
+
+# ----------------------------------------------------------------------- resample
+def _resample_to_map(input, sample_map, interp_weights, output_height, output_width,
+                     interpolation):
+    _contig(input=input, sample_map=sample_map, interp_weights=interp_weights)
+    _on_gpu("input", input, sample_map=sample_map, interp_weights=interp_weights)
+    dt = _dtype(input, maps=(sample_map, interp_weights))
+    P = _weighted_dims(sample_map, interp_weights, False)
+    B, C, IH, IW = input.shape
+    if tuple(sample_map.shape[:2]) != (IH, IW):
+        raise RuntimeError("sample_map spatial size must match the input")
+    OH, OW = int(output_height), int(output_width)
+    out = torch.empty((B, C, OH, OW), dtype=input.dtype, device=input.device)
+    with torch.cuda.device(input.device):
+        rc = _lib.load().mcx_resample_to_map(_ptr(input), _ptr(sample_map), _ptr(interp_weights),
+                                             _ptr(out), B, C, IH, IW, OH, OW, P,
+                                             int(interpolation), dt, _stream(input))
+    _lib.check(rc, "resample_to_map")
+    return out
+
+
+def _resample_from_map(input, sample_map, interp_weights, interpolation):
+    _contig(input=input, sample_map=sample_map, interp_weights=interp_weights)
+    _on_gpu("input", input, sample_map=sample_map, interp_weights=interp_weights)
+    dt = _dtype(input, maps=(sample_map, interp_weights))
+    P = _weighted_dims(sample_map, interp_weights, False)
+    B, C, SH, SW = input.shape
+    MH, MW = sample_map.shape[0], sample_map.shape[1]
+    out = torch.empty((B, C, MH, MW), dtype=input.dtype, device=input.device)
+    with torch.cuda.device(input.device):
+        rc = _lib.load().mcx_resample_from_map(_ptr(input), _ptr(sample_map),
+                                               _ptr(interp_weights), _ptr(out), B, C, SH, SW, MH,
+                                               MW, P, int(interpolation), dt, _stream(input))
+    _lib.check(rc, "resample_from_map")
+    return out
+
+
+def resample_to_map(input, sample_map, output_height, output_width, interpolation):
+    """include/nn/layers/resample_layer.h:38-40 (scatter)."""
+    return _resample_to_map(input, sample_map, None, output_height, output_width, interpolation)
+
+
+def resample_from_map(input, sample_map, interpolation):
+    """include/nn/layers/resample_layer.h:60-61 (gather)."""
+    return _resample_from_map(input, sample_map, None, interpolation)
+
+
+def weighted_resample_to_map(input, sample_map, interp_weights, output_height, output_width,
+                             interpolation):
+    """include/nn/layers/weighted_resample_layer.h:49-54."""
+    return _resample_to_map(input, sample_map, interp_weights, output_height, output_width,
+                            interpolation)
+
+
+def weighted_resample_from_map(input, sample_map, interp_weights, interpolation):
+    """include/nn/layers/weighted_resample_layer.h:78-81."""
+    return _resample_from_map(input, sample_map, interp_weights, interpolation)
+
+
+# ---------------------------------------------------------------------------- knn
+def knn_forward(ref, query, k):
+    """include/util/layers/knn_layer.h:25-35 -> [idx int64 [B,k,Q] (1-based), dist [B,k,Q]]."""
+    _contig(ref=ref, query=query)
+    _on_gpu("ref", ref, query=query)
+    dt = _dtype(ref, same=(query,))
+    if ref.dim() != 3 or query.dim() != 3 or ref.shape[:2] != query.shape[:2]:
+        raise RuntimeError("ref and query must be [B, D, *] with equal B and D")
+    B, D, R = ref.shape
+    Q, k = query.shape[2], int(k)
+    idx = torch.empty((B, k, Q), dtype=torch.int64, device=ref.device)
+    dist = torch.empty((B, k, Q), dtype=ref.dtype, device=ref.device)
+    with torch.cuda.device(ref.device):
+        rc = _lib.load().mcx_knn(_ptr(ref), _ptr(query), _ptr(idx), _ptr(dist), B, D, R, Q, k, dt,
+                                 _stream(ref))
+    _lib.check(rc, "knn_forward")
+    return [idx, dist]

@@ -1,0 +1,65 @@
+"""ctypes binding of libmcx_hip.so, the C ABI declared in include/mcx.h.
+
+The library is the only compute path: if it is missing this module raises at
+import of the first op, there is no CPU or eager fallback.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmcx_hip.so")
+
+MCX_F32, MCX_F64, MCX_BF16 = 0, 1, 2
+
+_p = ctypes.c_void_p
+_i64 = ctypes.c_int64
+_i = ctypes.c_int
+_sz = ctypes.c_size_t
+
+# name -> (restype, argtypes); mirrors include/mcx.h one to one.
+SIGNATURES = {
+    "mcx_abi_version": (_i, []),
+    "mcx_error_string": (ctypes.c_char_p, [_i]),
+    "mcx_resample_from_map": (_i, [_p] * 4 + [_i64] * 7 + [_i, _i, _p]),
+    "mcx_resample_to_map": (_i, [_p] * 4 + [_i64] * 7 + [_i, _i, _p]),
+    "mcx_max_pool": (_i, [_p] * 5 + [_i64] * 8 + [_i, _i, _p]),
+    "mcx_max_unpool": (_i, [_p] * 5 + [_i64] * 8 + [_i, _i, _p]),
+    "mcx_avg_pool": (_i, [_p] * 4 + [_i64] * 8 + [_i, _i, _p]),
+    "mcx_avg_unpool": (_i, [_p] * 4 + [_i64] * 8 + [_i, _i, _p]),
+    "mcx_conv_forward": (_i, [_p] * 6 + [_i64] * 9 + [_i, _i, _p]),
+    "mcx_conv_backward_workspace": (_sz, [_i64] * 9 + [_i]),
+    "mcx_conv_backward": (_i, [_p] * 9 + [_sz] + [_i64] * 9 + [_i, _i, _p]),
+    "mcx_tconv_forward": (_i, [_p] * 6 + [_i64] * 9 + [_i, _i, _p]),
+    "mcx_tconv_backward_workspace": (_sz, [_i64] * 9 + [_i]),
+    "mcx_tconv_backward": (_i, [_p] * 9 + [_sz] + [_i64] * 9 + [_i, _i, _p]),
+    "mcx_knn": (_i, [_p] * 4 + [_i64] * 5 + [_i, _p]),
+}
+
+_lib = None
+
+
+def load():
+    """Load the HIP library once; raise loudly when it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            "libmcx_hip.so not found at %s: build it with "
+            "`make -C mappedconvolutions_amd/csrc` (or __graft_entry__.build()); "
+            "there is no fallback path" % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is missing
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(code, what):
+    """Turn a non-zero return code into a RuntimeError (the reference raises
+    c10::Error -> RuntimeError from its checks, cuda_helper.h:12-20)."""
+    if code != 0:
+        msg = load().mcx_error_string(code).decode()
+        raise RuntimeError("%s failed: %s (code %d)" % (what, msg, code))

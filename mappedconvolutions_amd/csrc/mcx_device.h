@@ -1,0 +1,153 @@
+// Device-side building blocks shared by every kernel of the mapped-convolution
+// backend: the three interpolators (gather and scatter form), atomics and launch
+// helpers.  Semantics follow the reference's include/core/interpolation.h:85-238
+// and include/core/resample.h:34-162; the formulation (precomputed "taps" that
+// are reused across channels) is specific to this backend.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "mcx.h"
+
+namespace mcx {
+
+constexpr int kInterpNearest = 0;
+constexpr int kInterpBilinear = 1;
+constexpr int kInterpBispherical = 2;
+
+// Any interpolation code other than 1 or 2 means nearest (include/core/resample.h:69-71).
+__host__ __device__ inline int canonical_interp(int interp) {
+  return (interp == kInterpBilinear || interp == kInterpBispherical) ? interp : kInterpNearest;
+}
+
+#define MCX_HIP_CHECK_LAUNCH()                      \
+  do {                                              \
+    hipError_t e__ = hipGetLastError();             \
+    if (e__ != hipSuccess) return (int)e__;         \
+  } while (0)
+
+// ---- scalar helpers -------------------------------------------------------
+
+__device__ inline float mcx_floor(float v) { return floorf(v); }
+__device__ inline double mcx_floor(double v) { return floor(v); }
+__device__ inline float mcx_trunc(float v) { return truncf(v); }
+__device__ inline double mcx_trunc(double v) { return trunc(v); }
+__device__ inline float mcx_abs(float v) { return fabsf(v); }
+__device__ inline double mcx_abs(double v) { return fabs(v); }
+
+// llround(double(v)) of include/core/interpolation.h:90-91: halves go away from
+// zero.  v - trunc(v) is exact, so no double rounding can occur (adding 0.5 and
+// truncating would round 0.49999997f up).
+template <typename T>
+__device__ inline T round_half_away(T v) {
+  T t = mcx_trunc(v);
+  const T frac = v - t;
+  if (mcx_abs(frac) >= T(0.5)) t += (v < T(0)) ? T(-1) : T(1);
+  return t;
+}
+
+// Saturating conversion of an already integral floating value.
+__device__ inline int to_int(float v) { return (int)fminf(fmaxf(v, -2.0e9f), 2.0e9f); }
+__device__ inline int to_int(double v) { return (int)fmin(fmax(v, -2.0e9), 2.0e9); }
+
+__device__ inline int wrap_index(int v, int n) {
+  int r = v % n;
+  return r < 0 ? r + n : r;
+}
+
+__device__ inline void atomic_add(float *p, float v) {
+  __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ inline void atomic_add(double *p, double v) {
+  __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ---- taps -----------------------------------------------------------------
+// A tap is one (x, y) sample location resolved against an H x W plane: up to
+// four in-plane element offsets and their weights.  Offsets are -1 for corners
+// that fall outside the plane (they contribute exactly zero).  Because the map is
+// shared by every channel and image, a tap is computed once and applied to many
+// planes.
+template <typename T, int MODE>
+struct Tap;
+
+template <typename T>
+struct Tap<T, kInterpNearest> {
+  int off;
+  __device__ inline void set(T x, T y, int h, int w) {
+    const int xi = to_int(round_half_away(x));
+    const int yi = to_int(round_half_away(y));
+    const bool ok = xi >= 0 && xi <= w - 1 && yi >= 0 && yi <= h - 1;
+    off = ok ? yi * w + xi : -1;
+  }
+  template <typename TD>
+  __device__ inline T gather(const TD *plane) const {
+    return off >= 0 ? (T)plane[off] : T(0);
+  }
+  __device__ inline void scatter(T *plane, T v) const {
+    if (off >= 0) atomic_add(plane + off, v);
+  }
+};
+
+// Bilinear (zero padding on both axes) and bispherical (x wraps, y zero-padded).
+// Weight products are formed as (A*B), (A*C), (D*B), (D*C) and then multiplied by
+// the data, summed left to right: include/core/interpolation.h:22-32.
+template <typename T, int MODE>
+struct Tap {
+  int off[4];
+  T wt[4];
+  __device__ inline void set(T x, T y, int h, int w) {
+    const T x1f = mcx_floor(x), y1f = mcx_floor(y);
+    const T x2f = x1f + T(1), y2f = y1f + T(1);
+    int x1 = to_int(x1f), y1 = to_int(y1f);
+    int x2 = x1 + 1, y2 = y1 + 1;
+    bool x1ok, x2ok;
+    if (MODE == kInterpBispherical) {
+      x1 = wrap_index(x1, w);
+      x2 = wrap_index(x2, w);
+      x1ok = x2ok = true;
+    } else {
+      x1ok = x1 >= 0 && x1 <= w - 1;
+      x2ok = x2 >= 0 && x2 <= w - 1;
+    }
+    const bool y1ok = y1 >= 0 && y1 <= h - 1;
+    const bool y2ok = y2 >= 0 && y2 <= h - 1;
+    const T A = y2f - y, B = x2f - x, C = x - x1f, D = y - y1f;
+    off[0] = (x1ok && y1ok) ? y1 * w + x1 : -1;
+    off[1] = (x2ok && y1ok) ? y1 * w + x2 : -1;
+    off[2] = (x1ok && y2ok) ? y2 * w + x1 : -1;
+    off[3] = (x2ok && y2ok) ? y2 * w + x2 : -1;
+    wt[0] = A * B;
+    wt[1] = A * C;
+    wt[2] = D * B;
+    wt[3] = D * C;
+  }
+  template <typename TD>
+  __device__ inline T gather(const TD *plane) const {
+    const T d0 = off[0] >= 0 ? (T)plane[off[0]] : T(0);
+    const T d1 = off[1] >= 0 ? (T)plane[off[1]] : T(0);
+    const T d2 = off[2] >= 0 ? (T)plane[off[2]] : T(0);
+    const T d3 = off[3] >= 0 ? (T)plane[off[3]] : T(0);
+    return wt[0] * d0 + wt[1] * d1 + wt[2] * d2 + wt[3] * d3;
+  }
+  __device__ inline void scatter(T *plane, T v) const {
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      if (off[i] >= 0) atomic_add(plane + off[i], wt[i] * v);
+  }
+};
+
+// ---- launch helpers ---------------------------------------------------------
+
+inline unsigned div_up(int64_t a, int64_t b) { return (unsigned)((a + b - 1) / b); }
+
+// Dispatch a functor templated on the interpolation mode.
+#define MCX_DISPATCH_MODE(interp, ...)                                   \
+  switch (mcx::canonical_interp(interp)) {                               \
+    case mcx::kInterpBilinear: { constexpr int MODE = mcx::kInterpBilinear; __VA_ARGS__; } break; \
+    case mcx::kInterpBispherical: { constexpr int MODE = mcx::kInterpBispherical; __VA_ARGS__; } break; \
+    default: { constexpr int MODE = mcx::kInterpNearest; __VA_ARGS__; } break; \
+  }
+
+}  // namespace mcx

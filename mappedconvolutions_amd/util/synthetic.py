@@ -1,0 +1,90 @@
+"""Synthetic sample maps and point sets used by the tests and the benchmark.
+
+Everything is generated on the CPU with numpy in float64 from a fixed rule or a
+seeded generator and returned as torch tensors, so CPU checkers and GPU kernels
+see identical bits.
+"""
+import math
+
+import numpy as np
+import torch
+
+
+def latitude_map(height, width, radius=1, dtype=torch.float32):
+    """Latitude-distorted square kernel on an equirectangular grid.
+
+    For output pixel (i, j): lat = ((i + 0.5) / H) * pi - pi/2; taps are ordered
+    dy-major over offsets {-r..r}^2; x = (j + dx / max(cos lat, 0.05)) mod W,
+    y = clamp(i + dy, 0, H - 1).  Returns [H, W, (2r+1)^2, 2] with (x, y) last.
+    """
+    i = np.arange(height, dtype=np.float64)[:, None, None]
+    j = np.arange(width, dtype=np.float64)[None, :, None]
+    offs = np.arange(-radius, radius + 1, dtype=np.float64)
+    dy, dx = np.meshgrid(offs, offs, indexing='ij')
+    dy, dx = dy.reshape(1, 1, -1), dx.reshape(1, 1, -1)
+    lat = ((i + 0.5) / height) * math.pi - math.pi / 2
+    stretch = 1.0 / np.maximum(np.cos(lat), 0.05)
+    x = np.mod(j + dx * stretch, width)
+    y = np.clip(i + dy, 0, height - 1) + 0 * j
+    out = np.stack([np.broadcast_to(x, y.shape), y], axis=-1)
+    return torch.from_numpy(np.ascontiguousarray(out)).to(dtype)
+
+
+def identity_grid_map(height, width, radius=1, dtype=torch.float32):
+    """Regular grid taps x = j + dx, y = i + dy (dy-major): with this map a mapped
+    convolution equals a zero-padded (2r+1)x(2r+1) convolution."""
+    i = np.arange(height, dtype=np.float64)[:, None, None]
+    j = np.arange(width, dtype=np.float64)[None, :, None]
+    offs = np.arange(-radius, radius + 1, dtype=np.float64)
+    dy, dx = np.meshgrid(offs, offs, indexing='ij')
+    x = j + dx.reshape(1, 1, -1) + 0 * i
+    y = i + dy.reshape(1, 1, -1) + 0 * j
+    return torch.from_numpy(np.ascontiguousarray(np.stack([x, y], axis=-1))).to(dtype)
+
+
+def cube_to_equirect_map(face_dim, height, width, dtype=torch.float32):
+    """Equirectangular (x, y) of every pixel centre of a horizontally tiled
+    cube map [face_dim, 6 * face_dim], faces ordered -z, -x, +z, +x, +y, -y.
+
+    Exact gnomonic projection: pixel (u, v) of a face -> point on the cube
+    (face/axis convention of the reference's layers/util/conversions.py:123-180)
+    -> lon = atan2(x, z), lat = atan2(-y, sqrt(x^2 + z^2)) (:19-29) ->
+    x = (W/2)(lon/pi + 1), y = ((H-1)/2)(1 - 2 lat/pi) (:6-16).
+    Returns [face_dim, 6 * face_dim, 2].
+    """
+    v, u = np.meshgrid(np.arange(face_dim, dtype=np.float64),
+                       np.arange(face_dim, dtype=np.float64), indexing='ij')
+    u = 2 * (u + 0.5) / face_dim - 1
+    v = 2 * (v + 0.5) / face_dim - 1
+    one = np.ones_like(u)
+    faces = [(-u, -v, -one), (-one, -v, u), (u, -v, one), (one, -v, -u), (u, one, v),
+             (u, -one, -v)]
+    cols = []
+    for (x, y, z) in faces:
+        lon = np.arctan2(x, z)
+        lat = np.arctan2(-y, np.sqrt(x * x + z * z))
+        px = (width / 2) * (lon / math.pi + 1)
+        py = ((height - 1) / 2) * (1 - 2 * lat / math.pi)
+        cols.append(np.stack([px, py], axis=-1))
+    out = np.concatenate(cols, axis=1)
+    return torch.from_numpy(np.ascontiguousarray(out)).to(dtype)
+
+
+def mesh_weighted_map(num_vertices, kernel_size, num_points, seed=0, dtype=torch.float32):
+    """Weighted map of a mesh signal stored as a [1, V] image: every tap blends
+    `num_points` vertices.  x = integer vertex index ~ U{0..V-1} (stored as a
+    float), y = 0; weights ~ Dirichlet(1,..,1).  Returns
+    (sample_map [1, V, K, P, 2], interp_weights [1, V, K, P])."""
+    rng = np.random.default_rng(seed)
+    idx = rng.integers(0, num_vertices, size=(1, num_vertices, kernel_size, num_points))
+    smap = np.stack([idx.astype(np.float64), np.zeros(idx.shape)], axis=-1)
+    w = rng.dirichlet(np.ones(num_points), size=(1, num_vertices, kernel_size))
+    return (torch.from_numpy(smap).to(dtype), torch.from_numpy(w).to(dtype))
+
+
+def sphere_points(n, seed=0, dtype=torch.float32):
+    """n points uniform on the unit sphere (normalised N(0, I3)), shape [1, 3, n]."""
+    rng = np.random.default_rng(seed)
+    p = rng.standard_normal((3, n))
+    p /= np.linalg.norm(p, axis=0, keepdims=True)
+    return torch.from_numpy(p[None]).to(dtype).contiguous()

@@ -1,0 +1,326 @@
+"""GPU parity tests (run on the MI355X box): every op of the HIP boundary against
+the CPU oracle on the same seeded inputs, the reference's known answers and
+gradcheck through the layers (float64, as the reference's *_cuda tests do), and
+size-independent properties at larger shapes.
+
+Bars: gathers (resample_from_map, pools) are bit-exact against the oracle in
+every interpolation mode for fp32/fp64, max-pool argmax and KNN indices are
+bit-exact; scatters and convolutions (atomic / blocked accumulation order) agree
+within 1e-5 of the result's magnitude in fp32 and 1e-12 in fp64."""
+import pytest
+import torch
+import torch.nn.functional as F
+from torch.autograd import gradcheck
+
+import helpers
+from helpers import CASES, KNOWN, INTERP, rel_err
+from oracle import ops as O
+
+from mappedconvolutions_amd import _C, nn
+from mappedconvolutions_amd.util import knn, synthetic
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.float64]
+TOL = {torch.float32: 1e-5, torch.float64: 1e-12}
+
+
+def dev(*ts):
+    return [None if t is None else t.cuda() for t in ts]
+
+
+# ------------------------------------------------- reference known answers + gradcheck
+def _layer_for(case):
+    k, ci, co = KNOWN["kernel_size"], KNOWN["in_channels"], KNOWN["out_channels"]
+    op, interp = case["op"], case["interpolation"]
+    if op == "conv":
+        return nn.MappedConvolution(ci, co, k, interpolation=interp)
+    if op == "tconv":
+        return nn.MappedTransposedConvolution(ci, co, k, interpolation=interp)
+    if op == "max_pool":
+        return nn.MappedMaxPool(k, interpolation=interp)
+    if op == "avg_pool":
+        return nn.MappedAvgPool(k, interpolation=interp)
+    return nn.Unresample(interp)
+
+
+@pytest.mark.parametrize("name", sorted(CASES))
+def test_known_answers_and_gradcheck_through_layers(name, device):
+    case = CASES[name]
+    x, smap, iw, exp = helpers.case_tensors(case)
+    x, smap, iw = dev(x, smap, iw)
+    x.requires_grad_(True)
+    layer = _layer_for(case).double().to(device)
+    if case["op"] in ("conv", "tconv"):
+        w, b = helpers.case_weights(case)
+        layer.weight.data, layer.bias.data = w.cuda(), b.cuda()
+    if case["op"] == "tconv":
+        oh, ow = case["output_shape"]
+        args = (x, oh, ow, smap, iw)
+    else:
+        args = (x, smap, iw)
+    out = layer(*args)
+    torch.testing.assert_close(out.cpu(), exp.expand_as(out), rtol=1e-9, atol=1e-9)
+    out.backward(torch.ones_like(out))
+    assert gradcheck(layer, args)
+
+
+# ------------------------------------------------------------------ op-level parity
+def _conv_problem(dtype, seed, p, B=2, Ci=5, Co=7, IH=9, IW=11, OH=6, OW=10, K=5):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(B, Ci, IH, IW, generator=g, dtype=torch.float64).to(dtype)
+    smap, wts = helpers.random_map(g, OH, OW, K, p, IH, IW, dtype)
+    w = torch.randn(Co, Ci, K, generator=g, dtype=torch.float64).to(dtype)
+    b = torch.randn(Co, generator=g, dtype=torch.float64).to(dtype)
+    gy = torch.randn(B, Co, OH, OW, generator=g, dtype=torch.float64).to(dtype)
+    return x, smap, wts, w, b, gy, K
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("interp", [0, 1, 2])
+@pytest.mark.parametrize("p", [0, 3])
+def test_conv_forward_backward(dtype, interp, p, device):
+    x, smap, wts, w, b, gy, K = _conv_problem(dtype, 100 + interp + 10 * p, p)
+    y_o = O.weighted_mapped_conv_forward(x, smap, wts, w, b, K, interp)
+    g_o = O.weighted_mapped_conv_backward(gy, smap, wts, x, w, b, K, interp)
+    xd, sd, wd_, wgt, bd, gyd = dev(x, smap, wts, w, b, gy)
+    if p:
+        y = _C.weighted_mapped_conv_forward(xd, sd, wd_, wgt, bd, K, interp)
+        g = _C.weighted_mapped_conv_backward(gyd, sd, wd_, xd, wgt, bd, K, interp)
+    else:
+        y = _C.mapped_conv_forward(xd, sd, wgt, bd, K, interp)
+        g = _C.mapped_conv_backward(gyd, sd, xd, wgt, bd, K, interp)
+    assert rel_err(y, y_o) < TOL[dtype]
+    for a, r, nm in zip(g, g_o, ("grad_input", "grad_weight", "grad_bias")):
+        assert rel_err(a, r) < TOL[dtype], nm
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("interp", [0, 1, 2])
+@pytest.mark.parametrize("p", [0, 3])
+def test_transposed_conv_forward_backward(dtype, interp, p, device):
+    g = torch.Generator().manual_seed(200 + interp + 10 * p)
+    B, Ci, Co, IH, IW, OH, OW, K = 2, 5, 6, 6, 7, 9, 12, 4
+    x = torch.randn(B, Ci, IH, IW, generator=g, dtype=torch.float64).to(dtype)
+    smap, wts = helpers.random_map(g, IH, IW, K, p, OH, OW, dtype)
+    w = torch.randn(Ci, Co, K, generator=g, dtype=torch.float64).to(dtype)
+    b = torch.randn(Co, generator=g, dtype=torch.float64).to(dtype)
+    gy = torch.randn(B, Co, OH, OW, generator=g, dtype=torch.float64).to(dtype)
+    y_o = O.weighted_mapped_transposed_conv_forward(x, smap, wts, w, b, OH, OW, K, interp)
+    g_o = O.weighted_mapped_transposed_conv_backward(gy, smap, wts, x, w, b, K, interp)
+    xd, sd, wd_, wgt, bd, gyd = dev(x, smap, wts, w, b, gy)
+    if p:
+        y = _C.weighted_mapped_transposed_conv_forward(xd, sd, wd_, wgt, bd, OH, OW, K, interp)
+        gr = _C.weighted_mapped_transposed_conv_backward(gyd, sd, wd_, xd, wgt, bd, K, interp)
+    else:
+        y = _C.mapped_transposed_conv_forward(xd, sd, wgt, bd, OH, OW, K, interp)
+        gr = _C.mapped_transposed_conv_backward(gyd, sd, xd, wgt, bd, K, interp)
+    assert rel_err(y, y_o) < TOL[dtype]
+    for a, r, nm in zip(gr, g_o, ("grad_input", "grad_weight", "grad_bias")):
+        assert rel_err(a, r) < TOL[dtype], nm
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("interp", [0, 1, 2])
+@pytest.mark.parametrize("p", [0, 3])
+@pytest.mark.parametrize("half", [False, True])
+def test_pools(dtype, interp, p, half, device):
+    g = torch.Generator().manual_seed(300 + interp + 10 * p)
+    B, C, IH, IW, OH, OW, K = 2, 11, 9, 13, 7, 9, 5   # C=11: a ragged channel chunk
+    x = torch.randn(B, C, IH, IW, generator=g, dtype=torch.float64).to(dtype)
+    smap, wts = helpers.random_map(g, OH, OW, K, p, IH, IW, dtype, half=half)
+    gy = torch.randn(B, C, OH, OW, generator=g, dtype=torch.float64).to(dtype)
+    xd, sd, wd_, gyd = dev(x, smap, wts, gy)
+    mo, mi = O.weighted_mapped_max_pool(x, smap, wts, K, interp)
+    ao = O.weighted_mapped_avg_pool(x, smap, wts, K, interp)
+    if p:
+        m, i = _C.weighted_mapped_max_pool(xd, sd, wd_, K, interp)
+        a = _C.weighted_mapped_avg_pool(xd, sd, wd_, K, interp)
+        mu = _C.weighted_mapped_max_unpool(gyd, i, sd, wd_, IH, IW, K, interp)
+        au = _C.weighted_mapped_avg_unpool(gyd, sd, wd_, IH, IW, K, interp)
+    else:
+        m, i = _C.mapped_max_pool(xd, sd, K, interp)
+        a = _C.mapped_avg_pool(xd, sd, K, interp)
+        mu = _C.mapped_max_unpool(gyd, i, sd, IH, IW, K, interp)
+        au = _C.mapped_avg_unpool(gyd, sd, IH, IW, K, interp)
+    assert torch.equal(m.cpu(), mo), "max-pool values must be bit-exact"
+    assert torch.equal(i.cpu(), mi), "max-pool argmax must be bit-exact"
+    assert torch.equal(a.cpu(), ao), "avg-pool gather must be bit-exact"
+    muo = O.weighted_mapped_max_unpool(gy, mi, smap, wts, IH, IW, K, interp)
+    auo = O.weighted_mapped_avg_unpool(gy, smap, wts, IH, IW, K, interp)
+    assert rel_err(mu, muo) < TOL[dtype]
+    assert rel_err(au, auo) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("interp", [0, 1, 2])
+@pytest.mark.parametrize("p", [0, 4])
+@pytest.mark.parametrize("half", [False, True])
+def test_resample(dtype, interp, p, half, device):
+    g = torch.Generator().manual_seed(400 + interp + 10 * p)
+    B, C, IH, IW, OH, OW = 2, 9, 10, 12, 8, 15
+    x = torch.randn(B, C, IH, IW, generator=g, dtype=torch.float64).to(dtype)
+    smap, wts = helpers.random_map(g, IH, IW, 1, p, OH, OW, dtype, half=half)
+    smap = smap[:, :, 0].contiguous()
+    wts = None if wts is None else wts[:, :, 0].contiguous()
+    y = torch.randn(B, C, OH, OW, generator=g, dtype=torch.float64).to(dtype)
+    xd, sd, wd_, yd = dev(x, smap, wts, y)
+    to_o = O.weighted_resample_to_map(x, smap, wts, OH, OW, interp)
+    fr_o = O.weighted_resample_from_map(y, smap, wts, interp)
+    if p:
+        to = _C.weighted_resample_to_map(xd, sd, wd_, OH, OW, interp)
+        fr = _C.weighted_resample_from_map(yd, sd, wd_, interp)
+    else:
+        to = _C.resample_to_map(xd, sd, OH, OW, interp)
+        fr = _C.resample_from_map(yd, sd, interp)
+    assert torch.equal(fr.cpu(), fr_o), "gather must be bit-exact"
+    assert rel_err(to, to_o) < TOL[dtype]
+
+
+def test_empty_and_degenerate_inputs(device):
+    """Taps that all fall outside give zeros / -FLT_MAX with index -1; 1x1 images work."""
+    x = torch.rand(1, 2, 3, 3, device=device) + 1
+    far = torch.full((2, 2, 3, 2), 100.0, device=device)
+    assert _C.mapped_avg_pool(x, far, 3, 1).abs().sum() == 0
+    m, i = _C.mapped_max_pool(x, far, 3, 1)
+    # the zero of the padding beats -FLT_MAX at tap 0 of every pixel: offset n * K * 2
+    assert (m == 0).all() and i[0, 0].flatten().tolist() == [0, 6, 12, 18]
+    g = torch.ones(1, 2, 2, 2, device=device)
+    assert _C.mapped_max_unpool(g, i, far, 3, 3, 3, 1).abs().sum() == 0
+    neg = torch.full((1, 2, 2, 2), -1, device=device, dtype=torch.int64)
+    assert _C.mapped_max_unpool(g, neg, far, 3, 3, 3, 1).abs().sum() == 0
+    one = torch.rand(1, 1, 1, 1, device=device)
+    sm = torch.zeros(1, 1, 2, device=device)
+    assert torch.equal(_C.resample_from_map(one, sm, 0), one)
+
+
+# ------------------------------------------------------------- BASELINE config 1
+def test_config1_forward_fp32(device):
+    """B=1, 16->32, 64x128, 3x3 latitude map, bilinear, Kaiming weights, bias 0."""
+    torch.manual_seed(0)
+    x = torch.rand(1, 16, 64, 128) * 2 - 1
+    w = torch.randn(32, 16, 9) * (2.0 / (16 * 9)) ** 0.5
+    b = torch.zeros(32)
+    smap = synthetic.latitude_map(64, 128, 1)
+    ref = O.mapped_conv_forward(x, smap, w, b, 9, 1)
+    out = _C.mapped_conv_forward(*dev(x, smap, w, b), 9, 1)
+    assert rel_err(out, ref) < 1e-5
+
+
+@pytest.mark.parametrize("interp", [0, 1])
+def test_conv_medium_fp32_vs_oracle(interp, device):
+    """A config-2-shaped problem scaled to what the CPU oracle finishes in seconds
+    (B=2, 64->64, 32x64, 3x3 latitude map), forward and backward."""
+    torch.manual_seed(1)
+    B, C, H, W = 2, 64, 32, 64
+    x, gy = torch.randn(B, C, H, W), torch.randn(B, C, H, W)
+    w, b = torch.randn(C, C, 9) / 24, torch.randn(C)
+    smap = synthetic.latitude_map(H, W, 1)
+    y_o = O.mapped_conv_forward(x, smap, w, b, 9, interp)
+    g_o = O.mapped_conv_backward(gy, smap, x, w, b, 9, interp)
+    xd, sd, wd_, bd, gyd = dev(x, smap, w, b, gy)
+    y = _C.mapped_conv_forward(xd, sd, wd_, bd, 9, interp)
+    g = _C.mapped_conv_backward(gyd, sd, xd, wd_, bd, 9, interp)
+    assert rel_err(y, y_o) < 1e-5
+    for a, r, nm in zip(g, g_o, ("grad_input", "grad_weight", "grad_bias")):
+        assert rel_err(a, r) < 1e-5, nm
+
+
+# ----------------------------------------------------- size-independent properties
+@pytest.mark.parametrize("interp", [0, 1])
+def test_identity_map_equals_conv2d_large(interp, device):
+    """With the regular-grid map a mapped convolution is a zero-padded 3x3
+    convolution; checked against the library routine at B=2, 64->64, 128x256."""
+    torch.manual_seed(2)
+    B, C, H, W = 2, 64, 128, 256
+    x = torch.randn(B, C, H, W, device=device)
+    w = torch.randn(C, C, 9, device=device) / 24
+    b = torch.randn(C, device=device)
+    smap = synthetic.identity_grid_map(H, W, 1).to(device)
+    gy = torch.randn(B, C, H, W, device=device)
+    xr, wr = x.double().requires_grad_(True), w.double().requires_grad_(True)
+    ref = F.conv2d(xr, wr.view(C, C, 3, 3), b.double(), padding=1)
+    gx_r, gw_r = torch.autograd.grad(ref, (xr, wr), gy.double())
+    y = _C.mapped_conv_forward(x, smap, w, b, 9, interp)
+    gx, gw, gb = _C.mapped_conv_backward(gy, smap, x, w, b, 9, interp)
+    assert rel_err(y, ref.detach()) < 1e-5
+    assert rel_err(gx, gx_r) < 1e-5
+    assert rel_err(gw, gw_r) < 1e-5
+    assert rel_err(gb, gy.double().sum((0, 2, 3))) < 1e-5
+
+
+@pytest.mark.parametrize("interp", [0, 1, 2])
+def test_adjointness_large(interp, device):
+    """<conv(x), g> == <x, conv_backward_input(g)> and <from_map(s), g> == <s, to_map(g)>."""
+    torch.manual_seed(3)
+    B, C, H, W = 2, 32, 64, 128
+    x = torch.randn(B, C, H, W, device=device)
+    w = torch.randn(C, C, 9, device=device) / 17
+    zero = torch.zeros(C, device=device)
+    smap = synthetic.latitude_map(H, W, 1).to(device)
+    g = torch.randn(B, C, H, W, device=device)
+    y = _C.mapped_conv_forward(x, smap, w, zero, 9, interp)
+    gx = _C.mapped_conv_backward(g, smap, x, w, zero, 9, interp)[0]
+    lhs, rhs = (y.double() * g.double()).sum(), (x.double() * gx.double()).sum()
+    assert abs(lhs - rhs) / abs(lhs) < 1e-5
+    sm1 = smap[:, :, 3].contiguous()
+    lhs = (_C.resample_from_map(x, sm1, interp).double() * g.double()).sum()
+    rhs = (x.double() * _C.resample_to_map(g, sm1, H, W, interp).double()).sum()
+    assert abs(lhs - rhs) / abs(lhs) < 1e-5
+
+
+def test_linearity_of_forward(device):
+    torch.manual_seed(4)
+    B, C, H, W = 1, 16, 32, 64
+    x1, x2 = torch.randn(B, C, H, W, device=device), torch.randn(B, C, H, W, device=device)
+    w = torch.randn(8, C, 9, device=device)
+    zero = torch.zeros(8, device=device)
+    smap = synthetic.latitude_map(H, W, 1).to(device)
+    y = _C.mapped_conv_forward(x1 + 2 * x2, smap, w, zero, 9, 1)
+    y12 = _C.mapped_conv_forward(x1, smap, w, zero, 9, 1) + 2 * _C.mapped_conv_forward(
+        x2, smap, w, zero, 9, 1)
+    assert rel_err(y, y12) < 1e-5
+
+
+# ---------------------------------------------------------------------------- knn
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("k", [1, 8, 20])
+def test_knn_vs_oracle(dtype, k, device):
+    g = torch.Generator().manual_seed(500 + k)
+    B, D, R, Q = 2, 3, 1000, 700
+    ref = torch.randn(B, D, R, generator=g, dtype=torch.float64).to(dtype)
+    qry = torch.randn(B, D, Q, generator=g, dtype=torch.float64).to(dtype)
+    ref[:, :, 50] = ref[:, :, 10]
+    qry[:, :, 0] = ref[:, :, 10]
+    io, do = O.knn_forward(ref, qry, k)
+    i, d = knn(ref.cuda(), qry.cuda(), k)
+    assert torch.equal(i.cpu(), io), "KNN indices must be bit-exact"
+    assert torch.equal(d.cpu(), do)
+
+
+def test_knn_other_dimensions(device):
+    for D in (1, 2, 4, 6):
+        g = torch.Generator().manual_seed(D)
+        ref = torch.randn(1, D, 300, generator=g)
+        qry = torch.randn(1, D, 260, generator=g)
+        io, do = O.knn_forward(ref, qry, 5)
+        i, d = knn(ref.cuda(), qry.cuda(), 5)
+        assert torch.equal(i.cpu(), io) and torch.equal(d.cpu(), do)
+
+
+def test_knn_sphere_invariants(device):
+    """Unit-sphere points, 65536 queries x 40962 references, k=8: ascending
+    distances, distances match the indexed points, and no excluded point is closer
+    than the k-th on sampled queries."""
+    ref = synthetic.sphere_points(40962, seed=1).to(device)
+    qry = synthetic.sphere_points(65536, seed=2).to(device)
+    idx, dist = knn(ref, qry, 8)
+    assert idx.min() >= 1 and idx.max() <= 40962
+    assert (dist[:, 1:] >= dist[:, :-1]).all()
+    picked = ref[0][:, (idx[0] - 1).reshape(-1)].view(3, 8, -1)
+    d2 = ((picked - qry[0][:, None, :]) ** 2).sum(0).sqrt()
+    torch.testing.assert_close(d2, dist[0], rtol=1e-4, atol=1e-6)
+    sample = torch.arange(0, 65536, 997, device=device)
+    full = torch.cdist(qry[0][:, sample].t().double(), ref[0].t().double())
+    kth = full.sort(-1).values[:, 7]
+    torch.testing.assert_close(dist[0, 7, sample].double(), kth, rtol=1e-5, atol=1e-6)
