@@ -21,8 +21,8 @@ constexpr int kThreads = 256;
 
 __device__ inline float fma_t(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 __device__ inline double fma_t(double a, double b, double c) { return __builtin_fma(a, b, c); }
-__device__ inline float sqrt_t(float v) { return __fsqrt_rn(v); }
-__device__ inline double sqrt_t(double v) { return __dsqrt_rn(v); }
+__device__ inline float sqrt_t(float v) { return sqrtf(v); }
+__device__ inline double sqrt_t(double v) { return sqrt(v); }
 
 template <typename T>
 __device__ inline T inf_t() { return (T)__builtin_huge_valf(); }
