@@ -1,0 +1,130 @@
+"""Benchmark of the mapped-convolution hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--interp bilinear|nearest]
+
+A step is one forward + backward (grad_input, grad_weight, grad_bias) of a
+MappedConvolution at the headline configuration: B=8, 64->64 channels, 256x512
+equirectangular input, 3x3 latitude-distorted sample map, fp32, synthetic data
+resident in HBM.  Prints ONE JSON line: Mpix/s (B*OH*OW per step / time), the
+roofline position of the dominant kernel (timed with events on the launch stream
+inside the timed region) and the reference CPU implementation timed on this
+host's cores on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from mappedconvolutions_amd import _C  # noqa: E402
+from mappedconvolutions_amd.util import synthetic  # noqa: E402
+
+B, CI, CO, H, W, K = 8, 64, 64, 256, 512, 9
+PEAK_FP32_MFMA_TFLOPS = 157.3
+GEMM_FLOP = 2.0 * B * H * W * CO * CI * K  # one of the three products
+
+
+def make_inputs(device, batch=B):
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(batch, CI, H, W, generator=g)
+    gy = torch.randn(batch, CO, H, W, generator=g)
+    w = torch.randn(CO, CI, K, generator=g) * (2.0 / (CI * K)) ** 0.5
+    b = torch.zeros(CO)
+    smap = synthetic.latitude_map(H, W, 1)
+    return [t.to(device) for t in (x, gy, w, b, smap)]
+
+
+def step(x, gy, w, b, smap, interp):
+    y = _C.mapped_conv_forward(x, smap, w, b, K, interp)
+    grads = _C.mapped_conv_backward(gy, smap, x, w, b, K, interp)
+    return y, grads
+
+
+def cpu_baseline(interp):
+    """Reference CPU implementation (oracle/_ref, built from the reference's own
+    sources) on a B=1 slice of the workload; falls back to the C port."""
+    from oracle import reference
+    x, gy, w, b, smap = make_inputs("cpu", batch=1)
+    if reference.available():
+        mod, kind = reference.module("_mapped_convolution"), "reference"
+    else:
+        from oracle import ops as mod
+        kind = "port"
+    times = []
+    for rep in range(4):
+        t0 = time.perf_counter()
+        mod.mapped_conv_forward(x, smap, w, b, K, interp)
+        mod.mapped_conv_backward(gy, smap, x, w, b, K, interp)
+        times.append(time.perf_counter() - t0)
+    t = statistics.median(times[1:])
+    return {"value": round(H * W / t / 1e6, 4), "unit": "Mpix/s", "cores": torch.get_num_threads(),
+            "kind": kind,
+            "sample": "B=1 slice (1 of 8 images; the reference loops over the batch, so cost is "
+                      "linear in B), forward+backward, 1 warm-up + median of 3, %.2f s each" % t}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--interp", default="bilinear", choices=["bilinear", "nearest"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    interp = 1 if args.interp == "bilinear" else 0
+    dev = torch.device("cuda:0")
+    inputs = make_inputs(dev)
+
+    for _ in range(args.warmup):
+        step(*inputs, interp)
+    torch.cuda.synchronize()
+    _C.profile_events = []
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(*inputs, interp)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    events, _C.profile_events = _C.profile_events, None
+
+    per_label = {}
+    for label, start, end in events:
+        per_label.setdefault(label, []).append(start.elapsed_time(end))
+    kernel_ms = {k: sum(v) / len(v) for k, v in per_label.items()}
+    gemm_like = {k: v for k, v in kernel_ms.items() if k != "conv_backward_bias"}
+    dominant = max(gemm_like, key=gemm_like.get)
+    achieved = GEMM_FLOP / (gemm_like[dominant] * 1e-3) / 1e12
+
+    ms = elapsed / args.steps * 1e3
+    out = {
+        "metric": "Mapped-conv fwd+bwd Mpix/s (B8,C64,256x512,3x3); % HBM/MFMA roofline",
+        "value": round(B * H * W / (ms * 1e-3) / 1e6, 3),
+        "unit": "Mpix/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "MappedConvolution fwd+bwd B8 Ci64 Co64 256x512 K9 latitude map, "
+                               + args.interp, "interpolation": args.interp},
+        "roofline": {"bound": "mfma", "kernel": dominant,
+                     "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+                     "traffic": None},
+        "kernel_ms": {k: round(v, 4) for k, v in kernel_ms.items()},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(interp)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

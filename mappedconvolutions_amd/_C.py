@@ -15,6 +15,25 @@ from ._lib import MCX_BF16, MCX_F32, MCX_F64
 _DTYPES = {torch.float32: MCX_F32, torch.float64: MCX_F64, torch.bfloat16: MCX_BF16}
 
 
+# Optional timing hook: when set to a list, every C-ABI call made by the convolution
+# ops appends (label, start_event, end_event), recorded on the stream the kernels
+# are enqueued on.  Used by the benchmark to time individual kernels.
+profile_events = None
+
+
+def _timed(label, device, fn):
+    if profile_events is None:
+        return fn()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    stream = torch.cuda.current_stream(device)
+    start.record(stream)
+    rc = fn()
+    end.record(stream)
+    profile_events.append((label, start, end))
+    return rc
+
+
 def _contig(**tensors):
     for name, t in tensors.items():
         if t is not None and not t.is_contiguous():
@@ -86,10 +105,11 @@ def _conv_forward(input, sample_map, interp_weights, weight, bias, kernel_size, 
     if bias.numel() != Co:
         raise RuntimeError("bias must have %d elements" % Co)
     out = torch.empty((B, Co, OH, OW), dtype=input.dtype, device=input.device)
+    lib = _lib.load()
     with torch.cuda.device(input.device):
-        rc = _lib.load().mcx_conv_forward(_ptr(input), _ptr(sample_map), _ptr(interp_weights),
-                                          _ptr(weight), _ptr(bias), _ptr(out), B, Ci, Co, IH, IW,
-                                          OH, OW, K, P, int(interpolation), dt, _stream(input))
+        rc = _timed("conv_forward", input.device, lambda: lib.mcx_conv_forward(
+            _ptr(input), _ptr(sample_map), _ptr(interp_weights), _ptr(weight), _ptr(bias),
+            _ptr(out), B, Ci, Co, IH, IW, OH, OW, K, P, int(interpolation), dt, _stream(input)))
     _lib.check(rc, "mapped_conv_forward")
     return out
 
@@ -114,12 +134,17 @@ def _conv_backward(grad_output, sample_map, interp_weights, input, weight, bias,
     lib = _lib.load()
     ws_bytes = lib.mcx_conv_backward_workspace(B, Ci, Co, IH, IW, OH, OW, K, P, dt)
     ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=input.device)
+    # One C-ABI call per gradient (NULL skips the others) so each can be timed alone.
+    outs = {"conv_backward_input": (grad_input, None, None),
+            "conv_backward_weight": (None, grad_weight, None),
+            "conv_backward_bias": (None, None, grad_bias)}
     with torch.cuda.device(input.device):
-        rc = lib.mcx_conv_backward(_ptr(grad_output), _ptr(sample_map), _ptr(interp_weights),
-                                   _ptr(input), _ptr(weight), _ptr(grad_input), _ptr(grad_weight),
-                                   _ptr(grad_bias), _ptr(ws), ws_bytes, B, Ci, Co, IH, IW, OH, OW,
-                                   K, P, int(interpolation), dt, _stream(input))
-    _lib.check(rc, "mapped_conv_backward")
+        for label, (gx, gw, gb) in outs.items():
+            rc = _timed(label, input.device, lambda: lib.mcx_conv_backward(
+                _ptr(grad_output), _ptr(sample_map), _ptr(interp_weights), _ptr(input),
+                _ptr(weight), _ptr(gx), _ptr(gw), _ptr(gb), _ptr(ws), ws_bytes, B, Ci, Co, IH, IW,
+                OH, OW, K, P, int(interpolation), dt, _stream(input)))
+            _lib.check(rc, "mapped_conv_backward")
     return [grad_input, grad_weight, grad_bias]
 
 
