@@ -111,11 +111,15 @@ int mcx_avg_unpool(const void *gout, const void *map, const void *iw, void *gin,
  * The gather, the product with w and the bias are one fused kernel; no column
  * buffer exists. */
 int mcx_conv_forward(const void *x, const void *map, const void *iw, const void *w,
-                     const void *bias, void *y, int64_t B, int64_t Ci, int64_t Co, int64_t IH,
-                     int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
-                     int dtype, void *stream);
+                     const void *bias, void *y, void *workspace, size_t workspace_bytes,
+                     int64_t B, int64_t Ci, int64_t Co, int64_t IH, int64_t IW, int64_t OH,
+                     int64_t OW, int64_t K, int64_t P, int interp, int dtype, void *stream);
 
-/* Bytes of scratch mcx_conv_backward needs for these sizes (may be 0). */
+/* Bytes of device scratch the matching call needs for these sizes (may be 0).
+ * The scratch holds repacked weights and partial sums; its contents need not
+ * survive the call.  It must be 256-byte aligned. */
+size_t mcx_conv_forward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t IH, int64_t IW,
+                                  int64_t OH, int64_t OW, int64_t K, int64_t P, int dtype);
 size_t mcx_conv_backward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t IH, int64_t IW,
                                    int64_t OH, int64_t OW, int64_t K, int64_t P, int dtype);
 
@@ -125,7 +129,7 @@ size_t mcx_conv_backward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t IH
  * gy [B,Co,OH,OW], x, w as above -> gx [B,Ci,IH,IW] (cleared here),
  * gw [Co,Ci,K], gb [Co] (= gy summed over b,h,w).  Any of gx, gw, gb may be
  * NULL to skip that gradient.  workspace: device scratch of at least
- * mcx_conv_backward_workspace(...) bytes, 256-byte aligned. */
+ * mcx_conv_backward_workspace(...) bytes. */
 int mcx_conv_backward(const void *gy, const void *map, const void *iw, const void *x,
                       const void *w, void *gx, void *gw, void *gb, void *workspace,
                       size_t workspace_bytes, int64_t B, int64_t Ci, int64_t Co, int64_t IH,
@@ -139,10 +143,12 @@ int mcx_conv_backward(const void *gy, const void *map, const void *iw, const voi
  * x [B,Ci,IH,IW], map [IH,IW,K,(P,)2] pointing into the OUTPUT, w [Ci,Co,K],
  * bias [Co] -> y [B,Co,OH,OW] (initialised to the bias here, then accumulated). */
 int mcx_tconv_forward(const void *x, const void *map, const void *iw, const void *w,
-                      const void *bias, void *y, int64_t B, int64_t Ci, int64_t Co, int64_t IH,
-                      int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
-                      int dtype, void *stream);
+                      const void *bias, void *y, void *workspace, size_t workspace_bytes,
+                      int64_t B, int64_t Ci, int64_t Co, int64_t IH, int64_t IW, int64_t OH,
+                      int64_t OW, int64_t K, int64_t P, int interp, int dtype, void *stream);
 
+size_t mcx_tconv_forward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t IH, int64_t IW,
+                                   int64_t OH, int64_t OW, int64_t K, int64_t P, int dtype);
 size_t mcx_tconv_backward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t IH, int64_t IW,
                                     int64_t OH, int64_t OW, int64_t K, int64_t P, int dtype);
 

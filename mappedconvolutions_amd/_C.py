@@ -74,6 +74,11 @@ def _stream(t):
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
+def _workspace(nbytes, device):
+    """Scratch for one call (torch's caching allocator returns 512-byte aligned blocks)."""
+    return torch.empty((max(int(nbytes), 1),), dtype=torch.uint8, device=device)
+
+
 def _weighted_dims(sample_map, interp_weights, kernel):
     """Number of interpolation points P (0 = unweighted) after a shape check."""
     want = (4 if kernel else 3) + (0 if interp_weights is None else 1)
@@ -106,10 +111,13 @@ def _conv_forward(input, sample_map, interp_weights, weight, bias, kernel_size, 
         raise RuntimeError("bias must have %d elements" % Co)
     out = torch.empty((B, Co, OH, OW), dtype=input.dtype, device=input.device)
     lib = _lib.load()
+    ws_bytes = lib.mcx_conv_forward_workspace(B, Ci, Co, IH, IW, OH, OW, K, P, dt)
+    ws = _workspace(ws_bytes, input.device)
     with torch.cuda.device(input.device):
         rc = _timed("conv_forward", input.device, lambda: lib.mcx_conv_forward(
             _ptr(input), _ptr(sample_map), _ptr(interp_weights), _ptr(weight), _ptr(bias),
-            _ptr(out), B, Ci, Co, IH, IW, OH, OW, K, P, int(interpolation), dt, _stream(input)))
+            _ptr(out), _ptr(ws), ws_bytes, B, Ci, Co, IH, IW, OH, OW, K, P, int(interpolation),
+            dt, _stream(input)))
     _lib.check(rc, "mapped_conv_forward")
     return out
 
@@ -133,7 +141,7 @@ def _conv_backward(grad_output, sample_map, interp_weights, input, weight, bias,
     grad_bias = torch.empty((Co,), dtype=input.dtype, device=input.device)
     lib = _lib.load()
     ws_bytes = lib.mcx_conv_backward_workspace(B, Ci, Co, IH, IW, OH, OW, K, P, dt)
-    ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=input.device)
+    ws = _workspace(ws_bytes, input.device)
     # One C-ABI call per gradient (NULL skips the others) so each can be timed alone.
     outs = {"conv_backward_input": (grad_input, None, None),
             "conv_backward_weight": (None, grad_weight, None),
@@ -188,10 +196,14 @@ def _tconv_forward(input, sample_map, interp_weights, weight, bias, output_heigh
     if tuple(weight.shape) != (Ci, Co, K) or tuple(sample_map.shape[:3]) != (IH, IW, K):
         raise RuntimeError("shape mismatch in mapped_transposed_conv_forward")
     out = torch.empty((B, Co, OH, OW), dtype=input.dtype, device=input.device)
+    lib = _lib.load()
+    ws_bytes = lib.mcx_tconv_forward_workspace(B, Ci, Co, IH, IW, OH, OW, K, P, dt)
+    ws = _workspace(ws_bytes, input.device)
     with torch.cuda.device(input.device):
-        rc = _lib.load().mcx_tconv_forward(_ptr(input), _ptr(sample_map), _ptr(interp_weights),
-                                           _ptr(weight), _ptr(bias), _ptr(out), B, Ci, Co, IH, IW,
-                                           OH, OW, K, P, int(interpolation), dt, _stream(input))
+        rc = lib.mcx_tconv_forward(_ptr(input), _ptr(sample_map), _ptr(interp_weights),
+                                   _ptr(weight), _ptr(bias), _ptr(out), _ptr(ws), ws_bytes, B, Ci,
+                                   Co, IH, IW, OH, OW, K, P, int(interpolation), dt,
+                                   _stream(input))
     _lib.check(rc, "mapped_transposed_conv_forward")
     return out
 
@@ -215,7 +227,7 @@ def _tconv_backward(grad_output, sample_map, interp_weights, input, weight, bias
     grad_bias = torch.empty((Co,), dtype=input.dtype, device=input.device)
     lib = _lib.load()
     ws_bytes = lib.mcx_tconv_backward_workspace(B, Ci, Co, IH, IW, OH, OW, K, P, dt)
-    ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=input.device)
+    ws = _workspace(ws_bytes, input.device)
     with torch.cuda.device(input.device):
         rc = lib.mcx_tconv_backward(_ptr(grad_output), _ptr(sample_map), _ptr(interp_weights),
                                     _ptr(input), _ptr(weight), _ptr(grad_input), _ptr(grad_weight),

@@ -28,4 +28,12 @@ int channel_sum(const T *g, T *gb, int64_t B, int64_t C, int64_t N, hipStream_t 
 template <typename T>
 int fill_bias(T *y, const T *bias, int64_t B, int64_t C, int64_t N, hipStream_t s);
 
+// ---- fp32 matrix-core kernels (mcx_conv_mfma_f32.hip) -------------------------
+size_t mfma_f32_packed_weight_bytes(int64_t O, int64_t G, int64_t K);
+bool mfma_f32_gather_product_supported(int64_t P);
+int mfma_f32_gather_product(const float *src, const float *map, const float *iw, const float *w,
+                            const float *bias, float *y, float *wp, int64_t B, int64_t G,
+                            int64_t O, int64_t SH, int64_t SW, int64_t OH, int64_t OW, int64_t K,
+                            int64_t P, int interp, hipStream_t s);
+
 }  // namespace mcx

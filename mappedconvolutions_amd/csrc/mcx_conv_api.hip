@@ -1,5 +1,7 @@
 // extern "C" entry points of the mapped (transposed) convolution.  Validates the
-// arguments, then routes each of the three products to a kernel family.
+// arguments, then routes each of the three products (gather-product,
+// product-scatter, weight gradient; see mcx_conv_generic.hip for the roles) to the
+// matrix-core kernels when they cover the case and to the scalar kernels otherwise.
 #include <initializer_list>
 
 #include "mcx.h"
@@ -13,25 +15,25 @@ struct ConvDims {
   int64_t B, Ci, Co, IH, IW, OH, OW, K, P;
 };
 
-int check_dims(const ConvDims &d) {
+// map_h x map_w is the spatial size of the sample map (output for convolution,
+// input for transposed convolution).
+int check_dims(const ConvDims &d, int64_t map_h, int64_t map_w) {
   for (int64_t v : {d.B, d.Ci, d.Co, d.IH, d.IW, d.OH, d.OW, d.K, d.IH * d.IW, d.OH * d.OW})
     if (v <= 0 || v > 0x7fffffffLL) return MCX_E_SHAPE;
   if (d.P < 0 || d.P > 0x7fffffffLL || d.B > 65535) return MCX_E_SHAPE;
-  const int64_t pm = d.P ? d.P : 1;
-  // Largest tensors must be addressable with 63-bit element offsets and each
-  // plane / map with 31-bit ones.
-  if (d.OH * d.OW * d.K * pm * 2 > 0x7fffffffLL && d.IH * d.IW * d.K * pm * 2 > 0x7fffffffLL)
-    return MCX_E_SHAPE;
+  // every plane and the whole map are addressed with 31-bit element offsets
+  if (map_h * map_w * d.K * (d.P ? d.P : 1) * 2 > 0x7fffffffLL) return MCX_E_SHAPE;
+  if (d.Ci * d.Co * d.K > 0x7fffffffLL) return MCX_E_SHAPE;
   return 0;
 }
 
-template <typename T>
-int conv_forward_t(const void *x, const void *map, const void *iw, const void *w, const void *bias,
-                   void *y, const ConvDims &d, int interp, hipStream_t s) {
-  return generic_gather_product<T>((const T *)x, (const T *)map, (const T *)iw, (const T *)w,
-                                   (const T *)bias, (T *)y, d.B, d.Ci, d.Co, d.IH, d.IW,
-                                   d.OH * d.OW, d.K, d.P, interp, s);
+int check_ptrs(const void *a, const void *map, const void *iw, const void *w, int64_t P) {
+  if (!a || !map || !w) return MCX_E_NULL;
+  if ((P == 0) != (iw == nullptr)) return MCX_E_NULL;
+  return 0;
 }
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 template <typename T>
 int fill_zero(T *p, int64_t n, hipStream_t s);
@@ -40,9 +42,54 @@ int fill_zero<float>(float *p, int64_t n, hipStream_t s) { return fill_f32(p, n,
 template <>
 int fill_zero<double>(double *p, int64_t n, hipStream_t s) { return fill_f64(p, n, 0.0, s); }
 
+// ---- the three operators, typed ------------------------------------------------
+
+// y[b,o,n] = bias[o] + sum_{g,k} W[o,g,k] * sample(src[b,g], map[n,k]); n over MH x MW.
+size_t gather_product_ws(int dtype, int64_t G, int64_t O, int64_t K, int64_t P) {
+  if (dtype == MCX_F32 && mfma_f32_gather_product_supported(P))
+    return align256(mfma_f32_packed_weight_bytes(O, G, K));
+  return 0;
+}
+
+template <typename T>
+int gather_product(const T *src, const T *map, const T *iw, const T *w, const T *bias, T *y,
+                   void *ws, size_t ws_bytes, int64_t B, int64_t G, int64_t O, int64_t SH,
+                   int64_t SW, int64_t MH, int64_t MW, int64_t K, int64_t P, int interp,
+                   hipStream_t s) {
+  (void)ws;
+  (void)ws_bytes;
+  return generic_gather_product<T>(src, map, iw, w, bias, y, B, G, O, SH, SW, MH * MW, K, P,
+                                   interp, s);
+}
+
+template <>
+int gather_product<float>(const float *src, const float *map, const float *iw, const float *w,
+                          const float *bias, float *y, void *ws, size_t ws_bytes, int64_t B,
+                          int64_t G, int64_t O, int64_t SH, int64_t SW, int64_t MH, int64_t MW,
+                          int64_t K, int64_t P, int interp, hipStream_t s) {
+  if (!mfma_f32_gather_product_supported(P))
+    return generic_gather_product<float>(src, map, iw, w, bias, y, B, G, O, SH, SW, MH * MW, K, P,
+                                         interp, s);
+  if (!ws || ws_bytes < gather_product_ws(MCX_F32, G, O, K, P)) return MCX_E_WORKSPACE;
+  return mfma_f32_gather_product(src, map, iw, w, bias, y, (float *)ws, B, G, O, SH, SW, MH, MW,
+                                 K, P, interp, s);
+}
+
+template <typename T>
+int conv_forward_t(const void *x, const void *map, const void *iw, const void *w, const void *bias,
+                   void *y, void *ws, size_t ws_bytes, const ConvDims &d, int interp,
+                   hipStream_t s) {
+  return gather_product<T>((const T *)x, (const T *)map, (const T *)iw, (const T *)w,
+                           (const T *)bias, (T *)y, ws, ws_bytes, d.B, d.Ci, d.Co, d.IH, d.IW,
+                           d.OH, d.OW, d.K, d.P, interp, s);
+}
+
 template <typename T>
 int conv_backward_t(const void *gy, const void *map, const void *iw, const void *x, const void *w,
-                    void *gx, void *gw, void *gb, const ConvDims &d, int interp, hipStream_t s) {
+                    void *gx, void *gw, void *gb, void *ws, size_t ws_bytes, const ConvDims &d,
+                    int interp, hipStream_t s) {
+  (void)ws;
+  (void)ws_bytes;
   int rc = 0;
   const int64_t N = d.OH * d.OW;
   if (gx) {
@@ -74,14 +121,15 @@ int tconv_forward_t(const void *x, const void *map, const void *iw, const void *
 
 template <typename T>
 int tconv_backward_t(const void *gy, const void *map, const void *iw, const void *x,
-                     const void *w, void *gx, void *gw, void *gb, const ConvDims &d, int interp,
-                     hipStream_t s) {
+                     const void *w, void *gx, void *gw, void *gb, void *ws, size_t ws_bytes,
+                     const ConvDims &d, int interp, hipStream_t s) {
   int rc = 0;
   const int64_t N = d.IH * d.IW;
   if (gx) {
-    if ((rc = generic_gather_product<T>((const T *)gy, (const T *)map, (const T *)iw,
-                                        (const T *)w, (const T *)nullptr, (T *)gx, d.B, d.Co,
-                                        d.Ci, d.OH, d.OW, N, d.K, d.P, interp, s)))
+    // grad_input[b,ci] = sum_{co,k} W[ci,co,k] * sample(gy[b,co], map[n,k])
+    if ((rc = gather_product<T>((const T *)gy, (const T *)map, (const T *)iw, (const T *)w,
+                                (const T *)nullptr, (T *)gx, ws, ws_bytes, d.B, d.Co, d.Ci, d.OH,
+                                d.OW, d.IH, d.IW, d.K, d.P, interp, s)))
       return rc;
   }
   if (gw) {
@@ -94,26 +142,29 @@ int tconv_backward_t(const void *gy, const void *map, const void *iw, const void
   return rc;
 }
 
-int check_ptrs(const void *a, const void *map, const void *iw, const void *w, int64_t P) {
-  if (!a || !map || !w) return MCX_E_NULL;
-  if ((P == 0) != (iw == nullptr)) return MCX_E_NULL;
-  return 0;
-}
-
 }  // namespace
 
+extern "C" size_t mcx_conv_forward_workspace(int64_t, int64_t Ci, int64_t Co, int64_t, int64_t,
+                                             int64_t, int64_t, int64_t K, int64_t P, int dtype) {
+  return gather_product_ws(dtype, Ci, Co, K, P);
+}
+
 extern "C" int mcx_conv_forward(const void *x, const void *map, const void *iw, const void *w,
-                                const void *bias, void *y, int64_t B, int64_t Ci, int64_t Co,
+                                const void *bias, void *y, void *workspace,
+                                size_t workspace_bytes, int64_t B, int64_t Ci, int64_t Co,
                                 int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
                                 int64_t P, int interp, int dtype, void *stream) {
   const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
-  if (int rc = check_dims(d)) return rc;
+  if (int rc = check_dims(d, OH, OW)) return rc;
   if (int rc = check_ptrs(x, map, iw, w, P)) return rc;
   if (!bias || !y) return MCX_E_NULL;
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
-    case MCX_F32: return conv_forward_t<float>(x, map, iw, w, bias, y, d, interp, s);
-    case MCX_F64: return conv_forward_t<double>(x, map, iw, w, bias, y, d, interp, s);
+    case MCX_F32:
+      return conv_forward_t<float>(x, map, iw, w, bias, y, workspace, workspace_bytes, d, interp, s);
+    case MCX_F64:
+      return conv_forward_t<double>(x, map, iw, w, bias, y, workspace, workspace_bytes, d, interp,
+                                    s);
     default: return MCX_E_DTYPE;
   }
 }
@@ -128,26 +179,36 @@ extern "C" int mcx_conv_backward(const void *gy, const void *map, const void *iw
                                  size_t workspace_bytes, int64_t B, int64_t Ci, int64_t Co,
                                  int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
                                  int64_t P, int interp, int dtype, void *stream) {
-  (void)workspace;
-  (void)workspace_bytes;
   const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
-  if (int rc = check_dims(d)) return rc;
+  if (int rc = check_dims(d, OH, OW)) return rc;
   if (int rc = check_ptrs(gy, map, iw, w, P)) return rc;
   if (gw && !x) return MCX_E_NULL;
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
-    case MCX_F32: return conv_backward_t<float>(gy, map, iw, x, w, gx, gw, gb, d, interp, s);
-    case MCX_F64: return conv_backward_t<double>(gy, map, iw, x, w, gx, gw, gb, d, interp, s);
+    case MCX_F32:
+      return conv_backward_t<float>(gy, map, iw, x, w, gx, gw, gb, workspace, workspace_bytes, d,
+                                    interp, s);
+    case MCX_F64:
+      return conv_backward_t<double>(gy, map, iw, x, w, gx, gw, gb, workspace, workspace_bytes, d,
+                                     interp, s);
     default: return MCX_E_DTYPE;
   }
 }
 
+extern "C" size_t mcx_tconv_forward_workspace(int64_t, int64_t, int64_t, int64_t, int64_t,
+                                              int64_t, int64_t, int64_t, int64_t, int) {
+  return 0;
+}
+
 extern "C" int mcx_tconv_forward(const void *x, const void *map, const void *iw, const void *w,
-                                 const void *bias, void *y, int64_t B, int64_t Ci, int64_t Co,
+                                 const void *bias, void *y, void *workspace,
+                                 size_t workspace_bytes, int64_t B, int64_t Ci, int64_t Co,
                                  int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
                                  int64_t P, int interp, int dtype, void *stream) {
+  (void)workspace;
+  (void)workspace_bytes;
   const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
-  if (int rc = check_dims(d)) return rc;
+  if (int rc = check_dims(d, IH, IW)) return rc;
   if (int rc = check_ptrs(x, map, iw, w, P)) return rc;
   if (!bias || !y) return MCX_E_NULL;
   hipStream_t s = (hipStream_t)stream;
@@ -158,9 +219,11 @@ extern "C" int mcx_tconv_forward(const void *x, const void *map, const void *iw,
   }
 }
 
-extern "C" size_t mcx_tconv_backward_workspace(int64_t, int64_t, int64_t, int64_t, int64_t,
-                                               int64_t, int64_t, int64_t, int64_t, int) {
-  return 0;
+extern "C" size_t mcx_tconv_backward_workspace(int64_t, int64_t Ci, int64_t Co, int64_t, int64_t,
+                                               int64_t, int64_t, int64_t K, int64_t P,
+                                               int dtype) {
+  // backward-input is a gather-product with the channel roles swapped
+  return gather_product_ws(dtype, Co, Ci, K, P);
 }
 
 extern "C" int mcx_tconv_backward(const void *gy, const void *map, const void *iw, const void *x,
@@ -168,21 +231,23 @@ extern "C" int mcx_tconv_backward(const void *gy, const void *map, const void *i
                                   size_t workspace_bytes, int64_t B, int64_t Ci, int64_t Co,
                                   int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
                                   int64_t P, int interp, int dtype, void *stream) {
-  (void)workspace;
-  (void)workspace_bytes;
   const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
-  if (int rc = check_dims(d)) return rc;
+  if (int rc = check_dims(d, IH, IW)) return rc;
   if (int rc = check_ptrs(gy, map, iw, w, P)) return rc;
   if (gw && !x) return MCX_E_NULL;
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
-    case MCX_F32: return tconv_backward_t<float>(gy, map, iw, x, w, gx, gw, gb, d, interp, s);
-    case MCX_F64: return tconv_backward_t<double>(gy, map, iw, x, w, gx, gw, gb, d, interp, s);
+    case MCX_F32:
+      return tconv_backward_t<float>(gy, map, iw, x, w, gx, gw, gb, workspace, workspace_bytes, d,
+                                     interp, s);
+    case MCX_F64:
+      return tconv_backward_t<double>(gy, map, iw, x, w, gx, gw, gb, workspace, workspace_bytes, d,
+                                      interp, s);
     default: return MCX_E_DTYPE;
   }
 }
 
-extern "C" int mcx_abi_version(void) { return 1; }
+extern "C" int mcx_abi_version(void) { return 2; }
 
 extern "C" const char *mcx_error_string(int code) {
   switch (code) {

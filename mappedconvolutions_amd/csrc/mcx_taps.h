@@ -1,0 +1,56 @@
+// Weight-form taps for the matrix-core convolution kernels: a sample location is
+// resolved to NCORN (element offset, weight) pairs, and the sample is
+// sum_i wt[i] * plane[off[i]].  Corners outside the plane get weight 0 and offset 0
+// (a safe address), so the inner loops are branch-free.  interp_weights, when
+// present, are folded into the corner weights.  Semantics of each mode:
+// include/core/interpolation.h:85-238 of the reference.
+#pragma once
+
+#include "mcx_device.h"
+
+namespace mcx {
+
+template <int NCORN>
+struct PairTap {
+  int off[NCORN];
+  float wt[NCORN];
+};
+
+// NCORN == 1: nearest.  NCORN == 4: bilinear (wrap == false) or bispherical (wrap == true).
+template <int NCORN>
+__device__ inline void resolve_pairs(float x, float y, int h, int w, bool wrap, float scale,
+                                     PairTap<NCORN> &t) {
+  if (NCORN == 1) {
+    const int xi = to_int(round_half_away(x));
+    const int yi = to_int(round_half_away(y));
+    const bool ok = xi >= 0 && xi <= w - 1 && yi >= 0 && yi <= h - 1;
+    t.off[0] = ok ? yi * w + xi : 0;
+    t.wt[0] = ok ? scale : 0.f;
+  } else {
+    const float x1f = floorf(x), y1f = floorf(y);
+    int x1 = to_int(x1f), y1 = to_int(y1f);
+    int x2 = x1 + 1, y2 = y1 + 1;
+    bool x1ok, x2ok;
+    if (wrap) {
+      x1 = wrap_index(x1, w);
+      x2 = wrap_index(x2, w);
+      x1ok = x2ok = true;
+    } else {
+      x1ok = x1 >= 0 && x1 <= w - 1;
+      x2ok = x2 >= 0 && x2 <= w - 1;
+    }
+    const bool y1ok = y1 >= 0 && y1 <= h - 1;
+    const bool y2ok = y2 >= 0 && y2 <= h - 1;
+    const float A = (y1f + 1.f) - y, B = (x1f + 1.f) - x, C = x - x1f, D = y - y1f;
+    const bool ok[4] = {x1ok && y1ok, x2ok && y1ok, x1ok && y2ok, x2ok && y2ok};
+    const int o[4] = {y1 * w + x1, y1 * w + x2, y2 * w + x1, y2 * w + x2};
+    const float wv[4] = {A * B, A * C, D * B, D * C};
+#pragma unroll
+    for (int i = 0; i < NCORN; i++) {
+      t.off[i] = ok[i] ? o[i] : 0;
+      t.wt[i] = ok[i] ? wv[i] * scale : 0.f;
+    }
+  }
+}
+
+}  // namespace mcx
