@@ -36,4 +36,19 @@ int mfma_f32_gather_product(const float *src, const float *map, const float *iw,
                             int64_t O, int64_t SH, int64_t SW, int64_t OH, int64_t OW, int64_t K,
                             int64_t P, int interp, hipStream_t s);
 
+bool mfma_f32_weight_grad_supported(int64_t P);
+size_t mfma_f32_weight_grad_bytes(int64_t B, int64_t A, int64_t G, int64_t MH, int64_t MW,
+                                  int64_t K);
+int mfma_f32_weight_grad(const float *plain, const float *gath, const float *map, const float *iw,
+                         float *gw, float *part, int64_t B, int64_t A, int64_t G, int64_t GH,
+                         int64_t GW, int64_t MH, int64_t MW, int64_t K, int64_t P, int interp,
+                         hipStream_t s);
+
+bool mfma_f32_product_scatter_supported(int64_t P);
+size_t mfma_f32_scatter_weight_bytes(int64_t S, int64_t D, int64_t K);
+int mfma_f32_product_scatter(const float *src, const float *map, const float *iw, const float *w,
+                             float *dst, float *wq, int64_t B, int64_t S, int64_t D, int64_t DH,
+                             int64_t DW, int64_t MH, int64_t MW, int64_t K, int64_t P, int interp,
+                             hipStream_t s);
+
 }  // namespace mcx

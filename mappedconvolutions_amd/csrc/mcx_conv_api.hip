@@ -2,6 +2,7 @@
 // arguments, then routes each of the three products (gather-product,
 // product-scatter, weight gradient; see mcx_conv_generic.hip for the roles) to the
 // matrix-core kernels when they cover the case and to the scalar kernels otherwise.
+#include <algorithm>
 #include <initializer_list>
 
 #include "mcx.h"
@@ -75,6 +76,67 @@ int gather_product<float>(const float *src, const float *map, const float *iw, c
                                  K, P, interp, s);
 }
 
+// gW[a,g,k] = sum_{b,n} plain[b,a,n] * sample(gath[b,g], map[n,k]); n over MH x MW.
+size_t weight_grad_ws(int dtype, int64_t B, int64_t A, int64_t G, int64_t MH, int64_t MW,
+                      int64_t K, int64_t P) {
+  if (dtype == MCX_F32 && mfma_f32_weight_grad_supported(P))
+    return align256(mfma_f32_weight_grad_bytes(B, A, G, MH, MW, K));
+  return 0;
+}
+
+template <typename T>
+int weight_grad(const T *plain, const T *gath, const T *map, const T *iw, T *gw, void *ws,
+                size_t ws_bytes, int64_t B, int64_t A, int64_t G, int64_t GH, int64_t GW,
+                int64_t MH, int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s) {
+  (void)ws;
+  (void)ws_bytes;
+  return generic_weight_grad<T>(plain, gath, map, iw, gw, B, A, G, GH, GW, MH * MW, K, P, interp,
+                                s);
+}
+
+template <>
+int weight_grad<float>(const float *plain, const float *gath, const float *map, const float *iw,
+                       float *gw, void *ws, size_t ws_bytes, int64_t B, int64_t A, int64_t G,
+                       int64_t GH, int64_t GW, int64_t MH, int64_t MW, int64_t K, int64_t P,
+                       int interp, hipStream_t s) {
+  if (!mfma_f32_weight_grad_supported(P))
+    return generic_weight_grad<float>(plain, gath, map, iw, gw, B, A, G, GH, GW, MH * MW, K, P,
+                                      interp, s);
+  if (!ws || ws_bytes < weight_grad_ws(MCX_F32, B, A, G, MH, MW, K, P)) return MCX_E_WORKSPACE;
+  return mfma_f32_weight_grad(plain, gath, map, iw, gw, (float *)ws, B, A, G, GH, GW, MH, MW, K,
+                              P, interp, s);
+}
+
+// dst[b,d] += splat(sum_s W[s,d,k] * src[b,s,n], map[n,k]); n over MH x MW; dst pre-initialised.
+size_t product_scatter_ws(int dtype, int64_t S, int64_t D, int64_t K, int64_t P) {
+  if (dtype == MCX_F32 && mfma_f32_product_scatter_supported(P))
+    return align256(mfma_f32_scatter_weight_bytes(S, D, K));
+  return 0;
+}
+
+template <typename T>
+int product_scatter(const T *src, const T *map, const T *iw, const T *w, T *dst, void *ws,
+                    size_t ws_bytes, int64_t B, int64_t S, int64_t D, int64_t DH, int64_t DW,
+                    int64_t MH, int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s) {
+  (void)ws;
+  (void)ws_bytes;
+  return generic_product_scatter<T>(src, map, iw, w, dst, B, S, D, DH, DW, MH * MW, K, P, interp,
+                                    s);
+}
+
+template <>
+int product_scatter<float>(const float *src, const float *map, const float *iw, const float *w,
+                           float *dst, void *ws, size_t ws_bytes, int64_t B, int64_t S, int64_t D,
+                           int64_t DH, int64_t DW, int64_t MH, int64_t MW, int64_t K, int64_t P,
+                           int interp, hipStream_t s) {
+  if (!mfma_f32_product_scatter_supported(P))
+    return generic_product_scatter<float>(src, map, iw, w, dst, B, S, D, DH, DW, MH * MW, K, P,
+                                          interp, s);
+  if (!ws || ws_bytes < product_scatter_ws(MCX_F32, S, D, K, P)) return MCX_E_WORKSPACE;
+  return mfma_f32_product_scatter(src, map, iw, w, dst, (float *)ws, B, S, D, DH, DW, MH, MW, K,
+                                  P, interp, s);
+}
+
 template <typename T>
 int conv_forward_t(const void *x, const void *map, const void *iw, const void *w, const void *bias,
                    void *y, void *ws, size_t ws_bytes, const ConvDims &d, int interp,
@@ -88,21 +150,20 @@ template <typename T>
 int conv_backward_t(const void *gy, const void *map, const void *iw, const void *x, const void *w,
                     void *gx, void *gw, void *gb, void *ws, size_t ws_bytes, const ConvDims &d,
                     int interp, hipStream_t s) {
-  (void)ws;
-  (void)ws_bytes;
   int rc = 0;
   const int64_t N = d.OH * d.OW;
+  (void)N;
   if (gx) {
     if ((rc = fill_zero<T>((T *)gx, d.B * d.Ci * d.IH * d.IW, s))) return rc;
-    if ((rc = generic_product_scatter<T>((const T *)gy, (const T *)map, (const T *)iw,
-                                         (const T *)w, (T *)gx, d.B, d.Co, d.Ci, d.IH, d.IW, N,
-                                         d.K, d.P, interp, s)))
+    if ((rc = product_scatter<T>((const T *)gy, (const T *)map, (const T *)iw, (const T *)w,
+                                 (T *)gx, ws, ws_bytes, d.B, d.Co, d.Ci, d.IH, d.IW, d.OH, d.OW,
+                                 d.K, d.P, interp, s)))
       return rc;
   }
   if (gw) {
-    if ((rc = generic_weight_grad<T>((const T *)gy, (const T *)x, (const T *)map, (const T *)iw,
-                                     (T *)gw, d.B, d.Co, d.Ci, d.IH, d.IW, N, d.K, d.P, interp,
-                                     s)))
+    if ((rc = weight_grad<T>((const T *)gy, (const T *)x, (const T *)map, (const T *)iw, (T *)gw,
+                             ws, ws_bytes, d.B, d.Co, d.Ci, d.IH, d.IW, d.OH, d.OW, d.K, d.P,
+                             interp, s)))
       return rc;
   }
   if (gb) rc = channel_sum<T>((const T *)gy, (T *)gb, d.B, d.Co, N, s);
@@ -111,12 +172,13 @@ int conv_backward_t(const void *gy, const void *map, const void *iw, const void 
 
 template <typename T>
 int tconv_forward_t(const void *x, const void *map, const void *iw, const void *w,
-                    const void *bias, void *y, const ConvDims &d, int interp, hipStream_t s) {
+                    const void *bias, void *y, void *ws, size_t ws_bytes, const ConvDims &d,
+                    int interp, hipStream_t s) {
   int rc = fill_bias<T>((T *)y, (const T *)bias, d.B, d.Co, d.OH * d.OW, s);
   if (rc) return rc;
-  return generic_product_scatter<T>((const T *)x, (const T *)map, (const T *)iw, (const T *)w,
-                                    (T *)y, d.B, d.Ci, d.Co, d.OH, d.OW, d.IH * d.IW, d.K, d.P,
-                                    interp, s);
+  return product_scatter<T>((const T *)x, (const T *)map, (const T *)iw, (const T *)w, (T *)y, ws,
+                            ws_bytes, d.B, d.Ci, d.Co, d.OH, d.OW, d.IH, d.IW, d.K, d.P, interp,
+                            s);
 }
 
 template <typename T>
@@ -133,9 +195,9 @@ int tconv_backward_t(const void *gy, const void *map, const void *iw, const void
       return rc;
   }
   if (gw) {
-    if ((rc = generic_weight_grad<T>((const T *)x, (const T *)gy, (const T *)map, (const T *)iw,
-                                     (T *)gw, d.B, d.Ci, d.Co, d.OH, d.OW, N, d.K, d.P, interp,
-                                     s)))
+    if ((rc = weight_grad<T>((const T *)x, (const T *)gy, (const T *)map, (const T *)iw, (T *)gw,
+                             ws, ws_bytes, d.B, d.Ci, d.Co, d.OH, d.OW, d.IH, d.IW, d.K, d.P,
+                             interp, s)))
       return rc;
   }
   if (gb) rc = channel_sum<T>((const T *)gy, (T *)gb, d.B, d.Co, d.OH * d.OW, s);
@@ -169,9 +231,12 @@ extern "C" int mcx_conv_forward(const void *x, const void *map, const void *iw, 
   }
 }
 
-extern "C" size_t mcx_conv_backward_workspace(int64_t, int64_t, int64_t, int64_t, int64_t,
-                                              int64_t, int64_t, int64_t, int64_t, int) {
-  return 0;
+extern "C" size_t mcx_conv_backward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t,
+                                              int64_t, int64_t OH, int64_t OW, int64_t K,
+                                              int64_t P, int dtype) {
+  // the gradients run one after the other on the stream and share the scratch
+  return std::max(weight_grad_ws(dtype, B, Co, Ci, OH, OW, K, P),
+                  product_scatter_ws(dtype, Co, Ci, K, P));
 }
 
 extern "C" int mcx_conv_backward(const void *gy, const void *map, const void *iw, const void *x,
@@ -195,9 +260,9 @@ extern "C" int mcx_conv_backward(const void *gy, const void *map, const void *iw
   }
 }
 
-extern "C" size_t mcx_tconv_forward_workspace(int64_t, int64_t, int64_t, int64_t, int64_t,
-                                              int64_t, int64_t, int64_t, int64_t, int) {
-  return 0;
+extern "C" size_t mcx_tconv_forward_workspace(int64_t, int64_t Ci, int64_t Co, int64_t, int64_t,
+                                              int64_t, int64_t, int64_t K, int64_t P, int dtype) {
+  return product_scatter_ws(dtype, Ci, Co, K, P);
 }
 
 extern "C" int mcx_tconv_forward(const void *x, const void *map, const void *iw, const void *w,
@@ -205,25 +270,29 @@ extern "C" int mcx_tconv_forward(const void *x, const void *map, const void *iw,
                                  size_t workspace_bytes, int64_t B, int64_t Ci, int64_t Co,
                                  int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
                                  int64_t P, int interp, int dtype, void *stream) {
-  (void)workspace;
-  (void)workspace_bytes;
   const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
   if (int rc = check_dims(d, IH, IW)) return rc;
   if (int rc = check_ptrs(x, map, iw, w, P)) return rc;
   if (!bias || !y) return MCX_E_NULL;
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
-    case MCX_F32: return tconv_forward_t<float>(x, map, iw, w, bias, y, d, interp, s);
-    case MCX_F64: return tconv_forward_t<double>(x, map, iw, w, bias, y, d, interp, s);
+    case MCX_F32:
+      return tconv_forward_t<float>(x, map, iw, w, bias, y, workspace, workspace_bytes, d, interp,
+                                    s);
+    case MCX_F64:
+      return tconv_forward_t<double>(x, map, iw, w, bias, y, workspace, workspace_bytes, d,
+                                     interp, s);
     default: return MCX_E_DTYPE;
   }
 }
 
-extern "C" size_t mcx_tconv_backward_workspace(int64_t, int64_t Ci, int64_t Co, int64_t, int64_t,
-                                               int64_t, int64_t, int64_t K, int64_t P,
+extern "C" size_t mcx_tconv_backward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t IH,
+                                               int64_t IW, int64_t, int64_t, int64_t K, int64_t P,
                                                int dtype) {
-  // backward-input is a gather-product with the channel roles swapped
-  return gather_product_ws(dtype, Co, Ci, K, P);
+  // backward-input is a gather-product with the channel roles swapped; the two
+  // gradients run one after the other and share the scratch
+  return std::max(gather_product_ws(dtype, Co, Ci, K, P),
+                  weight_grad_ws(dtype, B, Ci, Co, IH, IW, K, P));
 }
 
 extern "C" int mcx_tconv_backward(const void *gy, const void *map, const void *iw, const void *x,

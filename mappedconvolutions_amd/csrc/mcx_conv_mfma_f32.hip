@@ -174,8 +174,589 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_mfma_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------------
+// weight_grad: gW[a,g,k] = sum_{b,n} plain[b,a,n] * sample(gath[b,g], map[n,k])
+// (convolution: plain = grad_output, gath = input; transposed: plain = input,
+// gath = grad_output).  The reduction dimension is the pixel axis, so a workgroup
+// walks a range of pixel tiles and keeps its slice of gW in MFMA accumulators:
+// 64 plain channels x 32 gathered channels x up to 9 taps.  Per tile the plain
+// tile P[64][128] is staged in LDS once and each wave keeps its 16 rows as MFMA A
+// operands in registers; per (tap, 16-channel block) the gathered samples go to
+// LDS as S[16][128] (same gather as the forward kernel) and every wave issues 32
+// v_mfma_f32_16x16x4_f32.  Each workgroup writes its partial gW to scratch; a
+// second kernel sums the partials in a fixed order (deterministic result).
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWgA = 64;            // plain channels per workgroup
+constexpr int kWgCB = 2;            // 16-channel blocks of gathered channels per workgroup
+constexpr int kWgKT = 9;            // taps per pass (accumulators in registers)
+constexpr int kLdPx = kTilePx + 4;  // LDS row stride (floats)
+
+template <int NCORN, int NP>
+__global__ __launch_bounds__(kThreads, 2) void weight_grad_mfma_kernel(
+    const float *__restrict__ plain, const float *__restrict__ gath,
+    const float *__restrict__ map, const float *__restrict__ iw, float *__restrict__ part, int A,
+    int G, int GH, int GW, int MH, int MW, int K, int weighted, int wrap, int tiles_x,
+    int tiles_per_img, int tw_shift, int total_tiles, int ranges, int cgroups) {
+  __shared__ __attribute__((aligned(16))) float Pt[kWgA][kLdPx];
+  __shared__ __attribute__((aligned(16))) float S[2][kGC][kLdPx];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l15 = lane & 15, lq = lane >> 4;
+  int range, cg;
+  if ((ranges & 7) == 0) {  // channel groups of one pixel range share an XCD (and its L2)
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    cg = slot % cgroups;
+    range = xcd * (ranges >> 3) + slot / cgroups;
+  } else {
+    cg = blockIdx.x % cgroups;
+    range = blockIdx.x / cgroups;
+  }
+  const int a0 = blockIdx.y * kWgA;
+  const int k_base = blockIdx.z * kWgKT;
+  const int ktaps = min(kWgKT, K - k_base);
+  const int tpr = (total_tiles + ranges - 1) / ranges;
+  const int t_begin = range * tpr, t_end = min(total_tiles, t_begin + tpr);
+  const int tw_mask = (1 << tw_shift) - 1, th = kTilePx >> tw_shift;
+  const int N = MH * MW;
+  const int64_t gplane = (int64_t)GH * GW;
+  const int p = tid & (kTilePx - 1), half = tid >> 7;
+  const int g_first = cg * (kWgCB * kGC);
+
+  floatx4 acc[kWgKT][kWgCB];
+#pragma unroll
+  for (int k = 0; k < kWgKT; k++)
+#pragma unroll
+    for (int cb = 0; cb < kWgCB; cb++) acc[k][cb] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  for (int tile = t_begin; tile < t_end; ++tile) {
+    const int b = tile / tiles_per_img;
+    const int t_in = tile - b * tiles_per_img;
+    const int tile_y = t_in / tiles_x, tile_x = t_in - tile_y * tiles_x;
+    const int i0 = tile_y * th, j0 = tile_x << tw_shift;
+
+    __syncthreads();  // everyone is done with the previous tile's LDS contents
+    {
+      const float *pb = plain + (int64_t)b * A * N;
+#pragma unroll 8
+      for (int r = 0; r < (kWgA * kTilePx) / kThreads; r++) {
+        const int e = tid + kThreads * r;
+        const int a = e >> 7, px = e & (kTilePx - 1);
+        const int i = i0 + (px >> tw_shift), j = j0 + (px & tw_mask);
+        const bool ok = (a0 + a) < A && i < MH && j < MW;
+        Pt[a][px] = ok ? pb[(int64_t)(a0 + a) * N + (int64_t)i * MW + j] : 0.f;
+      }
+    }
+    __syncthreads();
+    float areg[32];
+#pragma unroll
+    for (int s4 = 0; s4 < 8; s4++) {
+      const float4 t = *reinterpret_cast<const float4 *>(&Pt[wave * 16 + l15][16 * s4 + 4 * lq]);
+      areg[4 * s4 + 0] = t.x;
+      areg[4 * s4 + 1] = t.y;
+      areg[4 * s4 + 2] = t.z;
+      areg[4 * s4 + 3] = t.w;
+    }
+
+    const int gi = i0 + (p >> tw_shift), gj = j0 + (p & tw_mask);
+    const bool live = gi < MH && gj < MW;
+    const int64_t n_g = live ? (int64_t)gi * MW + gj : 0;
+    const float *gath_b = gath + (int64_t)b * G * gplane;
+
+    PairTap<NCORN> taps[NP];
+    float mx[NP], my[NP], mw[NP];
+    float v[8][NP * NCORN];
+    auto load_map = [&](int k) {
+#pragma unroll
+      for (int sp = 0; sp < NP; sp++) {
+        const int64_t e = (n_g * K + k) * NP + sp;
+        mx[sp] = map[e * 2];
+        my[sp] = map[e * 2 + 1];
+        mw[sp] = weighted ? iw[e] : 1.f;
+      }
+    };
+    auto resolve = [&]() {
+#pragma unroll
+      for (int sp = 0; sp < NP; sp++)
+        resolve_pairs<NCORN>(mx[sp], my[sp], GH, GW, wrap != 0, live ? mw[sp] : 0.f, taps[sp]);
+    };
+    auto issue = [&](int cb) {
+      const int g0 = g_first + cb * kGC + half * 8;
+#pragma unroll
+      for (int ch = 0; ch < 8; ch++) {
+        const float *pl = gath_b + (int64_t)min(g0 + ch, G - 1) * gplane;
+#pragma unroll
+        for (int sp = 0; sp < NP; sp++)
+#pragma unroll
+          for (int i = 0; i < NCORN; i++) v[ch][sp * NCORN + i] = pl[taps[sp].off[i]];
+      }
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+      for (int ch = 0; ch < 8; ch++) {
+        float s = 0.f;
+#pragma unroll
+        for (int sp = 0; sp < NP; sp++)
+#pragma unroll
+          for (int i = 0; i < NCORN; i++)
+            s = __builtin_fmaf(taps[sp].wt[i], v[ch][sp * NCORN + i], s);
+        S[buf][half * 8 + ch][p] = s;
+      }
+    };
+
+    load_map(k_base);
+    resolve();
+    if (ktaps > 1) load_map(k_base + 1);
+    issue(0);
+#pragma unroll
+    for (int k = 0; k < kWgKT; k++) {
+      if (k < ktaps) {
+#pragma unroll
+        for (int cb = 0; cb < kWgCB; cb++) {
+          const int buf = (k * kWgCB + cb) & 1;
+          stage(buf);
+          __syncthreads();
+          if (cb + 1 < kWgCB) {
+            issue(cb + 1);
+          } else if (k + 1 < ktaps) {
+            resolve();
+            if (k + 2 < ktaps) load_map(k_base + k + 2);
+            issue(0);
+          }
+#pragma unroll
+          for (int s4 = 0; s4 < 8; s4++) {
+            const float4 bq = *reinterpret_cast<const float4 *>(&S[buf][l15][16 * s4 + 4 * lq]);
+            acc[k][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[4 * s4 + 0], bq.x, acc[k][cb], 0, 0, 0);
+            acc[k][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[4 * s4 + 1], bq.y, acc[k][cb], 0, 0, 0);
+            acc[k][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[4 * s4 + 2], bq.z, acc[k][cb], 0, 0, 0);
+            acc[k][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[4 * s4 + 3], bq.w, acc[k][cb], 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+
+  // partial gW of this workgroup: lane holds gathered channel l15 of each block and
+  // plain channels a0 + 16*wave + 4*lq + i
+  float *pr = part + (int64_t)range * A * G * K;
+#pragma unroll
+  for (int k = 0; k < kWgKT; k++) {
+    if (k < ktaps) {
+#pragma unroll
+      for (int cb = 0; cb < kWgCB; cb++) {
+        const int g = g_first + cb * kGC + l15;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const int a = a0 + wave * 16 + lq * 4 + i;
+          if (a < A && g < G) pr[((int64_t)a * G + g) * K + k_base + k] = acc[k][cb][i];
+        }
+      }
+    }
+  }
+}
+
+__global__ void reduce_partials_kernel(const float *__restrict__ part, float *__restrict__ out,
+                                       int ranges, int64_t n) {
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= n) return;
+  float s = 0.f;
+  for (int r = 0; r < ranges; r++) s += part[(int64_t)r * n + e];
+  out[e] = s;
+}
+
+// ---------------------------------------------------------------------------------
+// product_scatter: dst[b,d] += splat(sum_s W[s,d,k] * src[b,s,n], map[n,k])
+// (convolution backward-input: s = Co, d = Ci; transposed forward: s = Ci, d = Co).
+// A workgroup owns a 2-D tile of 128 map pixels, one tile row of 32 per wave.  Each
+// wave keeps the source values of its 32 pixels (64 source channels) in registers
+// as MFMA B operands for the whole tile.  Destination channels are processed 16 at
+// a time: per tap the 64x16 weight slice is staged in LDS and
+// v_mfma_f32_16x16x4_f32 yields col[d][pixel] in registers.
+//
+// Scatter with LDS pre-reduction.  LDS float atomics retire about one lane every
+// few cycles on this part, so the window is accumulated WITHOUT atomics: every wave
+// owns a private LDS window covering the bounding box of its own pixels' destination
+// corners (rows x a circular interval of columns, found in a per-wave pre-pass over
+// the map), and adds into it with plain read-modify-write.  That is race-free when
+// the 16 lanes of one instruction hit 16 different slots, which holds whenever the
+// slots grow strictly along the pixel row; the kernel checks exactly that per
+// instruction (one cross-lane shift and a ballot) and sends the rare instruction
+// that fails the check, and waves whose box does not fit, to global atomics.  After
+// the K taps of a 16-channel block each wave flushes its window with one global
+// atomic per touched element and clears it.  Corners whose weight is exactly zero
+// (integer coordinates) are skipped.
+constexpr int kScDC = 16;        // destination channels per pass
+constexpr int kScWaveWin = 256;  // window slots per wave and destination channel
+constexpr int kScWinLd = 260;    // row stride: 4 rows apart = 16 banks apart
+constexpr int kScSC = 64;        // source channels per register block
+
+// Repack W[s][d][k] -> Wq[k][dc][s][16]: per (tap, 16-channel block) a contiguous
+// [Spad x 16] slice; s padded to 64, d padded to 16, zeros in the padding.
+__global__ void pack_scatter_weights_kernel(const float *__restrict__ w, float *__restrict__ wq,
+                                            int S, int D, int K, int Spad, int dchunks) {
+  const int64_t total = (int64_t)K * dchunks * Spad * kScDC;
+  for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total;
+       e += (int64_t)gridDim.x * blockDim.x) {
+    const int dl = (int)(e % kScDC);
+    const int s = (int)((e / kScDC) % Spad);
+    const int dc = (int)((e / ((int64_t)kScDC * Spad)) % dchunks);
+    const int k = (int)(e / ((int64_t)kScDC * Spad * dchunks));
+    const int d = dc * kScDC + dl;
+    wq[e] = (s < S && d < D) ? w[((int64_t)s * D + d) * K + k] : 0.f;
+  }
+}
+
+__device__ inline int wave_min(int v) {
+#pragma unroll
+  for (int m = 32; m > 0; m >>= 1) v = min(v, __shfl_xor(v, m, 64));
+  return v;
+}
+__device__ inline int wave_max(int v) {
+#pragma unroll
+  for (int m = 32; m > 0; m >>= 1) v = max(v, __shfl_xor(v, m, 64));
+  return v;
+}
+
+template <int NCORN, int NP>
+__global__ __launch_bounds__(kThreads, 2) void product_scatter_mfma_kernel(
+    const float *__restrict__ src, const float *__restrict__ map, const float *__restrict__ iw,
+    const float *__restrict__ wq, float *__restrict__ dst, int S, int D, int Spad, int DH, int DW,
+    int MH, int MW, int K, int weighted, int wrap, int tiles_x, int tiles_per_img, int tw_shift) {
+  __shared__ __attribute__((aligned(16))) float Win[kThreads / 64][kScDC][kScWinLd];
+  __shared__ __attribute__((aligned(16))) float Wt[2][kScSC][kScDC];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l15 = lane & 15, lq = lane >> 4;
+  const int tile = xcd_contiguous_tile(blockIdx.x, gridDim.x);
+  const int b = tile / tiles_per_img;
+  const int t_in = tile - b * tiles_per_img;
+  const int tile_y = t_in / tiles_x, tile_x = t_in - tile_y * tiles_x;
+  const int tw_mask = (1 << tw_shift) - 1, th = kTilePx >> tw_shift;
+  const int i0 = tile_y * th, j0 = tile_x << tw_shift;
+  const int N = MH * MW;
+  const int64_t dplane = (int64_t)DH * DW;
+  const int dchunks = (D + kScDC - 1) / kScDC;
+  const int schunks = Spad / kScSC;
+  const int halfw = DW >> 1;
+  float(*win)[kScWinLd] = Win[wave];
+
+  // ---- per-wave pre-pass: bounding box of the destination corners of the wave's
+  // 32 pixels (corners that are valid and carry a non-zero weight) ---------------
+  int xref, ymin, ymax, dmin, dmax;
+  {
+    const int px0 = wave * 32;
+    const int ri = min(i0 + (px0 >> tw_shift), MH - 1), rj = min(j0 + (px0 & tw_mask), MW - 1);
+    xref = wrap_index(to_int(floorf(map[((int64_t)ri * MW + rj) * K * NP * 2])), DW);
+    const int px = px0 + (lane & 31);
+    const int pi = i0 + (px >> tw_shift), pj = j0 + (px & tw_mask);
+    int vymin = 0x7fffffff, vymax = -0x7fffffff, vdmin = 0x7fffffff, vdmax = -0x7fffffff;
+    if (pi < MH && pj < MW) {
+      const int64_t n = (int64_t)pi * MW + pj;
+      for (int k = lane >> 5; k < K; k += 2) {
+#pragma unroll
+        for (int sp = 0; sp < NP; sp++) {
+          const int64_t e = (n * K + k) * NP + sp;
+          CoordTap<NCORN> t;
+          resolve_coords<NCORN>(map[e * 2], map[e * 2 + 1], DH, DW, wrap != 0,
+                                weighted ? iw[e] : 1.f, t);
+#pragma unroll
+          for (int c = 0; c < NCORN; c++) {
+            if ((t.ok & (1u << c)) && t.wt[c] != 0.f) {
+              const int dx = wrap_index(t.xx[c] - xref + halfw, DW) - halfw;
+              vymin = min(vymin, t.yy[c]);
+              vymax = max(vymax, t.yy[c]);
+              vdmin = min(vdmin, dx);
+              vdmax = max(vdmax, dx);
+            }
+          }
+        }
+      }
+    }
+    ymin = wave_min(vymin);
+    ymax = wave_max(vymax);
+    dmin = wave_min(vdmin);
+    dmax = wave_max(vdmax);
+  }
+  const bool any_target = ymin <= ymax;
+  const int ww = any_target ? dmax - dmin + 1 : 1, wh = any_target ? ymax - ymin + 1 : 1;
+  const int wsz = ww * wh;
+  const bool use_lds = any_target && wsz <= kScWaveWin;
+
+  // global offsets of the window slots this lane flushes
+  int goff[kScWaveWin / 64];
+#pragma unroll
+  for (int r = 0; r < kScWaveWin / 64; r++) {
+    const int slot = lane + r * 64;
+    if (use_lds && slot < wsz) {
+      const int wy = slot / ww, wx = slot - wy * ww;
+      goff[r] = (ymin + wy) * DW + wrap_index(xref + dmin + wx, DW);
+    } else {
+      goff[r] = -1;
+    }
+  }
+  for (int e = lane; e < kScDC * kScWinLd; e += 64) (&win[0][0])[e] = 0.f;
+
+  // ---- this lane's two pixels (MFMA column l15 of column blocks 0 and 1) -------
+  int64_t npx[2];
+  bool live[2];
+#pragma unroll
+  for (int nb = 0; nb < 2; nb++) {
+    const int px = wave * 32 + nb * 16 + l15;
+    const int pi = i0 + (px >> tw_shift), pj = j0 + (px & tw_mask);
+    live[nb] = pi < MH && pj < MW;
+    npx[nb] = live[nb] ? (int64_t)pi * MW + pj : 0;
+  }
+  const float *src_b = src + (int64_t)b * S * N;
+  float *dst_b = dst + (int64_t)b * D * dplane;
+
+  float breg[2][16];
+  auto load_b = [&](int sc) {
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+      for (int t = 0; t < 16; t++) {
+        const int s = sc * kScSC + 4 * t + lq;
+        breg[nb][t] = (live[nb] && s < S) ? src_b[(int64_t)s * N + npx[nb]] : 0.f;
+      }
+  };
+  if (schunks == 1) load_b(0);
+
+  const int units = dchunks * K * schunks;  // unit = (dc, k, sc), sc fastest
+  float4 wpre;
+  auto prefetch_w = [&](int dc, int k, int sc) {
+    wpre = reinterpret_cast<const float4 *>(
+        wq + (((int64_t)k * dchunks + dc) * Spad + sc * kScSC) * kScDC)[tid];
+  };
+  prefetch_w(0, 0, 0);
+
+  int dc = 0, k = 0, sc = 0;
+  floatx4 acc[2];
+  for (int u = 0; u < units; ++u) {
+    const int buf = u & 1;
+    reinterpret_cast<float4 *>(&Wt[buf][0][0])[tid] = wpre;
+    if (schunks > 1) load_b(sc);
+    if (sc == 0) {
+      acc[0] = floatx4{0.f, 0.f, 0.f, 0.f};
+      acc[1] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+    // map entries of this tap for the lane's two pixels (consumed after the MFMAs)
+    float mx[2][NP], my[2][NP], mw[2][NP];
+    const bool last_sc = sc + 1 == schunks;
+    if (last_sc) {
+#pragma unroll
+      for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+        for (int sp = 0; sp < NP; sp++) {
+          const int64_t e = (npx[nb] * K + k) * NP + sp;
+          mx[nb][sp] = map[e * 2];
+          my[nb][sp] = map[e * 2 + 1];
+          mw[nb][sp] = weighted ? iw[e] : 1.f;
+        }
+    }
+    __syncthreads();
+    // advance and prefetch the next unit's weights
+    const int cdc = dc, ck = k;
+    if (++sc == schunks) {
+      sc = 0;
+      if (++k == K) {
+        k = 0;
+        ++dc;
+      }
+    }
+    if (u + 1 < units) prefetch_w(dc, k, sc);
+
+#pragma unroll
+    for (int t = 0; t < 16; t++) {
+      const float a = Wt[buf][4 * t + lq][l15];
+      acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, breg[0][t], acc[0], 0, 0, 0);
+      acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, breg[1][t], acc[1], 0, 0, 0);
+    }
+
+    if (!last_sc) continue;
+    // scatter col[d = cdc*16 + lq*4 + i][pixel nb] through tap ck
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++) {
+#pragma unroll
+      for (int sp = 0; sp < NP; sp++) {
+        CoordTap<NCORN> t;
+        resolve_coords<NCORN>(mx[nb][sp], my[nb][sp], DH, DW, wrap != 0, mw[nb][sp], t);
+#pragma unroll
+        for (int c = 0; c < NCORN; c++) {
+          const bool valid = live[nb] && (t.ok & (1u << c)) && t.wt[c] != 0.f;
+          bool direct = !use_lds;
+          int slot = 0;
+          if (use_lds) {
+            const int dx = wrap_index(t.xx[c] - xref + halfw, DW) - halfw;
+            slot = (t.yy[c] - ymin) * ww + (dx - dmin);
+            // race-free iff the valid lanes of each 16-lane group form one run with
+            // strictly increasing slots (the four groups hold different channels)
+            const int prev = __shfl_up(slot, 1, 16);
+            const int pvalid = __shfl_up((int)valid, 1, 16);
+            const bool clash = valid && l15 > 0 && pvalid && slot <= prev;
+            const unsigned m = (unsigned)(__ballot(valid) & 0xffffu);
+            const unsigned run = m ? (m >> __builtin_ctz(m)) : 0u;
+            direct = __ballot(clash) != 0 || (run & (run + 1u)) != 0u;
+          }
+          if (!valid) continue;
+          if (!direct) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) win[lq * 4 + i][slot] += t.wt[c] * acc[nb][i];
+          } else {
+            const int off = t.yy[c] * DW + t.xx[c];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+              const int d = cdc * kScDC + lq * 4 + i;
+              if (d < D) atomic_add(dst_b + (int64_t)d * dplane + off, t.wt[c] * acc[nb][i]);
+            }
+          }
+        }
+      }
+    }
+    // after the last tap of a destination-channel block: flush and clear the window
+    if (use_lds && ck == K - 1) {
+#pragma unroll
+      for (int r = 0; r < kScWaveWin / 64; r++) {
+        if (goff[r] < 0) continue;
+        const int slot = lane + r * 64;
+#pragma unroll
+        for (int dl = 0; dl < kScDC; dl++) {
+          const float val = win[dl][slot];
+          const int d = cdc * kScDC + dl;
+          if (val != 0.f && d < D) atomic_add(dst_b + (int64_t)d * dplane + goff[r], val);
+          win[dl][slot] = 0.f;
+        }
+      }
+    }
+  }
+}
+
+struct PixelTiling {
+  int tw_shift, tiles_x, tiles_per_img;
+  int64_t total;
+};
+
+// 2-D pixel tiles of 128: 4 x 32 when the map has at least 4 rows, else 1 x 128.
+inline PixelTiling make_tiling(int64_t B, int64_t H, int64_t W) {
+  PixelTiling t;
+  t.tw_shift = H >= 4 ? 5 : 7;
+  const int tw = 1 << t.tw_shift, th = kTilePx >> t.tw_shift;
+  t.tiles_x = (int)((W + tw - 1) / tw);
+  t.tiles_per_img = t.tiles_x * (int)((H + th - 1) / th);
+  t.total = (int64_t)t.tiles_per_img * B;
+  return t;
+}
+
+inline int weight_grad_ranges(int64_t total_tiles, int64_t A, int64_t G, int64_t K) {
+  const int64_t per_range = ((G + kWgCB * kGC - 1) / (kWgCB * kGC)) * ((A + kWgA - 1) / kWgA) *
+                            ((K + kWgKT - 1) / kWgKT);
+  int64_t r = std::max<int64_t>(8, (512 / per_range) / 8 * 8);  // about two workgroups per CU
+  return (int)std::min<int64_t>(r, std::max<int64_t>(total_tiles, 1));
+}
+
 inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
 
+}  // namespace
+
+bool mfma_f32_weight_grad_supported(int64_t P) { return P >= 0 && P <= 4; }
+
+size_t mfma_f32_weight_grad_bytes(int64_t B, int64_t A, int64_t G, int64_t MH, int64_t MW,
+                                  int64_t K) {
+  const PixelTiling t = make_tiling(B, MH, MW);
+  return (size_t)weight_grad_ranges(t.total, A, G, K) * (size_t)(A * G * K) * sizeof(float);
+}
+
+// part: scratch of mfma_f32_weight_grad_bytes(...) bytes.
+int mfma_f32_weight_grad(const float *plain, const float *gath, const float *map, const float *iw,
+                         float *gw, float *part, int64_t B, int64_t A, int64_t G, int64_t GH,
+                         int64_t GW, int64_t MH, int64_t MW, int64_t K, int64_t P, int interp,
+                         hipStream_t s) {
+  const PixelTiling t = make_tiling(B, MH, MW);
+  if (t.total > 0x7fffffffLL) return MCX_E_SHAPE;
+  const int ranges = weight_grad_ranges(t.total, A, G, K);
+  const int cgroups = (int)((G + kWgCB * kGC - 1) / (kWgCB * kGC));
+  dim3 grid((unsigned)(ranges * cgroups), (unsigned)((A + kWgA - 1) / kWgA),
+            (unsigned)((K + kWgKT - 1) / kWgKT));
+  const int mode = canonical_interp(interp);
+  const int weighted = P > 0 ? 1 : 0, wrap = mode == kInterpBispherical ? 1 : 0;
+  const int np = P > 0 ? (int)P : 1;
+#define MCX_LAUNCH(NCORN, NP)                                                                    \
+  hipLaunchKernelGGL((weight_grad_mfma_kernel<NCORN, NP>), grid, dim3(kThreads), 0, s, plain,    \
+                     gath, map, iw, part, (int)A, (int)G, (int)GH, (int)GW, (int)MH, (int)MW,    \
+                     (int)K, weighted, wrap, t.tiles_x, t.tiles_per_img, t.tw_shift,             \
+                     (int)t.total, ranges, cgroups)
+  if (mode == kInterpNearest) {
+    switch (np) {
+      case 1: MCX_LAUNCH(1, 1); break;
+      case 2: MCX_LAUNCH(1, 2); break;
+      case 3: MCX_LAUNCH(1, 3); break;
+      default: MCX_LAUNCH(1, 4); break;
+    }
+  } else {
+    switch (np) {
+      case 1: MCX_LAUNCH(4, 1); break;
+      case 2: MCX_LAUNCH(4, 2); break;
+      case 3: MCX_LAUNCH(4, 3); break;
+      default: MCX_LAUNCH(4, 4); break;
+    }
+  }
+#undef MCX_LAUNCH
+  MCX_HIP_CHECK_LAUNCH();
+  const int64_t n = A * G * K;
+  hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s,
+                     part, gw, ranges, n);
+  MCX_HIP_CHECK_LAUNCH();
+  return 0;
+}
+
+bool mfma_f32_product_scatter_supported(int64_t P) { return P >= 0 && P <= 4; }
+
+size_t mfma_f32_scatter_weight_bytes(int64_t S, int64_t D, int64_t K) {
+  return (size_t)(K * ((D + kScDC - 1) / kScDC) * round_up(S, kScSC) * kScDC) * sizeof(float);
+}
+
+// dst must already hold its initial value (zeros or the bias); wq: scratch of
+// mfma_f32_scatter_weight_bytes(S, D, K) bytes.
+int mfma_f32_product_scatter(const float *src, const float *map, const float *iw, const float *w,
+                             float *dst, float *wq, int64_t B, int64_t S, int64_t D, int64_t DH,
+                             int64_t DW, int64_t MH, int64_t MW, int64_t K, int64_t P, int interp,
+                             hipStream_t s) {
+  const int Spad = (int)round_up(S, kScSC), dchunks = (int)((D + kScDC - 1) / kScDC);
+  const int64_t packed = (int64_t)K * dchunks * Spad * kScDC;
+  hipLaunchKernelGGL(pack_scatter_weights_kernel,
+                     dim3((unsigned)std::min<int64_t>((packed + 255) / 256, 4096)), dim3(256), 0, s,
+                     w, wq, (int)S, (int)D, (int)K, Spad, dchunks);
+  MCX_HIP_CHECK_LAUNCH();
+  const PixelTiling t = make_tiling(B, MH, MW);
+  if (t.total > 0x7fffffffLL) return MCX_E_SHAPE;
+  dim3 grid((unsigned)t.total);
+  const int mode = canonical_interp(interp);
+  const int weighted = P > 0 ? 1 : 0, wrap = mode == kInterpBispherical ? 1 : 0;
+  const int np = P > 0 ? (int)P : 1;
+#define MCX_LAUNCH(NCORN, NP)                                                                    \
+  hipLaunchKernelGGL((product_scatter_mfma_kernel<NCORN, NP>), grid, dim3(kThreads), 0, s, src,  \
+                     map, iw, wq, dst, (int)S, (int)D, Spad, (int)DH, (int)DW, (int)MH, (int)MW, \
+                     (int)K, weighted, wrap, t.tiles_x, t.tiles_per_img, t.tw_shift)
+  if (mode == kInterpNearest) {
+    switch (np) {
+      case 1: MCX_LAUNCH(1, 1); break;
+      case 2: MCX_LAUNCH(1, 2); break;
+      case 3: MCX_LAUNCH(1, 3); break;
+      default: MCX_LAUNCH(1, 4); break;
+    }
+  } else {
+    switch (np) {
+      case 1: MCX_LAUNCH(4, 1); break;
+      case 2: MCX_LAUNCH(4, 2); break;
+      case 3: MCX_LAUNCH(4, 3); break;
+      default: MCX_LAUNCH(4, 4); break;
+    }
+  }
+#undef MCX_LAUNCH
+  MCX_HIP_CHECK_LAUNCH();
+  return 0;
+}
+
+namespace {
 }  // namespace
 
 size_t mfma_f32_packed_weight_bytes(int64_t O, int64_t G, int64_t K) {
@@ -194,12 +775,9 @@ int mfma_f32_gather_product(const float *src, const float *map, const float *iw,
   hipLaunchKernelGGL(pack_weights_kernel, dim3((unsigned)std::min<int64_t>((packed + 255) / 256, 4096)),
                      dim3(256), 0, s, w, wp, (int)O, (int)G, (int)K, Opad, Gpad);
   MCX_HIP_CHECK_LAUNCH();
-  // 2-D pixel tiles: 4 x 32 when the output has at least 4 rows, else 1 x 128
-  const int tw_shift = OH >= 4 ? 5 : 7;
-  const int tw = 1 << tw_shift, th = kTilePx >> tw_shift;
-  const int tiles_x = (int)((OW + tw - 1) / tw), tiles_y = (int)((OH + th - 1) / th);
-  const int tiles_per_img = tiles_x * tiles_y;
-  const int64_t total = (int64_t)tiles_per_img * B;
+  const PixelTiling t = make_tiling(B, OH, OW);
+  const int tw_shift = t.tw_shift, tiles_x = t.tiles_x, tiles_per_img = t.tiles_per_img;
+  const int64_t total = t.total;
   if (total > 0x7fffffffLL) return MCX_E_SHAPE;
   dim3 grid((unsigned)total, (unsigned)(Opad / kOT));
   const int mode = canonical_interp(interp);

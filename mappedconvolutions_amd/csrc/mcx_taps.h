@@ -53,4 +53,53 @@ __device__ inline void resolve_pairs(float x, float y, int h, int w, bool wrap, 
   }
 }
 
+// Coordinate form of the same taps, for scatters that need the destination row
+// and column of every corner (valid bit i of `ok` set when corner i is inside).
+template <int NCORN>
+struct CoordTap {
+  int yy[NCORN], xx[NCORN];
+  float wt[NCORN];
+  unsigned ok;
+};
+
+template <int NCORN>
+__device__ inline void resolve_coords(float x, float y, int h, int w, bool wrap, float scale,
+                                      CoordTap<NCORN> &t) {
+  if (NCORN == 1) {
+    const int xi = to_int(round_half_away(x));
+    const int yi = to_int(round_half_away(y));
+    t.ok = (xi >= 0 && xi <= w - 1 && yi >= 0 && yi <= h - 1) ? 1u : 0u;
+    t.yy[0] = yi;
+    t.xx[0] = xi;
+    t.wt[0] = scale;
+  } else {
+    const float x1f = floorf(x), y1f = floorf(y);
+    int x1 = to_int(x1f), y1 = to_int(y1f);
+    int x2 = x1 + 1, y2 = y1 + 1;
+    bool x1ok, x2ok;
+    if (wrap) {
+      x1 = wrap_index(x1, w);
+      x2 = wrap_index(x2, w);
+      x1ok = x2ok = true;
+    } else {
+      x1ok = x1 >= 0 && x1 <= w - 1;
+      x2ok = x2 >= 0 && x2 <= w - 1;
+    }
+    const bool y1ok = y1 >= 0 && y1 <= h - 1;
+    const bool y2ok = y2 >= 0 && y2 <= h - 1;
+    const float A = (y1f + 1.f) - y, B = (x1f + 1.f) - x, C = x - x1f, D = y - y1f;
+    const int ys[4] = {y1, y1, y2, y2};
+    const int xs[4] = {x1, x2, x1, x2};
+    const float wv[4] = {A * B, A * C, D * B, D * C};
+    t.ok = (x1ok && y1ok ? 1u : 0u) | (x2ok && y1ok ? 2u : 0u) | (x1ok && y2ok ? 4u : 0u) |
+           (x2ok && y2ok ? 8u : 0u);
+#pragma unroll
+    for (int i = 0; i < NCORN; i++) {
+      t.yy[i] = ys[i];
+      t.xx[i] = xs[i];
+      t.wt[i] = wv[i] * scale;
+    }
+  }
+}
+
 }  // namespace mcx
