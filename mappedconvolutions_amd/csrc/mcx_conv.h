@@ -23,8 +23,10 @@ template <typename T>
 int generic_weight_grad(const T *plain, const T *gath, const T *map, const T *iw, T *gw,
                         int64_t B, int64_t A, int64_t G, int64_t GH, int64_t GW, int64_t N,
                         int64_t K, int64_t P, int interp, hipStream_t s);
+// scratch: channel_sum_scratch_bytes(...) bytes, or NULL for the single-kernel form.
+size_t channel_sum_scratch_bytes(int64_t B, int64_t C, int64_t N, size_t elem);
 template <typename T>
-int channel_sum(const T *g, T *gb, int64_t B, int64_t C, int64_t N, hipStream_t s);
+int channel_sum(const T *g, T *gb, T *scratch, int64_t B, int64_t C, int64_t N, hipStream_t s);
 template <typename T>
 int fill_bias(T *y, const T *bias, int64_t B, int64_t C, int64_t N, hipStream_t s);
 

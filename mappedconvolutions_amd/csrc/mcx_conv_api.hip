@@ -137,6 +137,15 @@ int product_scatter<float>(const float *src, const float *map, const float *iw, 
                                   P, interp, s);
 }
 
+// gb[c] = sum over (b, n) of gy[b,c,n]; uses the scratch when it is large enough.
+template <typename T>
+int bias_grad(const T *gy, T *gb, void *ws, size_t ws_bytes, int64_t B, int64_t C, int64_t N,
+              hipStream_t s) {
+  const size_t need = channel_sum_scratch_bytes(B, C, N, sizeof(T));
+  T *scratch = (ws && need > 0 && ws_bytes >= need) ? (T *)ws : nullptr;
+  return channel_sum<T>(gy, gb, scratch, B, C, N, s);
+}
+
 template <typename T>
 int conv_forward_t(const void *x, const void *map, const void *iw, const void *w, const void *bias,
                    void *y, void *ws, size_t ws_bytes, const ConvDims &d, int interp,
@@ -166,7 +175,7 @@ int conv_backward_t(const void *gy, const void *map, const void *iw, const void 
                              interp, s)))
       return rc;
   }
-  if (gb) rc = channel_sum<T>((const T *)gy, (T *)gb, d.B, d.Co, N, s);
+  if (gb) rc = bias_grad<T>((const T *)gy, (T *)gb, ws, ws_bytes, d.B, d.Co, d.OH * d.OW, s);
   return rc;
 }
 
@@ -200,7 +209,7 @@ int tconv_backward_t(const void *gy, const void *map, const void *iw, const void
                              interp, s)))
       return rc;
   }
-  if (gb) rc = channel_sum<T>((const T *)gy, (T *)gb, d.B, d.Co, d.OH * d.OW, s);
+  if (gb) rc = bias_grad<T>((const T *)gy, (T *)gb, ws, ws_bytes, d.B, d.Co, d.OH * d.OW, s);
   return rc;
 }
 
@@ -235,8 +244,10 @@ extern "C" size_t mcx_conv_backward_workspace(int64_t B, int64_t Ci, int64_t Co,
                                               int64_t, int64_t OH, int64_t OW, int64_t K,
                                               int64_t P, int dtype) {
   // the gradients run one after the other on the stream and share the scratch
-  return std::max(weight_grad_ws(dtype, B, Co, Ci, OH, OW, K, P),
-                  product_scatter_ws(dtype, Co, Ci, K, P));
+  const size_t elem = dtype == MCX_F64 ? 8 : 4;
+  return std::max({weight_grad_ws(dtype, B, Co, Ci, OH, OW, K, P),
+                   product_scatter_ws(dtype, Co, Ci, K, P),
+                   align256(channel_sum_scratch_bytes(B, Co, OH * OW, elem))});
 }
 
 extern "C" int mcx_conv_backward(const void *gy, const void *map, const void *iw, const void *x,
@@ -287,12 +298,14 @@ extern "C" int mcx_tconv_forward(const void *x, const void *map, const void *iw,
 }
 
 extern "C" size_t mcx_tconv_backward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t IH,
-                                               int64_t IW, int64_t, int64_t, int64_t K, int64_t P,
-                                               int dtype) {
-  // backward-input is a gather-product with the channel roles swapped; the two
+                                               int64_t IW, int64_t OH, int64_t OW, int64_t K,
+                                               int64_t P, int dtype) {
+  // backward-input is a gather-product with the channel roles swapped; the
   // gradients run one after the other and share the scratch
-  return std::max(gather_product_ws(dtype, Co, Ci, K, P),
-                  weight_grad_ws(dtype, B, Ci, Co, IH, IW, K, P));
+  const size_t elem = dtype == MCX_F64 ? 8 : 4;
+  return std::max({gather_product_ws(dtype, Co, Ci, K, P),
+                   weight_grad_ws(dtype, B, Ci, Co, IH, IW, K, P),
+                   align256(channel_sum_scratch_bytes(B, Co, OH * OW, elem))});
 }
 
 extern "C" int mcx_tconv_backward(const void *gy, const void *map, const void *iw, const void *x,

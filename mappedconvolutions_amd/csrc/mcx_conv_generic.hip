@@ -163,6 +163,38 @@ __global__ __launch_bounds__(kThreads) void channel_sum_kernel(const T *__restri
   if (threadIdx.x == 0) gb[c] = red[0];
 }
 
+// Two-stage form of the same sum for large tensors: stage 1 reduces one slice of one
+// (image, channel) plane per workgroup into part[c][b*splits + s]; stage 2 adds the
+// partials of a channel in a fixed order.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void channel_sum_partial_kernel(
+    const T *__restrict__ g, T *__restrict__ part, int C, int N, int splits) {
+  const int c = blockIdx.x, b = blockIdx.y, sp = blockIdx.z;
+  const int per = (N + splits - 1) / splits;
+  const int n0 = sp * per, n1 = min(N, n0 + per);
+  const T *p = g + ((int64_t)b * C + c) * N;
+  T acc = T(0);
+  for (int n = n0 + threadIdx.x; n < n1; n += kThreads) acc += p[n];
+  __shared__ T red[kThreads];
+  red[threadIdx.x] = acc;
+  __syncthreads();
+  for (int stride = kThreads / 2; stride > 0; stride >>= 1) {
+    if ((int)threadIdx.x < stride) red[threadIdx.x] += red[threadIdx.x + stride];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) part[(int64_t)c * gridDim.y * splits + b * splits + sp] = red[0];
+}
+
+template <typename T>
+__global__ void channel_sum_final_kernel(const T *__restrict__ part, T *__restrict__ gb, int C,
+                                         int per_channel) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  T acc = T(0);
+  for (int i = 0; i < per_channel; i++) acc += part[(int64_t)c * per_channel + i];
+  gb[c] = acc;
+}
+
 template <typename T>
 __global__ void fill_bias_kernel(T *__restrict__ y, const T *__restrict__ bias, int C, int N,
                                  int64_t total) {
@@ -211,10 +243,31 @@ int generic_weight_grad(const T *plain, const T *gath, const T *map, const T *iw
   return 0;
 }
 
+int channel_sum_splits(int64_t B, int64_t C, int64_t N) {
+  if (B * C * N < (1 << 20) || B > 65535) return 0;  // small: one kernel, no scratch
+  int splits = 1;
+  while (B * C * splits < 2048 && N / (splits * 2) >= 4096 && splits < 64) splits *= 2;
+  return splits;
+}
+
+size_t channel_sum_scratch_bytes(int64_t B, int64_t C, int64_t N, size_t elem) {
+  return (size_t)(B * C * channel_sum_splits(B, C, N)) * elem;
+}
+
 template <typename T>
-int channel_sum(const T *g, T *gb, int64_t B, int64_t C, int64_t N, hipStream_t s) {
-  hipLaunchKernelGGL(channel_sum_kernel<T>, dim3((unsigned)C), dim3(kThreads), 0, s, g, gb, (int)B,
-                     (int)C, (int)N);
+int channel_sum(const T *g, T *gb, T *scratch, int64_t B, int64_t C, int64_t N, hipStream_t s) {
+  const int splits = scratch ? channel_sum_splits(B, C, N) : 0;
+  if (splits == 0) {
+    hipLaunchKernelGGL(channel_sum_kernel<T>, dim3((unsigned)C), dim3(kThreads), 0, s, g, gb,
+                       (int)B, (int)C, (int)N);
+    MCX_HIP_CHECK_LAUNCH();
+    return 0;
+  }
+  hipLaunchKernelGGL(channel_sum_partial_kernel<T>, dim3((unsigned)C, (unsigned)B, (unsigned)splits),
+                     dim3(kThreads), 0, s, g, scratch, (int)C, (int)N, splits);
+  MCX_HIP_CHECK_LAUNCH();
+  hipLaunchKernelGGL(channel_sum_final_kernel<T>, dim3((unsigned)((C + 63) / 64)), dim3(64), 0, s,
+                     scratch, gb, (int)C, (int)(B * splits));
   MCX_HIP_CHECK_LAUNCH();
   return 0;
 }
@@ -239,7 +292,7 @@ int fill_bias(T *y, const T *bias, int64_t B, int64_t C, int64_t N, hipStream_t 
   template int generic_weight_grad<T>(const T *, const T *, const T *, const T *, T *, int64_t,   \
                                       int64_t, int64_t, int64_t, int64_t, int64_t, int64_t,       \
                                       int64_t, int, hipStream_t);                                 \
-  template int channel_sum<T>(const T *, T *, int64_t, int64_t, int64_t, hipStream_t);            \
+  template int channel_sum<T>(const T *, T *, T *, int64_t, int64_t, int64_t, hipStream_t);       \
   template int fill_bias<T>(T *, const T *, int64_t, int64_t, int64_t, hipStream_t);
 MCX_INSTANTIATE(float)
 MCX_INSTANTIATE(double)

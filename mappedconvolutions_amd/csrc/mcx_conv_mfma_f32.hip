@@ -68,7 +68,7 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_mfma_kernel(
 
   // gather role: pixel p of the tile, channels [half*8, half*8+8) of each chunk
   const int p = tid & (kTilePx - 1);
-  const int half = tid >> 7;
+  const int half = __builtin_amdgcn_readfirstlane(tid >> 7);  // wave-uniform: scalar addressing
   const int gi = tile_y * th + (p >> tw_shift), gj = (tile_x << tw_shift) + (p & tw_mask);
   const bool live = gi < OH && gj < OW;
   const int64_t n_g = live ? (int64_t)gi * OW + gj : 0;
@@ -81,6 +81,7 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_mfma_kernel(
   float mx[NP], my[NP], mw[NP];
   float v[8][NP * NCORN];
   float4 wv;
+  const int w_off = (tid >> 4) * Opad + (tid & 15) * 4;
 
   auto load_map = [&](int k) {
 #pragma unroll
@@ -105,11 +106,11 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_mfma_kernel(
 #pragma unroll
       for (int sp = 0; sp < NP; sp++)
 #pragma unroll
-        for (int i = 0; i < NCORN; i++) v[ch][sp * NCORN + i] = pl[taps[sp].off[i]];
+        for (int i = 0; i < NCORN; i++) v[ch][sp * NCORN + i] = load_at(pl, taps[sp].off[i]);
     }
     // weights of this chunk: 16 rows x 64 floats, one float4 per thread
-    const int cc = tid >> 4, o4 = (tid & 15) * 4;
-    wv = *reinterpret_cast<const float4 *>(wp + ((int64_t)k * Gpad + c * kGC + cc) * Opad + o0 + o4);
+    const float *wchunk = wp + ((int64_t)k * Gpad + c * kGC) * Opad + o0;  // uniform
+    wv = *reinterpret_cast<const float4 *>(wchunk + w_off);
   };
   auto stage = [&](int buf) {
 #pragma unroll
@@ -149,14 +150,19 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_mfma_kernel(
       }
     }
     if (it + 1 < iters) issue(k, c);
+    // fetch every operand of the chunk first, then issue the MFMAs back to back
+    float bv[kGC / 2], a0[kGC / 2], a1[kGC / 2];
 #pragma unroll
     for (int s = 0; s < kGC / 2; s++) {
       const int kk = 2 * s + lhi;
-      const float bv = S[buf][kk][wave * 32 + l31];
-      const float a0 = Wt[buf][kk][l31];
-      const float a1 = Wt[buf][kk][32 + l31];
-      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, bv, acc0, 0, 0, 0);
-      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, bv, acc1, 0, 0, 0);
+      bv[s] = S[buf][kk][wave * 32 + l31];
+      a0[s] = Wt[buf][kk][l31];
+      a1[s] = Wt[buf][kk][32 + l31];
+    }
+#pragma unroll
+    for (int s = 0; s < kGC / 2; s++) {
+      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[s], bv[s], acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[s], bv[s], acc1, 0, 0, 0);
     }
   }
 
@@ -220,7 +226,8 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_mfma_kernel(
   const int tw_mask = (1 << tw_shift) - 1, th = kTilePx >> tw_shift;
   const int N = MH * MW;
   const int64_t gplane = (int64_t)GH * GW;
-  const int p = tid & (kTilePx - 1), half = tid >> 7;
+  const int p = tid & (kTilePx - 1);
+  const int half = __builtin_amdgcn_readfirstlane(tid >> 7);  // wave-uniform: scalar addressing
   const int g_first = cg * (kWgCB * kGC);
 
   floatx4 acc[kWgKT][kWgCB];
@@ -288,7 +295,7 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_mfma_kernel(
 #pragma unroll
         for (int sp = 0; sp < NP; sp++)
 #pragma unroll
-          for (int i = 0; i < NCORN; i++) v[ch][sp * NCORN + i] = pl[taps[sp].off[i]];
+          for (int i = 0; i < NCORN; i++) v[ch][sp * NCORN + i] = load_at(pl, taps[sp].off[i]);
       }
     };
     auto stage = [&](int buf) {

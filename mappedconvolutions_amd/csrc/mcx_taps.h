@@ -10,11 +10,17 @@
 
 namespace mcx {
 
+// off[] are BYTE offsets of fp32 elements, unsigned, so that a load from a
+// wave-uniform plane pointer compiles to "scalar base + 32-bit vector offset".
 template <int NCORN>
 struct PairTap {
-  int off[NCORN];
+  unsigned off[NCORN];
   float wt[NCORN];
 };
+
+__device__ inline float load_at(const float *plane, unsigned byte_off) {
+  return *reinterpret_cast<const float *>(reinterpret_cast<const char *>(plane) + byte_off);
+}
 
 // NCORN == 1: nearest.  NCORN == 4: bilinear (wrap == false) or bispherical (wrap == true).
 template <int NCORN>
@@ -24,7 +30,7 @@ __device__ inline void resolve_pairs(float x, float y, int h, int w, bool wrap, 
     const int xi = to_int(round_half_away(x));
     const int yi = to_int(round_half_away(y));
     const bool ok = xi >= 0 && xi <= w - 1 && yi >= 0 && yi <= h - 1;
-    t.off[0] = ok ? yi * w + xi : 0;
+    t.off[0] = ok ? (unsigned)(yi * w + xi) * 4u : 0u;
     t.wt[0] = ok ? scale : 0.f;
   } else {
     const float x1f = floorf(x), y1f = floorf(y);
@@ -47,7 +53,7 @@ __device__ inline void resolve_pairs(float x, float y, int h, int w, bool wrap, 
     const float wv[4] = {A * B, A * C, D * B, D * C};
 #pragma unroll
     for (int i = 0; i < NCORN; i++) {
-      t.off[i] = ok[i] ? o[i] : 0;
+      t.off[i] = ok[i] ? (unsigned)o[i] * 4u : 0u;
       t.wt[i] = ok[i] ? wv[i] * scale : 0.f;
     }
   }
