@@ -229,6 +229,8 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_mfma_kernel(
   const int p = tid & (kTilePx - 1);
   const int half = __builtin_amdgcn_readfirstlane(tid >> 7);  // wave-uniform: scalar addressing
   const int g_first = cg * (kWgCB * kGC);
+  // 16-byte loads of the plain tile need every row segment 16-byte aligned
+  const bool vec_ok = (MW & 3) == 0 && (reinterpret_cast<uintptr_t>(plain) & 15) == 0;
 
   floatx4 acc[kWgKT][kWgCB];
 #pragma unroll
@@ -244,14 +246,27 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_mfma_kernel(
 
     __syncthreads();  // everyone is done with the previous tile's LDS contents
     {
-      const float *pb = plain + (int64_t)b * A * N;
-#pragma unroll 8
-      for (int r = 0; r < (kWgA * kTilePx) / kThreads; r++) {
-        const int e = tid + kThreads * r;
-        const int a = e >> 7, px = e & (kTilePx - 1);
-        const int i = i0 + (px >> tw_shift), j = j0 + (px & tw_mask);
-        const bool ok = (a0 + a) < A && i < MH && j < MW;
-        Pt[a][px] = ok ? pb[(int64_t)(a0 + a) * N + (int64_t)i * MW + j] : 0.f;
+      // Each thread stages 32 consecutive tile pixels of one plain channel: with
+      // either tile shape (4 x 32 or 1 x 128) they are contiguous in memory.
+      const int a = tid >> 2, px0 = (tid & 3) * 32;
+      const int si = i0 + (px0 >> tw_shift), sj = j0 + (px0 & tw_mask);
+      const bool row_ok = (a0 + a) < A && si < MH;
+      const float *prow = plain + ((int64_t)b * A + min(a0 + a, A - 1)) * N +
+                          (int64_t)min(si, MH - 1) * MW;
+      float4 *dstv = reinterpret_cast<float4 *>(&Pt[a][px0]);
+      if (vec_ok && row_ok && sj + 32 <= MW) {
+        const float4 *srcv = reinterpret_cast<const float4 *>(prow + sj);
+        float4 t[8];
+#pragma unroll
+        for (int r = 0; r < 8; r++) t[r] = srcv[r];
+#pragma unroll
+        for (int r = 0; r < 8; r++) dstv[r] = t[r];
+      } else {
+        float t[32];
+#pragma unroll
+        for (int r = 0; r < 32; r++) t[r] = prow[min(sj + r, MW - 1)];
+#pragma unroll
+        for (int r = 0; r < 32; r++) Pt[a][px0 + r] = (row_ok && sj + r < MW) ? t[r] : 0.f;
       }
     }
     __syncthreads();
@@ -393,8 +408,8 @@ __global__ void reduce_partials_kernel(const float *__restrict__ part, float *__
 // atomic per touched element and clears it.  Corners whose weight is exactly zero
 // (integer coordinates) are skipped.
 constexpr int kScDC = 16;        // destination channels per pass
-constexpr int kScWaveWin = 256;  // window slots per wave and destination channel
-constexpr int kScWinLd = 260;    // row stride: 4 rows apart = 16 banks apart
+constexpr int kScWaveWin = 192;  // window slots per wave and destination channel
+constexpr int kScWinLd = 196;    // row stride: 4 rows apart = 16 banks apart
 constexpr int kScSC = 64;        // source channels per register block
 
 // Repack W[s][d][k] -> Wq[k][dc][s][16]: per (tap, 16-channel block) a contiguous
@@ -424,15 +439,27 @@ __device__ inline int wave_max(int v) {
   return v;
 }
 
+// Column distance from a reference column on the circle of DW columns, in
+// [-DW/2, DW/2): both arguments are in [0, DW), so one conditional add/sub wraps.
+__device__ inline int circ_delta(int xx, int xref, int dw, int halfw) {
+  int d = xx - xref;
+  if (d >= dw - halfw) d -= dw;
+  if (d < -halfw) d += dw;
+  return d;
+}
+
+constexpr int kScMaxTaps = 64;  // taps whose race-check flags fit the LDS table
+
 template <int NCORN, int NP>
-__global__ __launch_bounds__(kThreads, 2) void product_scatter_mfma_kernel(
+__global__ __launch_bounds__(kThreads, 3) void product_scatter_mfma_kernel(
     const float *__restrict__ src, const float *__restrict__ map, const float *__restrict__ iw,
     const float *__restrict__ wq, float *__restrict__ dst, int S, int D, int Spad, int DH, int DW,
     int MH, int MW, int K, int weighted, int wrap, int tiles_x, int tiles_per_img, int tw_shift) {
   __shared__ __attribute__((aligned(16))) float Win[kThreads / 64][kScDC][kScWinLd];
-  __shared__ __attribute__((aligned(16))) float Wt[2][kScSC][kScDC];
+  __shared__ unsigned Flags[kThreads / 64][kScMaxTaps];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l15 = lane & 15, lq = lane >> 4;
   const int tile = xcd_contiguous_tile(blockIdx.x, gridDim.x);
   const int b = tile / tiles_per_img;
@@ -446,48 +473,98 @@ __global__ __launch_bounds__(kThreads, 2) void product_scatter_mfma_kernel(
   const int schunks = Spad / kScSC;
   const int halfw = DW >> 1;
   float(*win)[kScWinLd] = Win[wave];
+  unsigned *flags = Flags[wave];
 
-  // ---- per-wave pre-pass: bounding box of the destination corners of the wave's
-  // 32 pixels (corners that are valid and carry a non-zero weight) ---------------
-  int xref, ymin, ymax, dmin, dmax;
+  // ---- this lane's two pixels (MFMA column l15 of column blocks 0 and 1) -------
+  int64_t npx[2];
+  bool live[2];
+#pragma unroll
+  for (int nb = 0; nb < 2; nb++) {
+    const int px = wave * 32 + nb * 16 + l15;
+    const int pi = i0 + (px >> tw_shift), pj = j0 + (px & tw_mask);
+    live[nb] = pi < MH && pj < MW;
+    npx[nb] = live[nb] ? (int64_t)pi * MW + pj : 0;
+  }
+
+  // ---- per-wave pre-pass A: bounding box of the destination corners of the wave's
+  // 32 pixels (valid corners with a non-zero weight); the four 16-lane groups take
+  // every fourth tap ---------------------------------------------------------------
+  int xref;
   {
     const int px0 = wave * 32;
     const int ri = min(i0 + (px0 >> tw_shift), MH - 1), rj = min(j0 + (px0 & tw_mask), MW - 1);
     xref = wrap_index(to_int(floorf(map[((int64_t)ri * MW + rj) * K * NP * 2])), DW);
-    const int px = px0 + (lane & 31);
-    const int pi = i0 + (px >> tw_shift), pj = j0 + (px & tw_mask);
-    int vymin = 0x7fffffff, vymax = -0x7fffffff, vdmin = 0x7fffffff, vdmax = -0x7fffffff;
-    if (pi < MH && pj < MW) {
-      const int64_t n = (int64_t)pi * MW + pj;
-      for (int k = lane >> 5; k < K; k += 2) {
+  }
+  int ymin = 0x7fffffff, ymax = -0x7fffffff, dmin = 0x7fffffff, dmax = -0x7fffffff;
+  for (int k = lq; k < K; k += 4) {
 #pragma unroll
-        for (int sp = 0; sp < NP; sp++) {
-          const int64_t e = (n * K + k) * NP + sp;
-          CoordTap<NCORN> t;
-          resolve_coords<NCORN>(map[e * 2], map[e * 2 + 1], DH, DW, wrap != 0,
-                                weighted ? iw[e] : 1.f, t);
+    for (int nb = 0; nb < 2; nb++) {
+      if (!live[nb]) continue;
 #pragma unroll
-          for (int c = 0; c < NCORN; c++) {
-            if ((t.ok & (1u << c)) && t.wt[c] != 0.f) {
-              const int dx = wrap_index(t.xx[c] - xref + halfw, DW) - halfw;
-              vymin = min(vymin, t.yy[c]);
-              vymax = max(vymax, t.yy[c]);
-              vdmin = min(vdmin, dx);
-              vdmax = max(vdmax, dx);
-            }
+      for (int sp = 0; sp < NP; sp++) {
+        const int64_t e = (npx[nb] * K + k) * NP + sp;
+        CoordTap<NCORN> t;
+        resolve_coords<NCORN>(map[e * 2], map[e * 2 + 1], DH, DW, wrap != 0,
+                              weighted ? iw[e] : 1.f, t);
+#pragma unroll
+        for (int c = 0; c < NCORN; c++) {
+          if ((t.ok & (1u << c)) && t.wt[c] != 0.f) {
+            const int dx = circ_delta(t.xx[c], xref, DW, halfw);
+            ymin = min(ymin, t.yy[c]);
+            ymax = max(ymax, t.yy[c]);
+            dmin = min(dmin, dx);
+            dmax = max(dmax, dx);
           }
         }
       }
     }
-    ymin = wave_min(vymin);
-    ymax = wave_max(vymax);
-    dmin = wave_min(vdmin);
-    dmax = wave_max(vdmax);
   }
+  ymin = wave_min(ymin);
+  ymax = wave_max(ymax);
+  dmin = wave_min(dmin);
+  dmax = wave_max(dmax);
   const bool any_target = ymin <= ymax;
   const int ww = any_target ? dmax - dmin + 1 : 1, wh = any_target ? ymax - ymin + 1 : 1;
   const int wsz = ww * wh;
-  const bool use_lds = any_target && wsz <= kScWaveWin;
+  const bool use_lds = any_target && wsz <= kScWaveWin && K <= kScMaxTaps;
+
+  // ---- pre-pass B: for every (tap, pixel block, point, corner) decide whether the
+  // plain read-modify-write into the window is race-free: the valid lanes of the
+  // 16-lane group must form one run with strictly increasing slots (the four groups
+  // of an MFMA result hold different channels, i.e. different window rows) ----------
+  if (use_lds) {
+    for (int k0 = 0; k0 < K; k0 += 4) {  // uniform trip count: the ballots need every lane
+      const int k = k0 + lq;
+      unsigned fl = 0;
+#pragma unroll
+      for (int nb = 0; nb < 2; nb++) {
+#pragma unroll
+        for (int sp = 0; sp < NP; sp++) {
+          CoordTap<NCORN> t;
+          t.ok = 0;
+          if (k < K && live[nb]) {
+            const int64_t e = (npx[nb] * K + k) * NP + sp;
+            resolve_coords<NCORN>(map[e * 2], map[e * 2 + 1], DH, DW, wrap != 0,
+                                  weighted ? iw[e] : 1.f, t);
+          }
+#pragma unroll
+          for (int c = 0; c < NCORN; c++) {
+            const bool valid = (t.ok & (1u << c)) && t.wt[c] != 0.f;
+            const int slot =
+                valid ? (t.yy[c] - ymin) * ww + circ_delta(t.xx[c], xref, DW, halfw) - dmin : 0;
+            const int prev = __shfl_up(slot, 1, 16);
+            const int pvalid = __shfl_up((int)valid, 1, 16);
+            const bool clash = valid && l15 > 0 && pvalid && slot <= prev;
+            const unsigned m = (unsigned)((__ballot(valid) >> (16 * lq)) & 0xffffu);
+            const unsigned cl = (unsigned)((__ballot(clash) >> (16 * lq)) & 0xffffu);
+            const unsigned run = m ? (m >> __builtin_ctz(m)) : 0u;
+            if (cl != 0u || (run & (run + 1u)) != 0u) fl |= 1u << ((nb * NP + sp) * NCORN + c);
+          }
+        }
+      }
+      if (k < K && l15 == 0) flags[k] = fl;
+    }
+  }
 
   // global offsets of the window slots this lane flushes
   int goff[kScWaveWin / 64];
@@ -502,17 +579,8 @@ __global__ __launch_bounds__(kThreads, 2) void product_scatter_mfma_kernel(
     }
   }
   for (int e = lane; e < kScDC * kScWinLd; e += 64) (&win[0][0])[e] = 0.f;
+  __syncthreads();  // flags and cleared windows visible (the only workgroup barrier)
 
-  // ---- this lane's two pixels (MFMA column l15 of column blocks 0 and 1) -------
-  int64_t npx[2];
-  bool live[2];
-#pragma unroll
-  for (int nb = 0; nb < 2; nb++) {
-    const int px = wave * 32 + nb * 16 + l15;
-    const int pi = i0 + (px >> tw_shift), pj = j0 + (px & tw_mask);
-    live[nb] = pi < MH && pj < MW;
-    npx[nb] = live[nb] ? (int64_t)pi * MW + pj : 0;
-  }
   const float *src_b = src + (int64_t)b * S * N;
   float *dst_b = dst + (int64_t)b * D * dplane;
 
@@ -528,19 +596,21 @@ __global__ __launch_bounds__(kThreads, 2) void product_scatter_mfma_kernel(
   };
   if (schunks == 1) load_b(0);
 
-  const int units = dchunks * K * schunks;  // unit = (dc, k, sc), sc fastest
-  float4 wpre;
-  auto prefetch_w = [&](int dc, int k, int sc) {
-    wpre = reinterpret_cast<const float4 *>(
-        wq + (((int64_t)k * dchunks + dc) * Spad + sc * kScSC) * kScDC)[tid];
+  // MFMA A operands come straight from the packed weights (L1/L2 resident): lane
+  // (l15, lq) of step t needs Wq[k][dc][sc*64 + 4t + lq][l15].
+  const unsigned a_off = (unsigned)(lq * kScDC + l15) * 4u;
+  float acur[16], anext[16];
+  auto load_a = [&](int dc, int k, int sc, float *dstreg) {
+    const float *base = wq + (((int64_t)k * dchunks + dc) * Spad + sc * kScSC) * kScDC;  // uniform
+#pragma unroll
+    for (int t = 0; t < 16; t++) dstreg[t] = load_at(base + t * 4 * kScDC, a_off);
   };
-  prefetch_w(0, 0, 0);
+  load_a(0, 0, 0, acur);
 
+  const int units = dchunks * K * schunks;  // unit = (dc, k, sc), sc fastest
   int dc = 0, k = 0, sc = 0;
   floatx4 acc[2];
   for (int u = 0; u < units; ++u) {
-    const int buf = u & 1;
-    reinterpret_cast<float4 *>(&Wt[buf][0][0])[tid] = wpre;
     if (schunks > 1) load_b(sc);
     if (sc == 0) {
       acc[0] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -560,8 +630,7 @@ __global__ __launch_bounds__(kThreads, 2) void product_scatter_mfma_kernel(
           mw[nb][sp] = weighted ? iw[e] : 1.f;
         }
     }
-    __syncthreads();
-    // advance and prefetch the next unit's weights
+    // advance and put the next unit's weights in flight
     const int cdc = dc, ck = k;
     if (++sc == schunks) {
       sc = 0;
@@ -570,17 +639,19 @@ __global__ __launch_bounds__(kThreads, 2) void product_scatter_mfma_kernel(
         ++dc;
       }
     }
-    if (u + 1 < units) prefetch_w(dc, k, sc);
+    if (u + 1 < units) load_a(dc, k, sc, anext);
 
 #pragma unroll
     for (int t = 0; t < 16; t++) {
-      const float a = Wt[buf][4 * t + lq][l15];
-      acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, breg[0][t], acc[0], 0, 0, 0);
-      acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, breg[1][t], acc[1], 0, 0, 0);
+      acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(acur[t], breg[0][t], acc[0], 0, 0, 0);
+      acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(acur[t], breg[1][t], acc[1], 0, 0, 0);
     }
+#pragma unroll
+    for (int t = 0; t < 16; t++) acur[t] = anext[t];
 
     if (!last_sc) continue;
     // scatter col[d = cdc*16 + lq*4 + i][pixel nb] through tap ck
+    const unsigned fl = use_lds ? flags[ck] : 0xffffffffu;
 #pragma unroll
     for (int nb = 0; nb < 2; nb++) {
 #pragma unroll
@@ -590,22 +661,10 @@ __global__ __launch_bounds__(kThreads, 2) void product_scatter_mfma_kernel(
 #pragma unroll
         for (int c = 0; c < NCORN; c++) {
           const bool valid = live[nb] && (t.ok & (1u << c)) && t.wt[c] != 0.f;
-          bool direct = !use_lds;
-          int slot = 0;
-          if (use_lds) {
-            const int dx = wrap_index(t.xx[c] - xref + halfw, DW) - halfw;
-            slot = (t.yy[c] - ymin) * ww + (dx - dmin);
-            // race-free iff the valid lanes of each 16-lane group form one run with
-            // strictly increasing slots (the four groups hold different channels)
-            const int prev = __shfl_up(slot, 1, 16);
-            const int pvalid = __shfl_up((int)valid, 1, 16);
-            const bool clash = valid && l15 > 0 && pvalid && slot <= prev;
-            const unsigned m = (unsigned)(__ballot(valid) & 0xffffu);
-            const unsigned run = m ? (m >> __builtin_ctz(m)) : 0u;
-            direct = __ballot(clash) != 0 || (run & (run + 1u)) != 0u;
-          }
           if (!valid) continue;
-          if (!direct) {
+          if (!((fl >> ((nb * NP + sp) * NCORN + c)) & 1u)) {
+            const int slot =
+                (t.yy[c] - ymin) * ww + circ_delta(t.xx[c], xref, DW, halfw) - dmin;
 #pragma unroll
             for (int i = 0; i < 4; i++) win[lq * 4 + i][slot] += t.wt[c] * acc[nb][i];
           } else {
