@@ -408,8 +408,8 @@ __global__ void reduce_partials_kernel(const float *__restrict__ part, float *__
 // atomic per touched element and clears it.  Corners whose weight is exactly zero
 // (integer coordinates) are skipped.
 constexpr int kScDC = 16;        // destination channels per pass
-constexpr int kScWaveWin = 192;  // window slots per wave and destination channel
-constexpr int kScWinLd = 196;    // row stride: 4 rows apart = 16 banks apart
+constexpr int kScWaveWin = 160;  // window slots per wave
+constexpr int kScWinLd = 20;     // floats per slot: 16 channels + 4 of padding (bank spread)
 constexpr int kScSC = 64;        // source channels per register block
 
 // Repack W[s][d][k] -> Wq[k][dc][s][16]: per (tap, 16-channel block) a contiguous
@@ -455,7 +455,7 @@ __global__ __launch_bounds__(kThreads, 3) void product_scatter_mfma_kernel(
     const float *__restrict__ src, const float *__restrict__ map, const float *__restrict__ iw,
     const float *__restrict__ wq, float *__restrict__ dst, int S, int D, int Spad, int DH, int DW,
     int MH, int MW, int K, int weighted, int wrap, int tiles_x, int tiles_per_img, int tw_shift) {
-  __shared__ __attribute__((aligned(16))) float Win[kThreads / 64][kScDC][kScWinLd];
+  __shared__ __attribute__((aligned(16))) float Win[kThreads / 64][kScWaveWin][kScWinLd];
   __shared__ unsigned Flags[kThreads / 64][kScMaxTaps];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -472,7 +472,7 @@ __global__ __launch_bounds__(kThreads, 3) void product_scatter_mfma_kernel(
   const int dchunks = (D + kScDC - 1) / kScDC;
   const int schunks = Spad / kScSC;
   const int halfw = DW >> 1;
-  float(*win)[kScWinLd] = Win[wave];
+  float(*win)[kScWinLd] = Win[wave];  // [slot][channel]
   unsigned *flags = Flags[wave];
 
   // ---- this lane's two pixels (MFMA column l15 of column blocks 0 and 1) -------
@@ -567,9 +567,10 @@ __global__ __launch_bounds__(kThreads, 3) void product_scatter_mfma_kernel(
   }
 
   // global offsets of the window slots this lane flushes
-  int goff[kScWaveWin / 64];
+  constexpr int kFlushRounds = (kScWaveWin + 63) / 64;
+  int goff[kFlushRounds];
 #pragma unroll
-  for (int r = 0; r < kScWaveWin / 64; r++) {
+  for (int r = 0; r < kFlushRounds; r++) {
     const int slot = lane + r * 64;
     if (use_lds && slot < wsz) {
       const int wy = slot / ww, wx = slot - wy * ww;
@@ -578,7 +579,7 @@ __global__ __launch_bounds__(kThreads, 3) void product_scatter_mfma_kernel(
       goff[r] = -1;
     }
   }
-  for (int e = lane; e < kScDC * kScWinLd; e += 64) (&win[0][0])[e] = 0.f;
+  for (int e = lane; e < kScWaveWin * kScWinLd; e += 64) (&win[0][0])[e] = 0.f;
   __syncthreads();  // flags and cleared windows visible (the only workgroup barrier)
 
   const float *src_b = src + (int64_t)b * S * N;
@@ -665,8 +666,14 @@ __global__ __launch_bounds__(kThreads, 3) void product_scatter_mfma_kernel(
           if (!((fl >> ((nb * NP + sp) * NCORN + c)) & 1u)) {
             const int slot =
                 (t.yy[c] - ymin) * ww + circ_delta(t.xx[c], xref, DW, halfw) - dmin;
-#pragma unroll
-            for (int i = 0; i < 4; i++) win[lq * 4 + i][slot] += t.wt[c] * acc[nb][i];
+            // one 16-byte read-modify-write: the lane's four channels are adjacent
+            float4 *cell = reinterpret_cast<float4 *>(&win[slot][lq * 4]);
+            float4 cur = *cell;
+            cur.x += t.wt[c] * acc[nb][0];
+            cur.y += t.wt[c] * acc[nb][1];
+            cur.z += t.wt[c] * acc[nb][2];
+            cur.w += t.wt[c] * acc[nb][3];
+            *cell = cur;
           } else {
             const int off = t.yy[c] * DW + t.xx[c];
 #pragma unroll
@@ -681,15 +688,24 @@ __global__ __launch_bounds__(kThreads, 3) void product_scatter_mfma_kernel(
     // after the last tap of a destination-channel block: flush and clear the window
     if (use_lds && ck == K - 1) {
 #pragma unroll
-      for (int r = 0; r < kScWaveWin / 64; r++) {
+      for (int r = 0; r < kFlushRounds; r++) {
         if (goff[r] < 0) continue;
         const int slot = lane + r * 64;
+        float vals[kScDC];
+#pragma unroll
+        for (int q = 0; q < kScDC / 4; q++) {
+          float4 *cell = reinterpret_cast<float4 *>(&win[slot][q * 4]);
+          const float4 cur = *cell;
+          *cell = float4{0.f, 0.f, 0.f, 0.f};
+          vals[q * 4 + 0] = cur.x;
+          vals[q * 4 + 1] = cur.y;
+          vals[q * 4 + 2] = cur.z;
+          vals[q * 4 + 3] = cur.w;
+        }
 #pragma unroll
         for (int dl = 0; dl < kScDC; dl++) {
-          const float val = win[dl][slot];
           const int d = cdc * kScDC + dl;
-          if (val != 0.f && d < D) atomic_add(dst_b + (int64_t)d * dplane + goff[r], val);
-          win[dl][slot] = 0.f;
+          if (vals[dl] != 0.f && d < D) atomic_add(dst_b + (int64_t)d * dplane + goff[r], vals[dl]);
         }
       }
     }
