@@ -47,10 +47,10 @@ int mfma_f32_weight_grad(const float *plain, const float *gath, const float *map
                          hipStream_t s);
 
 bool mfma_f32_product_scatter_supported(int64_t P);
-size_t mfma_f32_scatter_weight_bytes(int64_t S, int64_t D, int64_t K);
+size_t mfma_f32_product_scatter_bytes(int64_t S, int64_t D, int64_t K, int64_t DH, int64_t DW);
 int mfma_f32_product_scatter(const float *src, const float *map, const float *iw, const float *w,
-                             float *dst, float *wq, int64_t B, int64_t S, int64_t D, int64_t DH,
-                             int64_t DW, int64_t MH, int64_t MW, int64_t K, int64_t P, int interp,
-                             hipStream_t s);
+                             const float *bias, float *dst, void *scratch, int64_t B, int64_t S,
+                             int64_t D, int64_t DH, int64_t DW, int64_t MH, int64_t MW, int64_t K,
+                             int64_t P, int interp, hipStream_t s);
 
 }  // namespace mcx

@@ -108,33 +108,37 @@ int weight_grad<float>(const float *plain, const float *gath, const float *map, 
 }
 
 // dst[b,d] += splat(sum_s W[s,d,k] * src[b,s,n], map[n,k]); n over MH x MW; dst pre-initialised.
-size_t product_scatter_ws(int dtype, int64_t S, int64_t D, int64_t K, int64_t P) {
+size_t product_scatter_ws(int dtype, int64_t S, int64_t D, int64_t K, int64_t P, int64_t DH,
+                          int64_t DW) {
   if (dtype == MCX_F32 && mfma_f32_product_scatter_supported(P))
-    return align256(mfma_f32_scatter_weight_bytes(S, D, K));
+    return align256(mfma_f32_product_scatter_bytes(S, D, K, DH, DW));
   return 0;
 }
 
+// `bias` (may be NULL) is the per-channel value dst was initialised with.
 template <typename T>
-int product_scatter(const T *src, const T *map, const T *iw, const T *w, T *dst, void *ws,
-                    size_t ws_bytes, int64_t B, int64_t S, int64_t D, int64_t DH, int64_t DW,
-                    int64_t MH, int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s) {
+int product_scatter(const T *src, const T *map, const T *iw, const T *w, const T *bias, T *dst,
+                    void *ws, size_t ws_bytes, int64_t B, int64_t S, int64_t D, int64_t DH,
+                    int64_t DW, int64_t MH, int64_t MW, int64_t K, int64_t P, int interp,
+                    hipStream_t s) {
   (void)ws;
   (void)ws_bytes;
+  (void)bias;
   return generic_product_scatter<T>(src, map, iw, w, dst, B, S, D, DH, DW, MH * MW, K, P, interp,
                                     s);
 }
 
 template <>
 int product_scatter<float>(const float *src, const float *map, const float *iw, const float *w,
-                           float *dst, void *ws, size_t ws_bytes, int64_t B, int64_t S, int64_t D,
-                           int64_t DH, int64_t DW, int64_t MH, int64_t MW, int64_t K, int64_t P,
-                           int interp, hipStream_t s) {
+                           const float *bias, float *dst, void *ws, size_t ws_bytes, int64_t B,
+                           int64_t S, int64_t D, int64_t DH, int64_t DW, int64_t MH, int64_t MW,
+                           int64_t K, int64_t P, int interp, hipStream_t s) {
   if (!mfma_f32_product_scatter_supported(P))
     return generic_product_scatter<float>(src, map, iw, w, dst, B, S, D, DH, DW, MH * MW, K, P,
                                           interp, s);
-  if (!ws || ws_bytes < product_scatter_ws(MCX_F32, S, D, K, P)) return MCX_E_WORKSPACE;
-  return mfma_f32_product_scatter(src, map, iw, w, dst, (float *)ws, B, S, D, DH, DW, MH, MW, K,
-                                  P, interp, s);
+  if (!ws || ws_bytes < product_scatter_ws(MCX_F32, S, D, K, P, DH, DW)) return MCX_E_WORKSPACE;
+  return mfma_f32_product_scatter(src, map, iw, w, bias, dst, ws, B, S, D, DH, DW, MH, MW, K, P,
+                                  interp, s);
 }
 
 // gb[c] = sum over (b, n) of gy[b,c,n]; uses the scratch when it is large enough.
@@ -165,8 +169,8 @@ int conv_backward_t(const void *gy, const void *map, const void *iw, const void 
   if (gx) {
     if ((rc = fill_zero<T>((T *)gx, d.B * d.Ci * d.IH * d.IW, s))) return rc;
     if ((rc = product_scatter<T>((const T *)gy, (const T *)map, (const T *)iw, (const T *)w,
-                                 (T *)gx, ws, ws_bytes, d.B, d.Co, d.Ci, d.IH, d.IW, d.OH, d.OW,
-                                 d.K, d.P, interp, s)))
+                                 (const T *)nullptr, (T *)gx, ws, ws_bytes, d.B, d.Co, d.Ci, d.IH,
+                                 d.IW, d.OH, d.OW, d.K, d.P, interp, s)))
       return rc;
   }
   if (gw) {
@@ -185,9 +189,9 @@ int tconv_forward_t(const void *x, const void *map, const void *iw, const void *
                     int interp, hipStream_t s) {
   int rc = fill_bias<T>((T *)y, (const T *)bias, d.B, d.Co, d.OH * d.OW, s);
   if (rc) return rc;
-  return product_scatter<T>((const T *)x, (const T *)map, (const T *)iw, (const T *)w, (T *)y, ws,
-                            ws_bytes, d.B, d.Ci, d.Co, d.OH, d.OW, d.IH, d.IW, d.K, d.P, interp,
-                            s);
+  return product_scatter<T>((const T *)x, (const T *)map, (const T *)iw, (const T *)w,
+                            (const T *)bias, (T *)y, ws, ws_bytes, d.B, d.Ci, d.Co, d.OH, d.OW,
+                            d.IH, d.IW, d.K, d.P, interp, s);
 }
 
 template <typename T>
@@ -240,13 +244,13 @@ extern "C" int mcx_conv_forward(const void *x, const void *map, const void *iw, 
   }
 }
 
-extern "C" size_t mcx_conv_backward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t,
-                                              int64_t, int64_t OH, int64_t OW, int64_t K,
+extern "C" size_t mcx_conv_backward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t IH,
+                                              int64_t IW, int64_t OH, int64_t OW, int64_t K,
                                               int64_t P, int dtype) {
   // the gradients run one after the other on the stream and share the scratch
   const size_t elem = dtype == MCX_F64 ? 8 : 4;
   return std::max({weight_grad_ws(dtype, B, Co, Ci, OH, OW, K, P),
-                   product_scatter_ws(dtype, Co, Ci, K, P),
+                   product_scatter_ws(dtype, Co, Ci, K, P, IH, IW),
                    align256(channel_sum_scratch_bytes(B, Co, OH * OW, elem))});
 }
 
@@ -272,8 +276,9 @@ extern "C" int mcx_conv_backward(const void *gy, const void *map, const void *iw
 }
 
 extern "C" size_t mcx_tconv_forward_workspace(int64_t, int64_t Ci, int64_t Co, int64_t, int64_t,
-                                              int64_t, int64_t, int64_t K, int64_t P, int dtype) {
-  return product_scatter_ws(dtype, Ci, Co, K, P);
+                                              int64_t OH, int64_t OW, int64_t K, int64_t P,
+                                              int dtype) {
+  return product_scatter_ws(dtype, Ci, Co, K, P, OH, OW);
 }
 
 extern "C" int mcx_tconv_forward(const void *x, const void *map, const void *iw, const void *w,

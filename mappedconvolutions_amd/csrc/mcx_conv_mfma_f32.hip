@@ -34,15 +34,17 @@ __device__ inline int xcd_contiguous_tile(int wg, int total) {
 
 // Repack W[o][g][k] -> Wp[k][g][o] with g padded to 16 and o padded to 64 (zeros),
 // so that a reduction chunk's weights are 16 rows of contiguous floats.
+// `transposed` reads W[g][o][k] instead (weights stored source-channel major).
 __global__ void pack_weights_kernel(const float *__restrict__ w, float *__restrict__ wp, int O,
-                                    int G, int K, int Opad, int Gpad) {
+                                    int G, int K, int Opad, int Gpad, int transposed) {
   const int64_t total = (int64_t)K * Gpad * Opad;
   for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total;
        e += (int64_t)gridDim.x * blockDim.x) {
     const int o = (int)(e % Opad);
     const int g = (int)((e / Opad) % Gpad);
     const int k = (int)(e / ((int64_t)Opad * Gpad));
-    wp[e] = (o < O && g < G) ? w[((int64_t)o * G + g) * K + k] : 0.f;
+    const int64_t wi = transposed ? ((int64_t)g * O + o) * K + k : ((int64_t)o * G + g) * K + k;
+    wp[e] = (o < O && g < G) ? w[wi] : 0.f;
   }
 }
 
@@ -51,8 +53,10 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_mfma_kernel(
     const float *__restrict__ src, const float *__restrict__ map, const float *__restrict__ iw,
     const float *__restrict__ wp, const float *__restrict__ bias, float *__restrict__ y, int G,
     int O, int Opad, int Gpad, int SH, int SW, int OH, int OW, int K, int weighted, int wrap,
-    int tiles_x, int tiles_per_img, int tw_shift) {
+    int tiles_x, int tiles_per_img, int tw_shift, const int *__restrict__ gate, int run_if_zero) {
   __shared__ __attribute__((aligned(16))) float S[2][kGC][kTilePx];
+  if (gate && ((*gate == 0) != (run_if_zero != 0))) return;  // device-side path selection
+
   __shared__ __attribute__((aligned(16))) float Wt[2][kGC][kWtLd];
 
   const int tid = threadIdx.x;
@@ -389,28 +393,35 @@ __global__ void reduce_partials_kernel(const float *__restrict__ part, float *__
 // ---------------------------------------------------------------------------------
 // product_scatter: dst[b,d] += splat(sum_s W[s,d,k] * src[b,s,n], map[n,k])
 // (convolution backward-input: s = Co, d = Ci; transposed forward: s = Ci, d = Co).
-// A workgroup owns a 2-D tile of 128 map pixels, one tile row of 32 per wave.  Each
-// wave keeps the source values of its 32 pixels (64 source channels) in registers
-// as MFMA B operands for the whole tile.  Destination channels are processed 16 at
-// a time: per tap the 64x16 weight slice is staged in LDS and
-// v_mfma_f32_16x16x4_f32 yields col[d][pixel] in registers.
+// One wavefront (= one workgroup) owns a row segment of 32 map pixels.  It keeps
+// the source values of its pixels (64 source channels) in registers as MFMA B
+// operands.  Destination channels are processed 16 at a time: per tap the 64x16
+// weight slice is read straight from the packed weights (L1/L2 resident) as A
+// operands and v_mfma_f32_16x16x4_f32 yields col[d][pixel] in registers.
 //
-// Scatter with LDS pre-reduction.  LDS float atomics retire about one lane every
-// few cycles on this part, so the window is accumulated WITHOUT atomics: every wave
-// owns a private LDS window covering the bounding box of its own pixels' destination
-// corners (rows x a circular interval of columns, found in a per-wave pre-pass over
-// the map), and adds into it with plain read-modify-write.  That is race-free when
-// the 16 lanes of one instruction hit 16 different slots, which holds whenever the
-// slots grow strictly along the pixel row; the kernel checks exactly that per
-// instruction (one cross-lane shift and a ballot) and sends the rare instruction
-// that fails the check, and waves whose box does not fit, to global atomics.  After
-// the K taps of a 16-channel block each wave flushes its window with one global
-// atomic per touched element and clears it.  Corners whose weight is exactly zero
-// (integer coordinates) are skipped.
+// Scatter with LDS pre-reduction.  MFMA and ordinary vector instructions do not
+// overlap on a SIMD here, and LDS float atomics retire about one lane every few
+// cycles, so the scatter is built to need few instructions and no atomics:
+//   * a pre-pass over the wave's map entries finds the bounding box of its
+//     destination corners (rows x a circular interval of columns) - the wave's
+//     private LDS window - and resolves every (pixel, tap, corner) ONCE into a
+//     window slot (one byte) and a weight, cached in LDS for all channel blocks;
+//   * the window is updated with plain 16-byte read-modify-writes (a lane's four
+//     channels of one slot are adjacent).  That is race-free when the 16 lanes of an
+//     instruction hit 16 different slots, which holds whenever the slots grow
+//     strictly along the pixel row; the pre-pass checks exactly that per (tap,
+//     corner) and marks the rare ones that fail, which go to global atomics, as do
+//     waves whose box does not fit the window;
+//   * after the taps of a group the window is flushed with one global atomic per
+//     touched element (consecutive lanes, consecutive addresses) and cleared.
+// Corners whose weight is exactly zero (integer coordinates) are skipped.
 constexpr int kScDC = 16;        // destination channels per pass
-constexpr int kScWaveWin = 160;  // window slots per wave
+constexpr int kScWaveWin = 160;  // window slots of a wave
 constexpr int kScWinLd = 20;     // floats per slot: 16 channels + 4 of padding (bank spread)
 constexpr int kScSC = 64;        // source channels per register block
+constexpr int kScPx = 32;        // pixels per wave
+constexpr int kScEntries = 40;   // cached (tap, point, corner) entries per pixel
+constexpr int kScThreads = 64;
 
 // Repack W[s][d][k] -> Wq[k][dc][s][16]: per (tap, 16-channel block) a contiguous
 // [Spad x 16] slice; s padded to 64, d padded to 16, zeros in the padding.
@@ -448,53 +459,48 @@ __device__ inline int circ_delta(int xx, int xref, int dw, int halfw) {
   return d;
 }
 
-constexpr int kScMaxTaps = 64;  // taps whose race-check flags fit the LDS table
-
 template <int NCORN, int NP>
-__global__ __launch_bounds__(kThreads, 3) void product_scatter_mfma_kernel(
+__global__ __launch_bounds__(kScThreads, 2) void product_scatter_mfma_kernel(
     const float *__restrict__ src, const float *__restrict__ map, const float *__restrict__ iw,
     const float *__restrict__ wq, float *__restrict__ dst, int S, int D, int Spad, int DH, int DW,
-    int MH, int MW, int K, int weighted, int wrap, int tiles_x, int tiles_per_img, int tw_shift) {
-  __shared__ __attribute__((aligned(16))) float Win[kThreads / 64][kScWaveWin][kScWinLd];
-  __shared__ unsigned Flags[kThreads / 64][kScMaxTaps];
+    int MH, int MW, int K, int weighted, int wrap, int tiles_x, int tiles_per_img,
+    const int *__restrict__ gate, int run_if_zero) {
+  if (gate && ((*gate == 0) != (run_if_zero != 0))) return;  // device-side path selection
+  constexpr int NE = NP * NCORN;           // cache entries per (pixel, tap)
+  constexpr int TG = kScEntries / NE;      // taps per group (their entries fit the cache)
+  static_assert(TG >= 1, "entry cache too small");
+  __shared__ __attribute__((aligned(16))) float win[kScWaveWin][kScWinLd];  // [slot][channel]
+  __shared__ float c_wt[TG * NE][kScPx];          // cached corner weights
+  __shared__ unsigned char c_slot[TG * NE][kScPx];  // cached window slots, 255 = not cached
+  __shared__ unsigned c_flag[TG][2];              // per tap: "any lane valid" / "needs atomics" bits
 
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = threadIdx.x;
   const int l15 = lane & 15, lq = lane >> 4;
   const int tile = xcd_contiguous_tile(blockIdx.x, gridDim.x);
   const int b = tile / tiles_per_img;
   const int t_in = tile - b * tiles_per_img;
-  const int tile_y = t_in / tiles_x, tile_x = t_in - tile_y * tiles_x;
-  const int tw_mask = (1 << tw_shift) - 1, th = kTilePx >> tw_shift;
-  const int i0 = tile_y * th, j0 = tile_x << tw_shift;
+  const int pi = t_in / tiles_x, j0 = (t_in - pi * tiles_x) * kScPx;
   const int N = MH * MW;
   const int64_t dplane = (int64_t)DH * DW;
   const int dchunks = (D + kScDC - 1) / kScDC;
   const int schunks = Spad / kScSC;
   const int halfw = DW >> 1;
-  float(*win)[kScWinLd] = Win[wave];  // [slot][channel]
-  unsigned *flags = Flags[wave];
 
   // ---- this lane's two pixels (MFMA column l15 of column blocks 0 and 1) -------
   int64_t npx[2];
   bool live[2];
 #pragma unroll
   for (int nb = 0; nb < 2; nb++) {
-    const int px = wave * 32 + nb * 16 + l15;
-    const int pi = i0 + (px >> tw_shift), pj = j0 + (px & tw_mask);
-    live[nb] = pi < MH && pj < MW;
-    npx[nb] = live[nb] ? (int64_t)pi * MW + pj : 0;
+    const int pj = j0 + nb * 16 + l15;
+    live[nb] = pj < MW;
+    npx[nb] = (int64_t)pi * MW + (live[nb] ? pj : j0);
   }
 
-  // ---- per-wave pre-pass A: bounding box of the destination corners of the wave's
-  // 32 pixels (valid corners with a non-zero weight); the four 16-lane groups take
-  // every fourth tap ---------------------------------------------------------------
-  int xref;
-  {
-    const int px0 = wave * 32;
-    const int ri = min(i0 + (px0 >> tw_shift), MH - 1), rj = min(j0 + (px0 & tw_mask), MW - 1);
-    xref = wrap_index(to_int(floorf(map[((int64_t)ri * MW + rj) * K * NP * 2])), DW);
-  }
+  // ---- pre-pass A: bounding box of the destination corners of the wave's pixels
+  // (valid corners with a non-zero weight); the four 16-lane groups take every
+  // fourth tap ------------------------------------------------------------------
+  const int xref =
+      wrap_index(to_int(floorf(map[((int64_t)pi * MW + j0) * K * NP * 2])), DW);
   int ymin = 0x7fffffff, ymax = -0x7fffffff, dmin = 0x7fffffff, dmax = -0x7fffffff;
   for (int k = lq; k < K; k += 4) {
 #pragma unroll
@@ -523,48 +529,10 @@ __global__ __launch_bounds__(kThreads, 3) void product_scatter_mfma_kernel(
   ymax = wave_max(ymax);
   dmin = wave_min(dmin);
   dmax = wave_max(dmax);
-  const bool any_target = ymin <= ymax;
-  const int ww = any_target ? dmax - dmin + 1 : 1, wh = any_target ? ymax - ymin + 1 : 1;
+  if (ymin > ymax) return;  // nothing of this wave lands inside the destination
+  const int ww = dmax - dmin + 1, wh = ymax - ymin + 1;
   const int wsz = ww * wh;
-  const bool use_lds = any_target && wsz <= kScWaveWin && K <= kScMaxTaps;
-
-  // ---- pre-pass B: for every (tap, pixel block, point, corner) decide whether the
-  // plain read-modify-write into the window is race-free: the valid lanes of the
-  // 16-lane group must form one run with strictly increasing slots (the four groups
-  // of an MFMA result hold different channels, i.e. different window rows) ----------
-  if (use_lds) {
-    for (int k0 = 0; k0 < K; k0 += 4) {  // uniform trip count: the ballots need every lane
-      const int k = k0 + lq;
-      unsigned fl = 0;
-#pragma unroll
-      for (int nb = 0; nb < 2; nb++) {
-#pragma unroll
-        for (int sp = 0; sp < NP; sp++) {
-          CoordTap<NCORN> t;
-          t.ok = 0;
-          if (k < K && live[nb]) {
-            const int64_t e = (npx[nb] * K + k) * NP + sp;
-            resolve_coords<NCORN>(map[e * 2], map[e * 2 + 1], DH, DW, wrap != 0,
-                                  weighted ? iw[e] : 1.f, t);
-          }
-#pragma unroll
-          for (int c = 0; c < NCORN; c++) {
-            const bool valid = (t.ok & (1u << c)) && t.wt[c] != 0.f;
-            const int slot =
-                valid ? (t.yy[c] - ymin) * ww + circ_delta(t.xx[c], xref, DW, halfw) - dmin : 0;
-            const int prev = __shfl_up(slot, 1, 16);
-            const int pvalid = __shfl_up((int)valid, 1, 16);
-            const bool clash = valid && l15 > 0 && pvalid && slot <= prev;
-            const unsigned m = (unsigned)((__ballot(valid) >> (16 * lq)) & 0xffffu);
-            const unsigned cl = (unsigned)((__ballot(clash) >> (16 * lq)) & 0xffffu);
-            const unsigned run = m ? (m >> __builtin_ctz(m)) : 0u;
-            if (cl != 0u || (run & (run + 1u)) != 0u) fl |= 1u << ((nb * NP + sp) * NCORN + c);
-          }
-        }
-      }
-      if (k < K && l15 == 0) flags[k] = fl;
-    }
-  }
+  const bool use_lds = wsz <= kScWaveWin;
 
   // global offsets of the window slots this lane flushes
   constexpr int kFlushRounds = (kScWaveWin + 63) / 64;
@@ -580,7 +548,6 @@ __global__ __launch_bounds__(kThreads, 3) void product_scatter_mfma_kernel(
     }
   }
   for (int e = lane; e < kScWaveWin * kScWinLd; e += 64) (&win[0][0])[e] = 0.f;
-  __syncthreads();  // flags and cleared windows visible (the only workgroup barrier)
 
   const float *src_b = src + (int64_t)b * S * N;
   float *dst_b = dst + (int64_t)b * D * dplane;
@@ -597,118 +564,166 @@ __global__ __launch_bounds__(kThreads, 3) void product_scatter_mfma_kernel(
   };
   if (schunks == 1) load_b(0);
 
-  // MFMA A operands come straight from the packed weights (L1/L2 resident): lane
-  // (l15, lq) of step t needs Wq[k][dc][sc*64 + 4t + lq][l15].
+  // MFMA A operands: lane (l15, lq) of step t needs Wq[k][dc][sc*64 + 4t + lq][l15].
   const unsigned a_off = (unsigned)(lq * kScDC + l15) * 4u;
-  float acur[16], anext[16];
-  auto load_a = [&](int dc, int k, int sc, float *dstreg) {
+  auto load_a = [&](int dc, int k, int sc, float *reg) {
     const float *base = wq + (((int64_t)k * dchunks + dc) * Spad + sc * kScSC) * kScDC;  // uniform
 #pragma unroll
-    for (int t = 0; t < 16; t++) dstreg[t] = load_at(base + t * 4 * kScDC, a_off);
+    for (int t = 0; t < 16; t++) reg[t] = load_at(base + t * 4 * kScDC, a_off);
   };
-  load_a(0, 0, 0, acur);
 
-  const int units = dchunks * K * schunks;  // unit = (dc, k, sc), sc fastest
-  int dc = 0, k = 0, sc = 0;
-  floatx4 acc[2];
-  for (int u = 0; u < units; ++u) {
-    if (schunks > 1) load_b(sc);
-    if (sc == 0) {
-      acc[0] = floatx4{0.f, 0.f, 0.f, 0.f};
-      acc[1] = floatx4{0.f, 0.f, 0.f, 0.f};
-    }
-    // map entries of this tap for the lane's two pixels (consumed after the MFMAs)
-    float mx[2][NP], my[2][NP], mw[2][NP];
-    const bool last_sc = sc + 1 == schunks;
-    if (last_sc) {
+  for (int k0 = 0; k0 < K; k0 += TG) {  // tap groups
+    const int kn = min(TG, K - k0);
+    // ---- pre-pass B: resolve the group's taps once into the LDS cache and decide,
+    // per (tap, pixel block, point, corner), whether the plain window update is
+    // race-free (valid lanes of the 16-lane group form one run of strictly
+    // increasing slots; the four groups of an MFMA result hold different channels)
+    for (int kb = 0; kb < kn; kb += 4) {  // uniform trip count: the ballots need every lane
+      const int kl = kb + lq;  // tap within the group handled by this 16-lane group
+      unsigned any_bits = 0, atom_bits = 0;
 #pragma unroll
-      for (int nb = 0; nb < 2; nb++)
+      for (int nb = 0; nb < 2; nb++) {
 #pragma unroll
         for (int sp = 0; sp < NP; sp++) {
-          const int64_t e = (npx[nb] * K + k) * NP + sp;
-          mx[nb][sp] = map[e * 2];
-          my[nb][sp] = map[e * 2 + 1];
-          mw[nb][sp] = weighted ? iw[e] : 1.f;
-        }
-    }
-    // advance and put the next unit's weights in flight
-    const int cdc = dc, ck = k;
-    if (++sc == schunks) {
-      sc = 0;
-      if (++k == K) {
-        k = 0;
-        ++dc;
-      }
-    }
-    if (u + 1 < units) load_a(dc, k, sc, anext);
-
+          CoordTap<NCORN> t;
+          t.ok = 0;
+          if (kl < kn && live[nb]) {
+            const int64_t e = (npx[nb] * K + k0 + kl) * NP + sp;
+            resolve_coords<NCORN>(map[e * 2], map[e * 2 + 1], DH, DW, wrap != 0,
+                                  weighted ? iw[e] : 1.f, t);
+          }
 #pragma unroll
-    for (int t = 0; t < 16; t++) {
-      acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(acur[t], breg[0][t], acc[0], 0, 0, 0);
-      acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(acur[t], breg[1][t], acc[1], 0, 0, 0);
-    }
-#pragma unroll
-    for (int t = 0; t < 16; t++) acur[t] = anext[t];
-
-    if (!last_sc) continue;
-    // scatter col[d = cdc*16 + lq*4 + i][pixel nb] through tap ck
-    const unsigned fl = use_lds ? flags[ck] : 0xffffffffu;
-#pragma unroll
-    for (int nb = 0; nb < 2; nb++) {
-#pragma unroll
-      for (int sp = 0; sp < NP; sp++) {
-        CoordTap<NCORN> t;
-        resolve_coords<NCORN>(mx[nb][sp], my[nb][sp], DH, DW, wrap != 0, mw[nb][sp], t);
-#pragma unroll
-        for (int c = 0; c < NCORN; c++) {
-          const bool valid = live[nb] && (t.ok & (1u << c)) && t.wt[c] != 0.f;
-          if (!valid) continue;
-          if (!((fl >> ((nb * NP + sp) * NCORN + c)) & 1u)) {
+          for (int c = 0; c < NCORN; c++) {
+            const bool valid = (t.ok & (1u << c)) && t.wt[c] != 0.f;
             const int slot =
-                (t.yy[c] - ymin) * ww + circ_delta(t.xx[c], xref, DW, halfw) - dmin;
-            // one 16-byte read-modify-write: the lane's four channels are adjacent
-            float4 *cell = reinterpret_cast<float4 *>(&win[slot][lq * 4]);
-            float4 cur = *cell;
-            cur.x += t.wt[c] * acc[nb][0];
-            cur.y += t.wt[c] * acc[nb][1];
-            cur.z += t.wt[c] * acc[nb][2];
-            cur.w += t.wt[c] * acc[nb][3];
-            *cell = cur;
-          } else {
-            const int off = t.yy[c] * DW + t.xx[c];
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-              const int d = cdc * kScDC + lq * 4 + i;
-              if (d < D) atomic_add(dst_b + (int64_t)d * dplane + off, t.wt[c] * acc[nb][i]);
+                (valid && use_lds)
+                    ? (t.yy[c] - ymin) * ww + circ_delta(t.xx[c], xref, DW, halfw) - dmin
+                    : 0;
+            const int prev = __shfl_up(slot, 1, 16);
+            const int pvalid = __shfl_up((int)valid, 1, 16);
+            const bool clash = valid && l15 > 0 && pvalid && slot <= prev;
+            const unsigned m = (unsigned)((__ballot(valid) >> (16 * lq)) & 0xffffu);
+            const unsigned cl = (unsigned)((__ballot(clash) >> (16 * lq)) & 0xffffu);
+            const unsigned run = m ? (m >> __builtin_ctz(m)) : 0u;
+            const bool atomics = !use_lds || cl != 0u || (run & (run + 1u)) != 0u;
+            const int bit = (nb * NP + sp) * NCORN + c;
+            if (m) any_bits |= 1u << bit;
+            if (m && atomics) atom_bits |= 1u << bit;
+            if (kl < kn) {
+              const int row = kl * NE + sp * NCORN + c;
+              c_slot[row][nb * 16 + l15] = (unsigned char)((valid && !atomics) ? slot : 255);
+              c_wt[row][nb * 16 + l15] = valid ? t.wt[c] : 0.f;
             }
           }
         }
       }
-    }
-    // after the last tap of a destination-channel block: flush and clear the window
-    if (use_lds && ck == K - 1) {
-#pragma unroll
-      for (int r = 0; r < kFlushRounds; r++) {
-        if (goff[r] < 0) continue;
-        const int slot = lane + r * 64;
-        float vals[kScDC];
-#pragma unroll
-        for (int q = 0; q < kScDC / 4; q++) {
-          float4 *cell = reinterpret_cast<float4 *>(&win[slot][q * 4]);
-          const float4 cur = *cell;
-          *cell = float4{0.f, 0.f, 0.f, 0.f};
-          vals[q * 4 + 0] = cur.x;
-          vals[q * 4 + 1] = cur.y;
-          vals[q * 4 + 2] = cur.z;
-          vals[q * 4 + 3] = cur.w;
-        }
-#pragma unroll
-        for (int dl = 0; dl < kScDC; dl++) {
-          const int d = cdc * kScDC + dl;
-          if (vals[dl] != 0.f && d < D) atomic_add(dst_b + (int64_t)d * dplane + goff[r], vals[dl]);
-        }
+      if (kl < kn && l15 == 0) {
+        c_flag[kl][0] = any_bits;
+        c_flag[kl][1] = atom_bits;
       }
     }
+    __syncthreads();  // single-wave workgroup: orders the cache writes before its reads
+
+    // ---- main loop over (destination-channel block, tap of the group, source block)
+    const int units = dchunks * kn * schunks;
+    float areg[2][16];
+    load_a(0, k0, 0, areg[0]);
+    int dc = 0, kl = 0, sc = 0;
+    floatx4 acc[2];
+    auto unit = [&](int u, float *acur, float *anext) {
+      if (schunks > 1) load_b(sc);
+      if (sc == 0) {
+        acc[0] = floatx4{0.f, 0.f, 0.f, 0.f};
+        acc[1] = floatx4{0.f, 0.f, 0.f, 0.f};
+      }
+      const bool last_sc = sc + 1 == schunks;
+      const int cdc = dc, ckl = kl;
+      if (++sc == schunks) {
+        sc = 0;
+        if (++kl == kn) {
+          kl = 0;
+          ++dc;
+        }
+      }
+      if (u + 1 < units) load_a(dc, k0 + kl, sc, anext);  // next unit's weights in flight
+#pragma unroll
+      for (int t = 0; t < 16; t++) {
+        acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(acur[t], breg[0][t], acc[0], 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(acur[t], breg[1][t], acc[1], 0, 0, 0);
+      }
+      if (!last_sc) return;
+
+      // scatter col[d = cdc*16 + lq*4 + i][pixel nb] through tap k0 + ckl
+      const unsigned any_bits = c_flag[ckl][0], atom_bits = c_flag[ckl][1];
+#pragma unroll
+      for (int nb = 0; nb < 2; nb++) {
+#pragma unroll
+        for (int e = 0; e < NE; e++) {
+          const int bit = nb * NE + e;
+          if (!((any_bits >> bit) & 1u)) continue;  // uniform: no lane uses this corner
+          const int row = ckl * NE + e;
+          if (!((atom_bits >> bit) & 1u)) {
+            const unsigned slot = c_slot[row][nb * 16 + l15];
+            const float wt = c_wt[row][nb * 16 + l15];
+            if (slot != 255u) {
+              // one 16-byte read-modify-write: the lane's four channels are adjacent
+              float4 *cell = reinterpret_cast<float4 *>(&win[slot][lq * 4]);
+              float4 cur = *cell;
+              cur.x += wt * acc[nb][0];
+              cur.y += wt * acc[nb][1];
+              cur.z += wt * acc[nb][2];
+              cur.w += wt * acc[nb][3];
+              *cell = cur;
+            }
+          } else if (live[nb]) {
+            // rare: re-resolve this corner and use global atomics
+            const int sp = e / NCORN, c = e % NCORN;
+            const int64_t me = (npx[nb] * K + k0 + ckl) * NP + sp;
+            CoordTap<NCORN> t;
+            resolve_coords<NCORN>(map[me * 2], map[me * 2 + 1], DH, DW, wrap != 0,
+                                  weighted ? iw[me] : 1.f, t);
+            if ((t.ok & (1u << c)) && t.wt[c] != 0.f) {
+              const int off = t.yy[c] * DW + t.xx[c];
+#pragma unroll
+              for (int i = 0; i < 4; i++) {
+                const int d = cdc * kScDC + lq * 4 + i;
+                if (d < D) atomic_add(dst_b + (int64_t)d * dplane + off, t.wt[c] * acc[nb][i]);
+              }
+            }
+          }
+        }
+      }
+      // after the last tap of the group: flush and clear the window
+      if (use_lds && ckl == kn - 1) {
+#pragma unroll
+        for (int r = 0; r < kFlushRounds; r++) {
+          if (goff[r] < 0) continue;
+          const int slot = lane + r * 64;
+          float vals[kScDC];
+#pragma unroll
+          for (int q = 0; q < kScDC / 4; q++) {
+            float4 *cell = reinterpret_cast<float4 *>(&win[slot][q * 4]);
+            const float4 cur = *cell;
+            *cell = float4{0.f, 0.f, 0.f, 0.f};
+            vals[q * 4 + 0] = cur.x;
+            vals[q * 4 + 1] = cur.y;
+            vals[q * 4 + 2] = cur.z;
+            vals[q * 4 + 3] = cur.w;
+          }
+#pragma unroll
+          for (int dl = 0; dl < kScDC; dl++) {
+            const int d = cdc * kScDC + dl;
+            if (vals[dl] != 0.f && d < D)
+              atomic_add(dst_b + (int64_t)d * dplane + goff[r], vals[dl]);
+          }
+        }
+      }
+    };
+    for (int u = 0; u < units; u += 2) {  // ping-pong the A operand registers
+      unit(u, areg[0], areg[1]);
+      if (u + 1 < units) unit(u + 1, areg[1], areg[0]);
+    }
+    __syncthreads();  // cache reads done before the next group's pre-pass rewrites it
   }
 }
 
@@ -792,32 +807,154 @@ int mfma_f32_weight_grad(const float *plain, const float *gath, const float *map
 
 bool mfma_f32_product_scatter_supported(int64_t P) { return P >= 0 && P <= 4; }
 
-size_t mfma_f32_scatter_weight_bytes(int64_t S, int64_t D, int64_t K) {
-  return (size_t)(K * ((D + kScDC - 1) / kScDC) * round_up(S, kScSC) * kScDC) * sizeof(float);
+namespace {
+
+// ---------------------------------------------------------------------------------
+// Transposed map.  A scatter through map[n,k] is a gather through the transposed
+// map: destination pixel p receives wt * col[., k, n] from every (n, corner) that
+// lands on it.  When no (p, k) receives more than kTransSlots contributions (true for
+// resolution-preserving maps such as the latitude-distorted kernels), the product-
+// scatter equals a weighted, nearest-neighbour gather-product over the transposed
+// map, which needs no atomics at all and reuses the forward kernel.  This kernel
+// builds that map: tmap[p][k][slot] = (x, y) of source pixel n, tiw = corner weight;
+// a slot counter per (p, k) hands out slots and an overflow flag selects the scatter
+// kernel instead (both kernels are always enqueued; the flag gates them on the device).
+constexpr int kTransSlots = 4;
+
+template <int NCORN>
+__global__ void build_transposed_map_kernel(const float *__restrict__ map,
+                                            const float *__restrict__ iw, int *__restrict__ cnt,
+                                            float *__restrict__ tmap, float *__restrict__ tiw,
+                                            int *__restrict__ overflow, int np, int weighted,
+                                            int wrap, int DH, int DW, int MW, int K,
+                                            int64_t total) {
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= total) return;
+  const int k = (int)(e % K);
+  const int64_t n = e / K;
+  const float nx = (float)(n % MW), ny = (float)(n / MW);
+  for (int sp = 0; sp < np; sp++) {
+    const int64_t m = e * np + sp;
+    CoordTap<NCORN> t;
+    resolve_coords<NCORN>(map[m * 2], map[m * 2 + 1], DH, DW, wrap != 0, weighted ? iw[m] : 1.f,
+                          t);
+#pragma unroll
+    for (int c = 0; c < NCORN; c++) {
+      if (!(t.ok & (1u << c)) || t.wt[c] == 0.f) continue;
+      const int64_t cell = ((int64_t)t.yy[c] * DW + t.xx[c]) * K + k;
+      const int slot = atomicAdd(&cnt[cell], 1);
+      if (slot < kTransSlots) {
+        tmap[(cell * kTransSlots + slot) * 2] = nx;
+        tmap[(cell * kTransSlots + slot) * 2 + 1] = ny;
+        tiw[cell * kTransSlots + slot] = t.wt[c];
+      } else {
+        *overflow = 1;  // benign race: every writer stores the same value
+      }
+    }
+  }
 }
 
-// dst must already hold its initial value (zeros or the bias); wq: scratch of
-// mfma_f32_scatter_weight_bytes(S, D, K) bytes.
+struct ScatterScratch {
+  size_t wq, wpt, cnt, tmap, tiw, total;  // byte offsets; cnt holds the counters + the flag
+  bool transposed_path;
+};
+
+inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+ScatterScratch scatter_scratch(int64_t S, int64_t D, int64_t K, int64_t DH, int64_t DW) {
+  ScatterScratch sc;
+  size_t off = 0;
+  sc.wq = off;
+  off += align256((size_t)(K * ((D + kScDC - 1) / kScDC) * round_up(S, kScSC) * kScDC) * 4);
+  const int64_t cells = DH * DW * K;
+  sc.transposed_path = cells * kTransSlots * 2 <= 0x7fffffffLL;
+  sc.wpt = sc.cnt = sc.tmap = sc.tiw = off;
+  if (sc.transposed_path) {
+    sc.wpt = off;
+    off += align256((size_t)(K * round_up(S, kGC) * round_up(D, kOT)) * 4);
+    sc.cnt = off;
+    off += align256((size_t)(cells + 1) * 4);
+    sc.tmap = off;
+    off += align256((size_t)cells * kTransSlots * 2 * 4);
+    sc.tiw = off;
+    off += align256((size_t)cells * kTransSlots * 4);
+  }
+  sc.total = off;
+  return sc;
+}
+
+int launch_gather_product(const float *src, const float *map, const float *iw, const float *wp,
+                          const float *bias, float *y, int64_t B, int64_t G, int64_t O, int64_t SH,
+                          int64_t SW, int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
+                          const int *gate, int run_if_zero, hipStream_t s);
+
+}  // namespace
+
+size_t mfma_f32_product_scatter_bytes(int64_t S, int64_t D, int64_t K, int64_t DH, int64_t DW) {
+  return scatter_scratch(S, D, K, DH, DW).total;
+}
+
+// dst must already hold its initial value (zeros or bias[d] broadcast); `bias` is
+// that per-channel initial value or NULL for zeros.  scratch: device memory of
+// mfma_f32_product_scatter_bytes(...) bytes.
 int mfma_f32_product_scatter(const float *src, const float *map, const float *iw, const float *w,
-                             float *dst, float *wq, int64_t B, int64_t S, int64_t D, int64_t DH,
-                             int64_t DW, int64_t MH, int64_t MW, int64_t K, int64_t P, int interp,
-                             hipStream_t s) {
+                             const float *bias, float *dst, void *scratch, int64_t B, int64_t S,
+                             int64_t D, int64_t DH, int64_t DW, int64_t MH, int64_t MW, int64_t K,
+                             int64_t P, int interp, hipStream_t s) {
+  const ScatterScratch sc = scatter_scratch(S, D, K, DH, DW);
+  char *base = (char *)scratch;
+  float *wq = (float *)(base + sc.wq);
   const int Spad = (int)round_up(S, kScSC), dchunks = (int)((D + kScDC - 1) / kScDC);
   const int64_t packed = (int64_t)K * dchunks * Spad * kScDC;
+  const int mode = canonical_interp(interp);
+  const int weighted = P > 0 ? 1 : 0, wrap = mode == kInterpBispherical ? 1 : 0;
+  const int np = P > 0 ? (int)P : 1;
+  const int *gate = nullptr;
+
+  if (sc.transposed_path) {
+    // build the transposed map, then try the atomic-free gather form first
+    int *cnt = (int *)(base + sc.cnt);
+    float *tmap = (float *)(base + sc.tmap), *tiw = (float *)(base + sc.tiw);
+    float *wpt = (float *)(base + sc.wpt);
+    const int64_t cells = DH * DW * K;
+    int *flag = cnt + cells;
+    gate = flag;
+    int rc = fill_f32((float *)cnt, (int64_t)((sc.total - sc.cnt) / 4), 0.f, s);
+    if (rc) return rc;
+    const int64_t entries = MH * MW * K;
+    const unsigned blocks = (unsigned)((entries + 255) / 256);
+    if (mode == kInterpNearest)
+      hipLaunchKernelGGL(build_transposed_map_kernel<1>, dim3(blocks), dim3(256), 0, s, map, iw,
+                         cnt, tmap, tiw, flag, np, weighted, wrap, (int)DH, (int)DW, (int)MW,
+                         (int)K, entries);
+    else
+      hipLaunchKernelGGL(build_transposed_map_kernel<4>, dim3(blocks), dim3(256), 0, s, map, iw,
+                         cnt, tmap, tiw, flag, np, weighted, wrap, (int)DH, (int)DW, (int)MW,
+                         (int)K, entries);
+    MCX_HIP_CHECK_LAUNCH();
+    const int Opad = (int)round_up(D, kOT), Gpad = (int)round_up(S, kGC);
+    const int64_t pk = (int64_t)K * Gpad * Opad;
+    hipLaunchKernelGGL(pack_weights_kernel, dim3((unsigned)std::min<int64_t>((pk + 255) / 256, 4096)),
+                       dim3(256), 0, s, w, wpt, (int)D, (int)S, (int)K, Opad, Gpad, 1);
+    MCX_HIP_CHECK_LAUNCH();
+    rc = launch_gather_product(src, tmap, tiw, wpt, bias, dst, B, S, D, MH, MW, DH, DW, K,
+                               kTransSlots, kInterpNearest, gate, 1, s);
+    if (rc) return rc;
+  }
+
   hipLaunchKernelGGL(pack_scatter_weights_kernel,
                      dim3((unsigned)std::min<int64_t>((packed + 255) / 256, 4096)), dim3(256), 0, s,
                      w, wq, (int)S, (int)D, (int)K, Spad, dchunks);
   MCX_HIP_CHECK_LAUNCH();
-  const PixelTiling t = make_tiling(B, MH, MW);
-  if (t.total > 0x7fffffffLL) return MCX_E_SHAPE;
-  dim3 grid((unsigned)t.total);
-  const int mode = canonical_interp(interp);
-  const int weighted = P > 0 ? 1 : 0, wrap = mode == kInterpBispherical ? 1 : 0;
-  const int np = P > 0 ? (int)P : 1;
+  const int tiles_x = (int)((MW + kScPx - 1) / kScPx);
+  const int64_t tiles_per_img = (int64_t)tiles_x * MH;
+  const int64_t total = tiles_per_img * B;
+  if (total > 0x7fffffffLL) return MCX_E_SHAPE;
+  dim3 grid((unsigned)total);
 #define MCX_LAUNCH(NCORN, NP)                                                                    \
-  hipLaunchKernelGGL((product_scatter_mfma_kernel<NCORN, NP>), grid, dim3(kThreads), 0, s, src,  \
-                     map, iw, wq, dst, (int)S, (int)D, Spad, (int)DH, (int)DW, (int)MH, (int)MW, \
-                     (int)K, weighted, wrap, t.tiles_x, t.tiles_per_img, t.tw_shift)
+  hipLaunchKernelGGL((product_scatter_mfma_kernel<NCORN, NP>), grid, dim3(kScThreads), 0, s,     \
+                     src, map, iw, wq, dst, (int)S, (int)D, Spad, (int)DH, (int)DW, (int)MH,     \
+                     (int)MW, (int)K, weighted, wrap, tiles_x, (int)tiles_per_img, gate, 0)
   if (mode == kInterpNearest) {
     switch (np) {
       case 1: MCX_LAUNCH(1, 1); break;
@@ -847,16 +984,12 @@ size_t mfma_f32_packed_weight_bytes(int64_t O, int64_t G, int64_t K) {
 
 bool mfma_f32_gather_product_supported(int64_t P) { return P >= 0 && P <= 4; }
 
-// wp: scratch of mfma_f32_packed_weight_bytes(O, G, K) bytes.
-int mfma_f32_gather_product(const float *src, const float *map, const float *iw, const float *w,
-                            const float *bias, float *y, float *wp, int64_t B, int64_t G,
-                            int64_t O, int64_t SH, int64_t SW, int64_t OH, int64_t OW, int64_t K,
-                            int64_t P, int interp, hipStream_t s) {
+namespace {
+int launch_gather_product(const float *src, const float *map, const float *iw, const float *wp,
+                          const float *bias, float *y, int64_t B, int64_t G, int64_t O, int64_t SH,
+                          int64_t SW, int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
+                          const int *gate, int run_if_zero, hipStream_t s) {
   const int Opad = (int)round_up(O, kOT), Gpad = (int)round_up(G, kGC);
-  const int64_t packed = (int64_t)K * Gpad * Opad;
-  hipLaunchKernelGGL(pack_weights_kernel, dim3((unsigned)std::min<int64_t>((packed + 255) / 256, 4096)),
-                     dim3(256), 0, s, w, wp, (int)O, (int)G, (int)K, Opad, Gpad);
-  MCX_HIP_CHECK_LAUNCH();
   const PixelTiling t = make_tiling(B, OH, OW);
   const int tw_shift = t.tw_shift, tiles_x = t.tiles_x, tiles_per_img = t.tiles_per_img;
   const int64_t total = t.total;
@@ -868,7 +1001,8 @@ int mfma_f32_gather_product(const float *src, const float *map, const float *iw,
 #define MCX_LAUNCH(NCORN, NP)                                                                    \
   hipLaunchKernelGGL((gather_product_mfma_kernel<NCORN, NP>), grid, dim3(kThreads), 0, s, src,   \
                      map, iw, wp, bias, y, (int)G, (int)O, Opad, Gpad, (int)SH, (int)SW,         \
-                     (int)OH, (int)OW, (int)K, weighted, wrap, tiles_x, tiles_per_img, tw_shift)
+                     (int)OH, (int)OW, (int)K, weighted, wrap, tiles_x, tiles_per_img, tw_shift, \
+                     gate, run_if_zero)
   if (mode == kInterpNearest) {
     switch (np) {
       case 1: MCX_LAUNCH(1, 1); break;
@@ -887,6 +1021,21 @@ int mfma_f32_gather_product(const float *src, const float *map, const float *iw,
 #undef MCX_LAUNCH
   MCX_HIP_CHECK_LAUNCH();
   return 0;
+}
+}  // namespace
+
+// wp: scratch of mfma_f32_packed_weight_bytes(O, G, K) bytes.
+int mfma_f32_gather_product(const float *src, const float *map, const float *iw, const float *w,
+                            const float *bias, float *y, float *wp, int64_t B, int64_t G,
+                            int64_t O, int64_t SH, int64_t SW, int64_t OH, int64_t OW, int64_t K,
+                            int64_t P, int interp, hipStream_t s) {
+  const int Opad = (int)round_up(O, kOT), Gpad = (int)round_up(G, kGC);
+  const int64_t packed = (int64_t)K * Gpad * Opad;
+  hipLaunchKernelGGL(pack_weights_kernel, dim3((unsigned)std::min<int64_t>((packed + 255) / 256, 4096)),
+                     dim3(256), 0, s, w, wp, (int)O, (int)G, (int)K, Opad, Gpad, 0);
+  MCX_HIP_CHECK_LAUNCH();
+  return launch_gather_product(src, map, iw, wp, bias, y, B, G, O, SH, SW, OH, OW, K, P, interp,
+                               nullptr, 0, s);
 }
 
 }  // namespace mcx
