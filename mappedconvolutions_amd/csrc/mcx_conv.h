@@ -30,27 +30,31 @@ int channel_sum(const T *g, T *gb, T *scratch, int64_t B, int64_t C, int64_t N, 
 template <typename T>
 int fill_bias(T *y, const T *bias, int64_t B, int64_t C, int64_t N, hipStream_t s);
 
-// ---- fp32 matrix-core kernels (mcx_conv_mfma_f32.hip) -------------------------
-size_t mfma_f32_packed_weight_bytes(int64_t O, int64_t G, int64_t K);
-bool mfma_f32_gather_product_supported(int64_t P);
-int mfma_f32_gather_product(const float *src, const float *map, const float *iw, const float *w,
-                            const float *bias, float *y, float *wp, int64_t B, int64_t G,
-                            int64_t O, int64_t SH, int64_t SW, int64_t OH, int64_t OW, int64_t K,
-                            int64_t P, int interp, hipStream_t s);
-
-bool mfma_f32_weight_grad_supported(int64_t P);
-size_t mfma_f32_weight_grad_bytes(int64_t B, int64_t A, int64_t G, int64_t MH, int64_t MW,
-                                  int64_t K);
-int mfma_f32_weight_grad(const float *plain, const float *gath, const float *map, const float *iw,
-                         float *gw, float *part, int64_t B, int64_t A, int64_t G, int64_t GH,
-                         int64_t GW, int64_t MH, int64_t MW, int64_t K, int64_t P, int interp,
-                         hipStream_t s);
-
-bool mfma_f32_product_scatter_supported(int64_t P);
-size_t mfma_f32_product_scatter_bytes(int64_t S, int64_t D, int64_t K, int64_t DH, int64_t DW);
-int mfma_f32_product_scatter(const float *src, const float *map, const float *iw, const float *w,
-                             const float *bias, float *dst, void *scratch, int64_t B, int64_t S,
-                             int64_t D, int64_t DH, int64_t DW, int64_t MH, int64_t MW, int64_t K,
-                             int64_t P, int interp, hipStream_t s);
+// ---- matrix-core kernels (mcx_conv_mfma.hip), templated on the storage type TD
+// (float or bf16_t; arithmetic and accumulation are fp32 in both cases) -----------
+struct bf16_t;
+bool mfma_supported(int64_t P);
+size_t mfma_gather_product_bytes(int64_t O, int64_t G, int64_t K);
+template <typename TD>
+int mfma_gather_product(const TD *src, const float *map, const float *iw, const TD *w,
+                        const TD *bias, TD *y, void *scratch, int64_t B, int64_t G, int64_t O,
+                        int64_t SH, int64_t SW, int64_t OH, int64_t OW, int64_t K, int64_t P,
+                        int interp, hipStream_t s);
+size_t mfma_weight_grad_bytes(int64_t B, int64_t A, int64_t G, int64_t MH, int64_t MW, int64_t K);
+template <typename TD>
+int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const float *iw, TD *gw,
+                     void *scratch, int64_t B, int64_t A, int64_t G, int64_t GH, int64_t GW,
+                     int64_t MH, int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s);
+size_t mfma_product_scatter_bytes(int64_t B, int64_t S, int64_t D, int64_t K, int64_t DH,
+                                  int64_t DW, size_t elem);
+template <typename TD>
+int mfma_product_scatter(const TD *src, const float *map, const float *iw, const TD *w,
+                         const TD *bias, TD *dst, void *scratch, int64_t B, int64_t S, int64_t D,
+                         int64_t DH, int64_t DW, int64_t MH, int64_t MW, int64_t K, int64_t P,
+                         int interp, hipStream_t s);
+size_t mfma_bias_grad_bytes(int64_t B, int64_t C, int64_t N);
+template <typename TD>
+int mfma_bias_grad(const TD *g, TD *gb, void *scratch, int64_t B, int64_t C, int64_t N,
+                   hipStream_t s);
 
 }  // namespace mcx

@@ -1,12 +1,15 @@
 // extern "C" entry points of the mapped (transposed) convolution.  Validates the
 // arguments, then routes each of the three products (gather-product,
 // product-scatter, weight gradient; see mcx_conv_generic.hip for the roles) to the
-// matrix-core kernels when they cover the case and to the scalar kernels otherwise.
+// matrix-core kernels when they cover the case (fp32 and bf16 storage, at most 4
+// interpolation points per tap) and to the scalar kernels otherwise (fp64, or fp32
+// with more points).
 #include <algorithm>
 #include <initializer_list>
 
 #include "mcx.h"
 #include "mcx_conv.h"
+#include "mcx_taps.h"
 
 using namespace mcx;
 
@@ -34,7 +37,10 @@ int check_ptrs(const void *a, const void *map, const void *iw, const void *w, in
   return 0;
 }
 
-size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+size_t elem_size(int dtype) { return dtype == MCX_F64 ? 8 : dtype == MCX_BF16 ? 2 : 4; }
+bool use_mfma(int dtype, int64_t P) {
+  return (dtype == MCX_F32 || dtype == MCX_BF16) && mfma_supported(P);
+}
 
 template <typename T>
 int fill_zero(T *p, int64_t n, hipStream_t s);
@@ -43,179 +49,250 @@ int fill_zero<float>(float *p, int64_t n, hipStream_t s) { return fill_f32(p, n,
 template <>
 int fill_zero<double>(double *p, int64_t n, hipStream_t s) { return fill_f64(p, n, 0.0, s); }
 
-// ---- the three operators, typed ------------------------------------------------
-
-// y[b,o,n] = bias[o] + sum_{g,k} W[o,g,k] * sample(src[b,g], map[n,k]); n over MH x MW.
+// ---- scratch sizes of the three operators -------------------------------------------
 size_t gather_product_ws(int dtype, int64_t G, int64_t O, int64_t K, int64_t P) {
-  if (dtype == MCX_F32 && mfma_f32_gather_product_supported(P))
-    return align256(mfma_f32_packed_weight_bytes(O, G, K));
-  return 0;
+  return use_mfma(dtype, P) ? mfma_gather_product_bytes(O, G, K) : 0;
 }
-
-template <typename T>
-int gather_product(const T *src, const T *map, const T *iw, const T *w, const T *bias, T *y,
-                   void *ws, size_t ws_bytes, int64_t B, int64_t G, int64_t O, int64_t SH,
-                   int64_t SW, int64_t MH, int64_t MW, int64_t K, int64_t P, int interp,
-                   hipStream_t s) {
-  (void)ws;
-  (void)ws_bytes;
-  return generic_gather_product<T>(src, map, iw, w, bias, y, B, G, O, SH, SW, MH * MW, K, P,
-                                   interp, s);
-}
-
-template <>
-int gather_product<float>(const float *src, const float *map, const float *iw, const float *w,
-                          const float *bias, float *y, void *ws, size_t ws_bytes, int64_t B,
-                          int64_t G, int64_t O, int64_t SH, int64_t SW, int64_t MH, int64_t MW,
-                          int64_t K, int64_t P, int interp, hipStream_t s) {
-  if (!mfma_f32_gather_product_supported(P))
-    return generic_gather_product<float>(src, map, iw, w, bias, y, B, G, O, SH, SW, MH * MW, K, P,
-                                         interp, s);
-  if (!ws || ws_bytes < gather_product_ws(MCX_F32, G, O, K, P)) return MCX_E_WORKSPACE;
-  return mfma_f32_gather_product(src, map, iw, w, bias, y, (float *)ws, B, G, O, SH, SW, MH, MW,
-                                 K, P, interp, s);
-}
-
-// gW[a,g,k] = sum_{b,n} plain[b,a,n] * sample(gath[b,g], map[n,k]); n over MH x MW.
 size_t weight_grad_ws(int dtype, int64_t B, int64_t A, int64_t G, int64_t MH, int64_t MW,
                       int64_t K, int64_t P) {
-  if (dtype == MCX_F32 && mfma_f32_weight_grad_supported(P))
-    return align256(mfma_f32_weight_grad_bytes(B, A, G, MH, MW, K));
-  return 0;
+  return use_mfma(dtype, P) ? mfma_weight_grad_bytes(B, A, G, MH, MW, K) : 0;
+}
+size_t product_scatter_ws(int dtype, int64_t B, int64_t S, int64_t D, int64_t K, int64_t P,
+                          int64_t DH, int64_t DW) {
+  return use_mfma(dtype, P) ? mfma_product_scatter_bytes(B, S, D, K, DH, DW, elem_size(dtype)) : 0;
+}
+size_t bias_grad_ws(int dtype, int64_t B, int64_t C, int64_t N) {
+  if (dtype == MCX_BF16) return mfma_bias_grad_bytes(B, C, N);
+  return (channel_sum_scratch_bytes(B, C, N, elem_size(dtype)) + 255) & ~(size_t)255;
 }
 
+// ---- typed operators: scalar kernels for any T, matrix-core kernels for TD -----------
+// y[b,o,n] = bias[o] + sum_{g,k} W[o,g,k] * sample(src[b,g], map[n,k]); n over MH x MW.
 template <typename T>
-int weight_grad(const T *plain, const T *gath, const T *map, const T *iw, T *gw, void *ws,
-                size_t ws_bytes, int64_t B, int64_t A, int64_t G, int64_t GH, int64_t GW,
-                int64_t MH, int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s) {
-  (void)ws;
-  (void)ws_bytes;
-  return generic_weight_grad<T>(plain, gath, map, iw, gw, B, A, G, GH, GW, MH * MW, K, P, interp,
-                                s);
+int gather_product(bool mfma, const void *src, const void *map, const void *iw, const void *w,
+                   const void *bias, void *y, void *ws, size_t ws_bytes, int64_t B, int64_t G,
+                   int64_t O, int64_t SH, int64_t SW, int64_t MH, int64_t MW, int64_t K, int64_t P,
+                   int interp, hipStream_t s);
+
+// dst[b,d] = bias[d] (or 0) + splat(sum_s W[s,d,k] * src[b,s,n], map[n,k]); n over MH x MW.
+template <typename T>
+int product_scatter(bool mfma, const void *src, const void *map, const void *iw, const void *w,
+                    const void *bias, void *dst, void *ws, size_t ws_bytes, int64_t B, int64_t S,
+                    int64_t D, int64_t DH, int64_t DW, int64_t MH, int64_t MW, int64_t K, int64_t P,
+                    int interp, hipStream_t s);
+
+// gW[a,g,k] = sum_{b,n} plain[b,a,n] * sample(gath[b,g], map[n,k]); n over MH x MW.
+template <typename T>
+int weight_grad(bool mfma, const void *plain, const void *gath, const void *map, const void *iw,
+                void *gw, void *ws, size_t ws_bytes, int64_t B, int64_t A, int64_t G, int64_t GH,
+                int64_t GW, int64_t MH, int64_t MW, int64_t K, int64_t P, int interp,
+                hipStream_t s);
+
+// gb[c] = sum over (b, n) of gy[b,c,n].
+template <typename T>
+int bias_grad(const void *gy, void *gb, void *ws, size_t ws_bytes, int64_t B, int64_t C, int64_t N,
+              hipStream_t s);
+
+#define MCX_SCALAR_OPS(T)                                                                          \
+  template <>                                                                                      \
+  int gather_product<T>(bool, const void *src, const void *map, const void *iw, const void *w,     \
+                        const void *bias, void *y, void *, size_t, int64_t B, int64_t G,           \
+                        int64_t O, int64_t SH, int64_t SW, int64_t MH, int64_t MW, int64_t K,      \
+                        int64_t P, int interp, hipStream_t s) {                                    \
+    return generic_gather_product<T>((const T *)src, (const T *)map, (const T *)iw,                \
+                                     (const T *)w, (const T *)bias, (T *)y, B, G, O, SH, SW,       \
+                                     MH * MW, K, P, interp, s);                                    \
+  }                                                                                                \
+  template <>                                                                                      \
+  int product_scatter<T>(bool, const void *src, const void *map, const void *iw, const void *w,    \
+                         const void *bias, void *dst, void *, size_t, int64_t B, int64_t S,        \
+                         int64_t D, int64_t DH, int64_t DW, int64_t MH, int64_t MW, int64_t K,     \
+                         int64_t P, int interp, hipStream_t s) {                                   \
+    int rc = bias ? fill_bias<T>((T *)dst, (const T *)bias, B, D, DH * DW, s)                      \
+                  : fill_zero<T>((T *)dst, B * D * DH * DW, s);                                    \
+    if (rc) return rc;                                                                             \
+    return generic_product_scatter<T>((const T *)src, (const T *)map, (const T *)iw,               \
+                                      (const T *)w, (T *)dst, B, S, D, DH, DW, MH * MW, K, P,      \
+                                      interp, s);                                                  \
+  }                                                                                                \
+  template <>                                                                                      \
+  int weight_grad<T>(bool, const void *plain, const void *gath, const void *map, const void *iw,   \
+                     void *gw, void *, size_t, int64_t B, int64_t A, int64_t G, int64_t GH,        \
+                     int64_t GW, int64_t MH, int64_t MW, int64_t K, int64_t P, int interp,         \
+                     hipStream_t s) {                                                              \
+    return generic_weight_grad<T>((const T *)plain, (const T *)gath, (const T *)map,               \
+                                  (const T *)iw, (T *)gw, B, A, G, GH, GW, MH * MW, K, P, interp,  \
+                                  s);                                                              \
+  }                                                                                                \
+  template <>                                                                                      \
+  int bias_grad<T>(const void *gy, void *gb, void *ws, size_t ws_bytes, int64_t B, int64_t C,      \
+                   int64_t N, hipStream_t s) {                                                     \
+    const size_t need = channel_sum_scratch_bytes(B, C, N, sizeof(T));                             \
+    T *scratch = (ws && need > 0 && ws_bytes >= need) ? (T *)ws : nullptr;                         \
+    return channel_sum<T>((const T *)gy, (T *)gb, scratch, B, C, N, s);                            \
+  }
+
+// double: scalar kernels only
+MCX_SCALAR_OPS(double)
+
+// float: matrix-core kernels when `mfma`, scalar kernels otherwise
+
+template <>
+int gather_product<float>(bool mfma, const void *src, const void *map, const void *iw,
+                          const void *w, const void *bias, void *y, void *ws, size_t ws_bytes,
+                          int64_t B, int64_t G, int64_t O, int64_t SH, int64_t SW, int64_t MH,
+                          int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s) {
+  if (!mfma)
+    return generic_gather_product<float>((const float *)src, (const float *)map,
+                                         (const float *)iw, (const float *)w, (const float *)bias,
+                                         (float *)y, B, G, O, SH, SW, MH * MW, K, P, interp, s);
+  if (!ws || ws_bytes < mfma_gather_product_bytes(O, G, K)) return MCX_E_WORKSPACE;
+  return mfma_gather_product<float>((const float *)src, (const float *)map, (const float *)iw,
+                                    (const float *)w, (const float *)bias, (float *)y, ws, B, G, O,
+                                    SH, SW, MH, MW, K, P, interp, s);
 }
 
 template <>
-int weight_grad<float>(const float *plain, const float *gath, const float *map, const float *iw,
-                       float *gw, void *ws, size_t ws_bytes, int64_t B, int64_t A, int64_t G,
-                       int64_t GH, int64_t GW, int64_t MH, int64_t MW, int64_t K, int64_t P,
-                       int interp, hipStream_t s) {
-  if (!mfma_f32_weight_grad_supported(P))
-    return generic_weight_grad<float>(plain, gath, map, iw, gw, B, A, G, GH, GW, MH * MW, K, P,
-                                      interp, s);
-  if (!ws || ws_bytes < weight_grad_ws(MCX_F32, B, A, G, MH, MW, K, P)) return MCX_E_WORKSPACE;
-  return mfma_f32_weight_grad(plain, gath, map, iw, gw, (float *)ws, B, A, G, GH, GW, MH, MW, K,
-                              P, interp, s);
-}
-
-// dst[b,d] += splat(sum_s W[s,d,k] * src[b,s,n], map[n,k]); n over MH x MW; dst pre-initialised.
-size_t product_scatter_ws(int dtype, int64_t S, int64_t D, int64_t K, int64_t P, int64_t DH,
-                          int64_t DW) {
-  if (dtype == MCX_F32 && mfma_f32_product_scatter_supported(P))
-    return align256(mfma_f32_product_scatter_bytes(S, D, K, DH, DW));
-  return 0;
-}
-
-// `bias` (may be NULL) is the per-channel value dst was initialised with.
-template <typename T>
-int product_scatter(const T *src, const T *map, const T *iw, const T *w, const T *bias, T *dst,
-                    void *ws, size_t ws_bytes, int64_t B, int64_t S, int64_t D, int64_t DH,
-                    int64_t DW, int64_t MH, int64_t MW, int64_t K, int64_t P, int interp,
-                    hipStream_t s) {
-  (void)ws;
-  (void)ws_bytes;
-  (void)bias;
-  return generic_product_scatter<T>(src, map, iw, w, dst, B, S, D, DH, DW, MH * MW, K, P, interp,
-                                    s);
+int product_scatter<float>(bool mfma, const void *src, const void *map, const void *iw,
+                           const void *w, const void *bias, void *dst, void *ws, size_t ws_bytes,
+                           int64_t B, int64_t S, int64_t D, int64_t DH, int64_t DW, int64_t MH,
+                           int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s) {
+  if (!mfma) {
+    int rc = bias ? fill_bias<float>((float *)dst, (const float *)bias, B, D, DH * DW, s)
+                  : fill_zero<float>((float *)dst, B * D * DH * DW, s);
+    if (rc) return rc;
+    return generic_product_scatter<float>((const float *)src, (const float *)map,
+                                          (const float *)iw, (const float *)w, (float *)dst, B, S,
+                                          D, DH, DW, MH * MW, K, P, interp, s);
+  }
+  if (!ws || ws_bytes < mfma_product_scatter_bytes(B, S, D, K, DH, DW, 4)) return MCX_E_WORKSPACE;
+  return mfma_product_scatter<float>((const float *)src, (const float *)map, (const float *)iw,
+                                     (const float *)w, (const float *)bias, (float *)dst, ws, B, S,
+                                     D, DH, DW, MH, MW, K, P, interp, s);
 }
 
 template <>
-int product_scatter<float>(const float *src, const float *map, const float *iw, const float *w,
-                           const float *bias, float *dst, void *ws, size_t ws_bytes, int64_t B,
-                           int64_t S, int64_t D, int64_t DH, int64_t DW, int64_t MH, int64_t MW,
-                           int64_t K, int64_t P, int interp, hipStream_t s) {
-  if (!mfma_f32_product_scatter_supported(P))
-    return generic_product_scatter<float>(src, map, iw, w, dst, B, S, D, DH, DW, MH * MW, K, P,
-                                          interp, s);
-  if (!ws || ws_bytes < product_scatter_ws(MCX_F32, S, D, K, P, DH, DW)) return MCX_E_WORKSPACE;
-  return mfma_f32_product_scatter(src, map, iw, w, bias, dst, ws, B, S, D, DH, DW, MH, MW, K, P,
-                                  interp, s);
+int weight_grad<float>(bool mfma, const void *plain, const void *gath, const void *map,
+                       const void *iw, void *gw, void *ws, size_t ws_bytes, int64_t B, int64_t A,
+                       int64_t G, int64_t GH, int64_t GW, int64_t MH, int64_t MW, int64_t K,
+                       int64_t P, int interp, hipStream_t s) {
+  if (!mfma)
+    return generic_weight_grad<float>((const float *)plain, (const float *)gath,
+                                      (const float *)map, (const float *)iw, (float *)gw, B, A, G,
+                                      GH, GW, MH * MW, K, P, interp, s);
+  if (!ws || ws_bytes < mfma_weight_grad_bytes(B, A, G, MH, MW, K)) return MCX_E_WORKSPACE;
+  return mfma_weight_grad<float>((const float *)plain, (const float *)gath, (const float *)map,
+                                 (const float *)iw, (float *)gw, ws, B, A, G, GH, GW, MH, MW, K, P,
+                                 interp, s);
 }
 
-// gb[c] = sum over (b, n) of gy[b,c,n]; uses the scratch when it is large enough.
-template <typename T>
-int bias_grad(const T *gy, T *gb, void *ws, size_t ws_bytes, int64_t B, int64_t C, int64_t N,
-              hipStream_t s) {
-  const size_t need = channel_sum_scratch_bytes(B, C, N, sizeof(T));
-  T *scratch = (ws && need > 0 && ws_bytes >= need) ? (T *)ws : nullptr;
-  return channel_sum<T>(gy, gb, scratch, B, C, N, s);
+template <>
+int bias_grad<float>(const void *gy, void *gb, void *ws, size_t ws_bytes, int64_t B, int64_t C,
+                     int64_t N, hipStream_t s) {
+  const size_t need = channel_sum_scratch_bytes(B, C, N, sizeof(float));
+  float *scratch = (ws && need > 0 && ws_bytes >= need) ? (float *)ws : nullptr;
+  return channel_sum<float>((const float *)gy, (float *)gb, scratch, B, C, N, s);
 }
 
+// bf16 storage: matrix-core kernels only (sample_map / interp_weights are fp32)
+template <>
+int gather_product<bf16_t>(bool mfma, const void *src, const void *map, const void *iw,
+                           const void *w, const void *bias, void *y, void *ws, size_t ws_bytes,
+                           int64_t B, int64_t G, int64_t O, int64_t SH, int64_t SW, int64_t MH,
+                           int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s) {
+  if (!mfma) return MCX_E_DTYPE;
+  if (!ws || ws_bytes < mfma_gather_product_bytes(O, G, K)) return MCX_E_WORKSPACE;
+  return mfma_gather_product<bf16_t>((const bf16_t *)src, (const float *)map, (const float *)iw,
+                                     (const bf16_t *)w, (const bf16_t *)bias, (bf16_t *)y, ws, B,
+                                     G, O, SH, SW, MH, MW, K, P, interp, s);
+}
+
+template <>
+int product_scatter<bf16_t>(bool mfma, const void *src, const void *map, const void *iw,
+                            const void *w, const void *bias, void *dst, void *ws, size_t ws_bytes,
+                            int64_t B, int64_t S, int64_t D, int64_t DH, int64_t DW, int64_t MH,
+                            int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s) {
+  if (!mfma) return MCX_E_DTYPE;
+  if (!ws || ws_bytes < mfma_product_scatter_bytes(B, S, D, K, DH, DW, 2)) return MCX_E_WORKSPACE;
+  return mfma_product_scatter<bf16_t>((const bf16_t *)src, (const float *)map, (const float *)iw,
+                                      (const bf16_t *)w, (const bf16_t *)bias, (bf16_t *)dst, ws,
+                                      B, S, D, DH, DW, MH, MW, K, P, interp, s);
+}
+
+template <>
+int weight_grad<bf16_t>(bool mfma, const void *plain, const void *gath, const void *map,
+                        const void *iw, void *gw, void *ws, size_t ws_bytes, int64_t B, int64_t A,
+                        int64_t G, int64_t GH, int64_t GW, int64_t MH, int64_t MW, int64_t K,
+                        int64_t P, int interp, hipStream_t s) {
+  if (!mfma) return MCX_E_DTYPE;
+  if (!ws || ws_bytes < mfma_weight_grad_bytes(B, A, G, MH, MW, K)) return MCX_E_WORKSPACE;
+  return mfma_weight_grad<bf16_t>((const bf16_t *)plain, (const bf16_t *)gath, (const float *)map,
+                                  (const float *)iw, (bf16_t *)gw, ws, B, A, G, GH, GW, MH, MW, K,
+                                  P, interp, s);
+}
+
+template <>
+int bias_grad<bf16_t>(const void *gy, void *gb, void *ws, size_t ws_bytes, int64_t B, int64_t C,
+                      int64_t N, hipStream_t s) {
+  if (!ws || ws_bytes < mfma_bias_grad_bytes(B, C, N)) return MCX_E_WORKSPACE;
+  return mfma_bias_grad<bf16_t>((const bf16_t *)gy, (bf16_t *)gb, ws, B, C, N, s);
+}
+
+// ---- the four layer-level operations, in terms of the operators ----------------------
 template <typename T>
-int conv_forward_t(const void *x, const void *map, const void *iw, const void *w, const void *bias,
-                   void *y, void *ws, size_t ws_bytes, const ConvDims &d, int interp,
-                   hipStream_t s) {
-  return gather_product<T>((const T *)x, (const T *)map, (const T *)iw, (const T *)w,
-                           (const T *)bias, (T *)y, ws, ws_bytes, d.B, d.Ci, d.Co, d.IH, d.IW,
+int conv_forward_t(bool mfma, const void *x, const void *map, const void *iw, const void *w,
+                   const void *bias, void *y, void *ws, size_t ws_bytes, const ConvDims &d,
+                   int interp, hipStream_t s) {
+  return gather_product<T>(mfma, x, map, iw, w, bias, y, ws, ws_bytes, d.B, d.Ci, d.Co, d.IH, d.IW,
                            d.OH, d.OW, d.K, d.P, interp, s);
 }
 
 template <typename T>
-int conv_backward_t(const void *gy, const void *map, const void *iw, const void *x, const void *w,
-                    void *gx, void *gw, void *gb, void *ws, size_t ws_bytes, const ConvDims &d,
-                    int interp, hipStream_t s) {
+int conv_backward_t(bool mfma, const void *gy, const void *map, const void *iw, const void *x,
+                    const void *w, void *gx, void *gw, void *gb, void *ws, size_t ws_bytes,
+                    const ConvDims &d, int interp, hipStream_t s) {
   int rc = 0;
-  const int64_t N = d.OH * d.OW;
-  (void)N;
-  if (gx) {
-    if ((rc = fill_zero<T>((T *)gx, d.B * d.Ci * d.IH * d.IW, s))) return rc;
-    if ((rc = product_scatter<T>((const T *)gy, (const T *)map, (const T *)iw, (const T *)w,
-                                 (const T *)nullptr, (T *)gx, ws, ws_bytes, d.B, d.Co, d.Ci, d.IH,
+  if (gx && (rc = product_scatter<T>(mfma, gy, map, iw, w, nullptr, gx, ws, ws_bytes, d.B, d.Co,
+                                     d.Ci, d.IH, d.IW, d.OH, d.OW, d.K, d.P, interp, s)))
+    return rc;
+  if (gw && (rc = weight_grad<T>(mfma, gy, x, map, iw, gw, ws, ws_bytes, d.B, d.Co, d.Ci, d.IH,
                                  d.IW, d.OH, d.OW, d.K, d.P, interp, s)))
-      return rc;
-  }
-  if (gw) {
-    if ((rc = weight_grad<T>((const T *)gy, (const T *)x, (const T *)map, (const T *)iw, (T *)gw,
-                             ws, ws_bytes, d.B, d.Co, d.Ci, d.IH, d.IW, d.OH, d.OW, d.K, d.P,
-                             interp, s)))
-      return rc;
-  }
-  if (gb) rc = bias_grad<T>((const T *)gy, (T *)gb, ws, ws_bytes, d.B, d.Co, d.OH * d.OW, s);
+    return rc;
+  if (gb) rc = bias_grad<T>(gy, gb, ws, ws_bytes, d.B, d.Co, d.OH * d.OW, s);
   return rc;
 }
 
 template <typename T>
-int tconv_forward_t(const void *x, const void *map, const void *iw, const void *w,
+int tconv_forward_t(bool mfma, const void *x, const void *map, const void *iw, const void *w,
                     const void *bias, void *y, void *ws, size_t ws_bytes, const ConvDims &d,
                     int interp, hipStream_t s) {
-  int rc = fill_bias<T>((T *)y, (const T *)bias, d.B, d.Co, d.OH * d.OW, s);
-  if (rc) return rc;
-  return product_scatter<T>((const T *)x, (const T *)map, (const T *)iw, (const T *)w,
-                            (const T *)bias, (T *)y, ws, ws_bytes, d.B, d.Ci, d.Co, d.OH, d.OW,
-                            d.IH, d.IW, d.K, d.P, interp, s);
+  return product_scatter<T>(mfma, x, map, iw, w, bias, y, ws, ws_bytes, d.B, d.Ci, d.Co, d.OH,
+                            d.OW, d.IH, d.IW, d.K, d.P, interp, s);
 }
 
 template <typename T>
-int tconv_backward_t(const void *gy, const void *map, const void *iw, const void *x,
+int tconv_backward_t(bool mfma, const void *gy, const void *map, const void *iw, const void *x,
                      const void *w, void *gx, void *gw, void *gb, void *ws, size_t ws_bytes,
                      const ConvDims &d, int interp, hipStream_t s) {
   int rc = 0;
-  const int64_t N = d.IH * d.IW;
-  if (gx) {
-    // grad_input[b,ci] = sum_{co,k} W[ci,co,k] * sample(gy[b,co], map[n,k])
-    if ((rc = gather_product<T>((const T *)gy, (const T *)map, (const T *)iw, (const T *)w,
-                                (const T *)nullptr, (T *)gx, ws, ws_bytes, d.B, d.Co, d.Ci, d.OH,
-                                d.OW, d.IH, d.IW, d.K, d.P, interp, s)))
-      return rc;
-  }
-  if (gw) {
-    if ((rc = weight_grad<T>((const T *)x, (const T *)gy, (const T *)map, (const T *)iw, (T *)gw,
-                             ws, ws_bytes, d.B, d.Ci, d.Co, d.OH, d.OW, d.IH, d.IW, d.K, d.P,
-                             interp, s)))
-      return rc;
-  }
-  if (gb) rc = bias_grad<T>((const T *)gy, (T *)gb, ws, ws_bytes, d.B, d.Co, d.OH * d.OW, s);
+  // grad_input[b,ci] = sum_{co,k} W[ci,co,k] * sample(gy[b,co], map[n,k])
+  if (gx && (rc = gather_product<T>(mfma, gy, map, iw, w, nullptr, gx, ws, ws_bytes, d.B, d.Co,
+                                    d.Ci, d.OH, d.OW, d.IH, d.IW, d.K, d.P, interp, s)))
+    return rc;
+  if (gw && (rc = weight_grad<T>(mfma, x, gy, map, iw, gw, ws, ws_bytes, d.B, d.Ci, d.Co, d.OH,
+                                 d.OW, d.IH, d.IW, d.K, d.P, interp, s)))
+    return rc;
+  if (gb) rc = bias_grad<T>(gy, gb, ws, ws_bytes, d.B, d.Co, d.OH * d.OW, s);
   return rc;
 }
+
+#define MCX_DISPATCH_DTYPE(dtype, CALL)           \
+  switch (dtype) {                                \
+    case MCX_F32: { using T = float; return CALL; }   \
+    case MCX_F64: { using T = double; return CALL; }  \
+    case MCX_BF16: { using T = bf16_t; return CALL; } \
+    default: return MCX_E_DTYPE;                  \
+  }
 
 }  // namespace
 
@@ -234,24 +311,18 @@ extern "C" int mcx_conv_forward(const void *x, const void *map, const void *iw, 
   if (int rc = check_ptrs(x, map, iw, w, P)) return rc;
   if (!bias || !y) return MCX_E_NULL;
   hipStream_t s = (hipStream_t)stream;
-  switch (dtype) {
-    case MCX_F32:
-      return conv_forward_t<float>(x, map, iw, w, bias, y, workspace, workspace_bytes, d, interp, s);
-    case MCX_F64:
-      return conv_forward_t<double>(x, map, iw, w, bias, y, workspace, workspace_bytes, d, interp,
-                                    s);
-    default: return MCX_E_DTYPE;
-  }
+  const bool mfma = use_mfma(dtype, P);
+  MCX_DISPATCH_DTYPE(dtype, conv_forward_t<T>(mfma, x, map, iw, w, bias, y, workspace,
+                                              workspace_bytes, d, interp, s));
 }
 
 extern "C" size_t mcx_conv_backward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t IH,
                                               int64_t IW, int64_t OH, int64_t OW, int64_t K,
                                               int64_t P, int dtype) {
   // the gradients run one after the other on the stream and share the scratch
-  const size_t elem = dtype == MCX_F64 ? 8 : 4;
   return std::max({weight_grad_ws(dtype, B, Co, Ci, OH, OW, K, P),
-                   product_scatter_ws(dtype, Co, Ci, K, P, IH, IW),
-                   align256(channel_sum_scratch_bytes(B, Co, OH * OW, elem))});
+                   product_scatter_ws(dtype, B, Co, Ci, K, P, IH, IW),
+                   bias_grad_ws(dtype, B, Co, OH * OW)});
 }
 
 extern "C" int mcx_conv_backward(const void *gy, const void *map, const void *iw, const void *x,
@@ -264,21 +335,15 @@ extern "C" int mcx_conv_backward(const void *gy, const void *map, const void *iw
   if (int rc = check_ptrs(gy, map, iw, w, P)) return rc;
   if (gw && !x) return MCX_E_NULL;
   hipStream_t s = (hipStream_t)stream;
-  switch (dtype) {
-    case MCX_F32:
-      return conv_backward_t<float>(gy, map, iw, x, w, gx, gw, gb, workspace, workspace_bytes, d,
-                                    interp, s);
-    case MCX_F64:
-      return conv_backward_t<double>(gy, map, iw, x, w, gx, gw, gb, workspace, workspace_bytes, d,
-                                     interp, s);
-    default: return MCX_E_DTYPE;
-  }
+  const bool mfma = use_mfma(dtype, P);
+  MCX_DISPATCH_DTYPE(dtype, conv_backward_t<T>(mfma, gy, map, iw, x, w, gx, gw, gb, workspace,
+                                               workspace_bytes, d, interp, s));
 }
 
-extern "C" size_t mcx_tconv_forward_workspace(int64_t, int64_t Ci, int64_t Co, int64_t, int64_t,
+extern "C" size_t mcx_tconv_forward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t, int64_t,
                                               int64_t OH, int64_t OW, int64_t K, int64_t P,
                                               int dtype) {
-  return product_scatter_ws(dtype, Ci, Co, K, P, OH, OW);
+  return product_scatter_ws(dtype, B, Ci, Co, K, P, OH, OW);
 }
 
 extern "C" int mcx_tconv_forward(const void *x, const void *map, const void *iw, const void *w,
@@ -291,15 +356,9 @@ extern "C" int mcx_tconv_forward(const void *x, const void *map, const void *iw,
   if (int rc = check_ptrs(x, map, iw, w, P)) return rc;
   if (!bias || !y) return MCX_E_NULL;
   hipStream_t s = (hipStream_t)stream;
-  switch (dtype) {
-    case MCX_F32:
-      return tconv_forward_t<float>(x, map, iw, w, bias, y, workspace, workspace_bytes, d, interp,
-                                    s);
-    case MCX_F64:
-      return tconv_forward_t<double>(x, map, iw, w, bias, y, workspace, workspace_bytes, d,
-                                     interp, s);
-    default: return MCX_E_DTYPE;
-  }
+  const bool mfma = use_mfma(dtype, P);
+  MCX_DISPATCH_DTYPE(dtype, tconv_forward_t<T>(mfma, x, map, iw, w, bias, y, workspace,
+                                               workspace_bytes, d, interp, s));
 }
 
 extern "C" size_t mcx_tconv_backward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t IH,
@@ -307,10 +366,9 @@ extern "C" size_t mcx_tconv_backward_workspace(int64_t B, int64_t Ci, int64_t Co
                                                int64_t P, int dtype) {
   // backward-input is a gather-product with the channel roles swapped; the
   // gradients run one after the other and share the scratch
-  const size_t elem = dtype == MCX_F64 ? 8 : 4;
   return std::max({gather_product_ws(dtype, Co, Ci, K, P),
                    weight_grad_ws(dtype, B, Ci, Co, IH, IW, K, P),
-                   align256(channel_sum_scratch_bytes(B, Co, OH * OW, elem))});
+                   bias_grad_ws(dtype, B, Co, OH * OW)});
 }
 
 extern "C" int mcx_tconv_backward(const void *gy, const void *map, const void *iw, const void *x,
@@ -323,23 +381,17 @@ extern "C" int mcx_tconv_backward(const void *gy, const void *map, const void *i
   if (int rc = check_ptrs(gy, map, iw, w, P)) return rc;
   if (gw && !x) return MCX_E_NULL;
   hipStream_t s = (hipStream_t)stream;
-  switch (dtype) {
-    case MCX_F32:
-      return tconv_backward_t<float>(gy, map, iw, x, w, gx, gw, gb, workspace, workspace_bytes, d,
-                                     interp, s);
-    case MCX_F64:
-      return tconv_backward_t<double>(gy, map, iw, x, w, gx, gw, gb, workspace, workspace_bytes, d,
-                                      interp, s);
-    default: return MCX_E_DTYPE;
-  }
+  const bool mfma = use_mfma(dtype, P);
+  MCX_DISPATCH_DTYPE(dtype, tconv_backward_t<T>(mfma, gy, map, iw, x, w, gx, gw, gb, workspace,
+                                                workspace_bytes, d, interp, s));
 }
 
-extern "C" int mcx_abi_version(void) { return 2; }
+extern "C" int mcx_abi_version(void) { return 3; }
 
 extern "C" const char *mcx_error_string(int code) {
   switch (code) {
     case MCX_OK: return "success";
-    case MCX_E_DTYPE: return "mcx: dtype not supported by this entry point";
+    case MCX_E_DTYPE: return "mcx: dtype (or dtype / interpolation-point combination) not supported by this entry point";
     case MCX_E_SHAPE: return "mcx: invalid or too large dimension";
     case MCX_E_NULL: return "mcx: required pointer is NULL, or interp_weights and P disagree";
     case MCX_E_WORKSPACE: return "mcx: workspace missing or too small";

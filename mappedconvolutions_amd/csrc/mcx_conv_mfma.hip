@@ -35,7 +35,8 @@ __device__ inline int xcd_contiguous_tile(int wg, int total) {
 // Repack W[o][g][k] -> Wp[k][g][o] with g padded to 16 and o padded to 64 (zeros),
 // so that a reduction chunk's weights are 16 rows of contiguous floats.
 // `transposed` reads W[g][o][k] instead (weights stored source-channel major).
-__global__ void pack_weights_kernel(const float *__restrict__ w, float *__restrict__ wp, int O,
+template <typename TD>
+__global__ void pack_weights_kernel(const TD *__restrict__ w, float *__restrict__ wp, int O,
                                     int G, int K, int Opad, int Gpad, int transposed) {
   const int64_t total = (int64_t)K * Gpad * Opad;
   for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total;
@@ -44,14 +45,14 @@ __global__ void pack_weights_kernel(const float *__restrict__ w, float *__restri
     const int g = (int)((e / Opad) % Gpad);
     const int k = (int)(e / ((int64_t)Opad * Gpad));
     const int64_t wi = transposed ? ((int64_t)g * O + o) * K + k : ((int64_t)o * G + g) * K + k;
-    wp[e] = (o < O && g < G) ? w[wi] : 0.f;
+    wp[e] = (o < O && g < G) ? to_f32(w[wi]) : 0.f;
   }
 }
 
-template <int NCORN, int NP>
+template <typename TD, int NCORN, int NP>
 __global__ __launch_bounds__(kThreads, 2) void gather_product_mfma_kernel(
-    const float *__restrict__ src, const float *__restrict__ map, const float *__restrict__ iw,
-    const float *__restrict__ wp, const float *__restrict__ bias, float *__restrict__ y, int G,
+    const TD *__restrict__ src, const float *__restrict__ map, const float *__restrict__ iw,
+    const float *__restrict__ wp, const TD *__restrict__ bias, TD *__restrict__ y, int G,
     int O, int Opad, int Gpad, int SH, int SW, int OH, int OW, int K, int weighted, int wrap,
     int tiles_x, int tiles_per_img, int tw_shift, const int *__restrict__ gate, int run_if_zero) {
   __shared__ __attribute__((aligned(16))) float S[2][kGC][kTilePx];
@@ -77,7 +78,7 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_mfma_kernel(
   const bool live = gi < OH && gj < OW;
   const int64_t n_g = live ? (int64_t)gi * OW + gj : 0;
 
-  const float *src_b = src + (int64_t)b * G * plane;
+  const TD *src_b = src + (int64_t)b * G * plane;
   const int chunks = Gpad / kGC;
   const int iters = K * chunks;
 
@@ -99,14 +100,15 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_mfma_kernel(
   auto resolve = [&]() {
 #pragma unroll
     for (int sp = 0; sp < NP; sp++)
-      resolve_pairs<NCORN>(mx[sp], my[sp], SH, SW, wrap != 0, live ? mw[sp] : 0.f, taps[sp]);
+      resolve_pairs<NCORN, sizeof(TD)>(mx[sp], my[sp], SH, SW, wrap != 0, live ? mw[sp] : 0.f,
+                                       taps[sp]);
   };
   auto issue = [&](int k, int c) {
     const int g0 = c * kGC + half * 8;
 #pragma unroll
     for (int ch = 0; ch < 8; ch++) {
       const int g = min(g0 + ch, G - 1);  // padded channels read a valid plane, weights are 0
-      const float *pl = src_b + (int64_t)g * plane;
+      const TD *pl = src_b + (int64_t)g * plane;
 #pragma unroll
       for (int sp = 0; sp < NP; sp++)
 #pragma unroll
@@ -174,12 +176,13 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_mfma_kernel(
   const int pe = wave * 32 + l31;
   const int ei = tile_y * th + (pe >> tw_shift), ej = (tile_x << tw_shift) + (pe & tw_mask);
   if (ei < OH && ej < OW) {
-    float *yb = y + (int64_t)b * O * N + (int64_t)ei * OW + ej;
+    TD *yb = y + (int64_t)b * O * N + (int64_t)ei * OW + ej;
 #pragma unroll
     for (int i = 0; i < 16; i++) {
       const int o = o0 + (i >> 2) * 8 + lhi * 4 + (i & 3);
-      if (o < O) yb[(int64_t)o * N] = acc0[i] + (bias ? bias[o] : 0.f);
-      if (o + 32 < O) yb[(int64_t)(o + 32) * N] = acc1[i] + (bias ? bias[o + 32] : 0.f);
+      if (o < O) yb[(int64_t)o * N] = from_f32<TD>(acc0[i] + (bias ? to_f32(bias[o]) : 0.f));
+      if (o + 32 < O)
+        yb[(int64_t)(o + 32) * N] = from_f32<TD>(acc1[i] + (bias ? to_f32(bias[o + 32]) : 0.f));
     }
   }
 }
@@ -202,9 +205,9 @@ constexpr int kWgCB = 2;            // 16-channel blocks of gathered channels pe
 constexpr int kWgKT = 9;            // taps per pass (accumulators in registers)
 constexpr int kLdPx = kTilePx + 4;  // LDS row stride (floats)
 
-template <int NCORN, int NP>
+template <typename TD, int NCORN, int NP>
 __global__ __launch_bounds__(kThreads, 2) void weight_grad_mfma_kernel(
-    const float *__restrict__ plain, const float *__restrict__ gath,
+    const TD *__restrict__ plain, const TD *__restrict__ gath,
     const float *__restrict__ map, const float *__restrict__ iw, float *__restrict__ part, int A,
     int G, int GH, int GW, int MH, int MW, int K, int weighted, int wrap, int tiles_x,
     int tiles_per_img, int tw_shift, int total_tiles, int ranges, int cgroups) {
@@ -234,7 +237,8 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_mfma_kernel(
   const int half = __builtin_amdgcn_readfirstlane(tid >> 7);  // wave-uniform: scalar addressing
   const int g_first = cg * (kWgCB * kGC);
   // 16-byte loads of the plain tile need every row segment 16-byte aligned
-  const bool vec_ok = (MW & 3) == 0 && (reinterpret_cast<uintptr_t>(plain) & 15) == 0;
+  const bool vec_ok = (MW & (16 / (int)sizeof(TD) - 1)) == 0 &&
+                      (reinterpret_cast<uintptr_t>(plain) & 15) == 0;
 
   floatx4 acc[kWgKT][kWgCB];
 #pragma unroll
@@ -255,23 +259,30 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_mfma_kernel(
       const int a = tid >> 2, px0 = (tid & 3) * 32;
       const int si = i0 + (px0 >> tw_shift), sj = j0 + (px0 & tw_mask);
       const bool row_ok = (a0 + a) < A && si < MH;
-      const float *prow = plain + ((int64_t)b * A + min(a0 + a, A - 1)) * N +
-                          (int64_t)min(si, MH - 1) * MW;
-      float4 *dstv = reinterpret_cast<float4 *>(&Pt[a][px0]);
+      const TD *prow = plain + ((int64_t)b * A + min(a0 + a, A - 1)) * N +
+                       (int64_t)min(si, MH - 1) * MW;
+      float t[32];
       if (vec_ok && row_ok && sj + 32 <= MW) {
-        const float4 *srcv = reinterpret_cast<const float4 *>(prow + sj);
-        float4 t[8];
+        constexpr int kPer = 16 / (int)sizeof(TD);  // elements per 16-byte load
+        const uint4 *srcv = reinterpret_cast<const uint4 *>(prow + sj);
+        uint4 raw[32 / kPer];
 #pragma unroll
-        for (int r = 0; r < 8; r++) t[r] = srcv[r];
+        for (int r = 0; r < 32 / kPer; r++) raw[r] = srcv[r];
 #pragma unroll
-        for (int r = 0; r < 8; r++) dstv[r] = t[r];
+        for (int r = 0; r < 32 / kPer; r++) {
+          const TD *e = reinterpret_cast<const TD *>(&raw[r]);
+#pragma unroll
+          for (int q = 0; q < kPer; q++) t[r * kPer + q] = to_f32(e[q]);
+        }
       } else {
-        float t[32];
 #pragma unroll
-        for (int r = 0; r < 32; r++) t[r] = prow[min(sj + r, MW - 1)];
+        for (int r = 0; r < 32; r++) t[r] = to_f32(prow[min(sj + r, MW - 1)]);
 #pragma unroll
-        for (int r = 0; r < 32; r++) Pt[a][px0 + r] = (row_ok && sj + r < MW) ? t[r] : 0.f;
+        for (int r = 0; r < 32; r++) t[r] = (row_ok && sj + r < MW) ? t[r] : 0.f;
       }
+      float4 *dstv = reinterpret_cast<float4 *>(&Pt[a][px0]);
+#pragma unroll
+      for (int r = 0; r < 8; r++) dstv[r] = float4{t[4 * r], t[4 * r + 1], t[4 * r + 2], t[4 * r + 3]};
     }
     __syncthreads();
     float areg[32];
@@ -287,7 +298,7 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_mfma_kernel(
     const int gi = i0 + (p >> tw_shift), gj = j0 + (p & tw_mask);
     const bool live = gi < MH && gj < MW;
     const int64_t n_g = live ? (int64_t)gi * MW + gj : 0;
-    const float *gath_b = gath + (int64_t)b * G * gplane;
+    const TD *gath_b = gath + (int64_t)b * G * gplane;
 
     PairTap<NCORN> taps[NP];
     float mx[NP], my[NP], mw[NP];
@@ -304,13 +315,14 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_mfma_kernel(
     auto resolve = [&]() {
 #pragma unroll
       for (int sp = 0; sp < NP; sp++)
-        resolve_pairs<NCORN>(mx[sp], my[sp], GH, GW, wrap != 0, live ? mw[sp] : 0.f, taps[sp]);
+        resolve_pairs<NCORN, sizeof(TD)>(mx[sp], my[sp], GH, GW, wrap != 0, live ? mw[sp] : 0.f,
+                                         taps[sp]);
     };
     auto issue = [&](int cb) {
       const int g0 = g_first + cb * kGC + half * 8;
 #pragma unroll
       for (int ch = 0; ch < 8; ch++) {
-        const float *pl = gath_b + (int64_t)min(g0 + ch, G - 1) * gplane;
+        const TD *pl = gath_b + (int64_t)min(g0 + ch, G - 1) * gplane;
 #pragma unroll
         for (int sp = 0; sp < NP; sp++)
 #pragma unroll
@@ -381,13 +393,14 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_mfma_kernel(
   }
 }
 
-__global__ void reduce_partials_kernel(const float *__restrict__ part, float *__restrict__ out,
+template <typename TD>
+__global__ void reduce_partials_kernel(const float *__restrict__ part, TD *__restrict__ out,
                                        int ranges, int64_t n) {
   const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (e >= n) return;
   float s = 0.f;
   for (int r = 0; r < ranges; r++) s += part[(int64_t)r * n + e];
-  out[e] = s;
+  out[e] = from_f32<TD>(s);
 }
 
 // ---------------------------------------------------------------------------------
@@ -425,7 +438,8 @@ constexpr int kScThreads = 64;
 
 // Repack W[s][d][k] -> Wq[k][dc][s][16]: per (tap, 16-channel block) a contiguous
 // [Spad x 16] slice; s padded to 64, d padded to 16, zeros in the padding.
-__global__ void pack_scatter_weights_kernel(const float *__restrict__ w, float *__restrict__ wq,
+template <typename TD>
+__global__ void pack_scatter_weights_kernel(const TD *__restrict__ w, float *__restrict__ wq,
                                             int S, int D, int K, int Spad, int dchunks) {
   const int64_t total = (int64_t)K * dchunks * Spad * kScDC;
   for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total;
@@ -435,7 +449,7 @@ __global__ void pack_scatter_weights_kernel(const float *__restrict__ w, float *
     const int dc = (int)((e / ((int64_t)kScDC * Spad)) % dchunks);
     const int k = (int)(e / ((int64_t)kScDC * Spad * dchunks));
     const int d = dc * kScDC + dl;
-    wq[e] = (s < S && d < D) ? w[((int64_t)s * D + d) * K + k] : 0.f;
+    wq[e] = (s < S && d < D) ? to_f32(w[((int64_t)s * D + d) * K + k]) : 0.f;
   }
 }
 
@@ -459,9 +473,9 @@ __device__ inline int circ_delta(int xx, int xref, int dw, int halfw) {
   return d;
 }
 
-template <int NCORN, int NP>
+template <typename TD, int NCORN, int NP>
 __global__ __launch_bounds__(kScThreads, 2) void product_scatter_mfma_kernel(
-    const float *__restrict__ src, const float *__restrict__ map, const float *__restrict__ iw,
+    const TD *__restrict__ src, const float *__restrict__ map, const float *__restrict__ iw,
     const float *__restrict__ wq, float *__restrict__ dst, int S, int D, int Spad, int DH, int DW,
     int MH, int MW, int K, int weighted, int wrap, int tiles_x, int tiles_per_img,
     const int *__restrict__ gate, int run_if_zero) {
@@ -549,7 +563,7 @@ __global__ __launch_bounds__(kScThreads, 2) void product_scatter_mfma_kernel(
   }
   for (int e = lane; e < kScWaveWin * kScWinLd; e += 64) (&win[0][0])[e] = 0.f;
 
-  const float *src_b = src + (int64_t)b * S * N;
+  const TD *src_b = src + (int64_t)b * S * N;
   float *dst_b = dst + (int64_t)b * D * dplane;
 
   float breg[2][16];
@@ -559,7 +573,7 @@ __global__ __launch_bounds__(kScThreads, 2) void product_scatter_mfma_kernel(
 #pragma unroll
       for (int t = 0; t < 16; t++) {
         const int s = sc * kScSC + 4 * t + lq;
-        breg[nb][t] = (live[nb] && s < S) ? src_b[(int64_t)s * N + npx[nb]] : 0.f;
+        breg[nb][t] = (live[nb] && s < S) ? to_f32(src_b[(int64_t)s * N + npx[nb]]) : 0.f;
       }
   };
   if (schunks == 1) load_b(0);
@@ -754,62 +768,138 @@ inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
 
 }  // namespace
 
-bool mfma_f32_weight_grad_supported(int64_t P) { return P >= 0 && P <= 4; }
+// =================================================================================
+// Host side.  Every launcher is a template on the storage type TD (float or bf16_t)
+// and is instantiated for both at the end of the file.
+// =================================================================================
 
-size_t mfma_f32_weight_grad_bytes(int64_t B, int64_t A, int64_t G, int64_t MH, int64_t MW,
-                                  int64_t K) {
-  const PixelTiling t = make_tiling(B, MH, MW);
-  return (size_t)weight_grad_ranges(t.total, A, G, K) * (size_t)(A * G * K) * sizeof(float);
+bool mfma_supported(int64_t P) { return P >= 0 && P <= 4; }
+
+namespace {
+
+inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+struct ModeArgs {
+  int mode, weighted, wrap, np;
+};
+inline ModeArgs mode_args(int interp, int64_t P) {
+  ModeArgs m;
+  m.mode = canonical_interp(interp);
+  m.weighted = P > 0 ? 1 : 0;
+  m.wrap = m.mode == kInterpBispherical ? 1 : 0;
+  m.np = P > 0 ? (int)P : 1;
+  return m;
 }
 
-// part: scratch of mfma_f32_weight_grad_bytes(...) bytes.
-int mfma_f32_weight_grad(const float *plain, const float *gath, const float *map, const float *iw,
-                         float *gw, float *part, int64_t B, int64_t A, int64_t G, int64_t GH,
-                         int64_t GW, int64_t MH, int64_t MW, int64_t K, int64_t P, int interp,
-                         hipStream_t s) {
+// Expands LAUNCH(NCORN, NP) for the interpolation mode and point count at hand.
+#define MCX_DISPATCH_TAPS(m, LAUNCH)   \
+  if ((m).mode == kInterpNearest) {    \
+    switch ((m).np) {                  \
+      case 1: LAUNCH(1, 1); break;     \
+      case 2: LAUNCH(1, 2); break;     \
+      case 3: LAUNCH(1, 3); break;     \
+      default: LAUNCH(1, 4); break;    \
+    }                                  \
+  } else {                             \
+    switch ((m).np) {                  \
+      case 1: LAUNCH(4, 1); break;     \
+      case 2: LAUNCH(4, 2); break;     \
+      case 3: LAUNCH(4, 3); break;     \
+      default: LAUNCH(4, 4); break;    \
+    }                                  \
+  }
+
+template <typename TD>
+int launch_gather_product(const TD *src, const float *map, const float *iw, const float *wp,
+                          const TD *bias, TD *y, int64_t B, int64_t G, int64_t O, int64_t SH,
+                          int64_t SW, int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
+                          const int *gate, int run_if_zero, hipStream_t s) {
+  const int Opad = (int)round_up(O, kOT), Gpad = (int)round_up(G, kGC);
+  const PixelTiling t = make_tiling(B, OH, OW);
+  if (t.total > 0x7fffffffLL) return MCX_E_SHAPE;
+  dim3 grid((unsigned)t.total, (unsigned)(Opad / kOT));
+  const ModeArgs m = mode_args(interp, P);
+#define MCX_LAUNCH(NCORN, NP)                                                                    \
+  hipLaunchKernelGGL((gather_product_mfma_kernel<TD, NCORN, NP>), grid, dim3(kThreads), 0, s,    \
+                     src, map, iw, wp, bias, y, (int)G, (int)O, Opad, Gpad, (int)SH, (int)SW,    \
+                     (int)OH, (int)OW, (int)K, m.weighted, m.wrap, t.tiles_x, t.tiles_per_img,   \
+                     t.tw_shift, gate, run_if_zero)
+  MCX_DISPATCH_TAPS(m, MCX_LAUNCH)
+#undef MCX_LAUNCH
+  MCX_HIP_CHECK_LAUNCH();
+  return 0;
+}
+
+template <typename TD>
+int launch_pack_weights(const TD *w, float *wp, int64_t O, int64_t G, int64_t K, int transposed,
+                        hipStream_t s) {
+  const int Opad = (int)round_up(O, kOT), Gpad = (int)round_up(G, kGC);
+  const int64_t packed = (int64_t)K * Gpad * Opad;
+  hipLaunchKernelGGL(pack_weights_kernel<TD>,
+                     dim3((unsigned)std::min<int64_t>((packed + 255) / 256, 4096)), dim3(256), 0, s,
+                     w, wp, (int)O, (int)G, (int)K, Opad, Gpad, transposed);
+  MCX_HIP_CHECK_LAUNCH();
+  return 0;
+}
+
+}  // namespace
+
+// ---- gather-product --------------------------------------------------------------
+size_t mfma_gather_product_bytes(int64_t O, int64_t G, int64_t K) {
+  return align256((size_t)(K * round_up(G, kGC) * round_up(O, kOT)) * sizeof(float));
+}
+
+// scratch: mfma_gather_product_bytes(O, G, K) bytes (packed weights).
+template <typename TD>
+int mfma_gather_product(const TD *src, const float *map, const float *iw, const TD *w,
+                        const TD *bias, TD *y, void *scratch, int64_t B, int64_t G, int64_t O,
+                        int64_t SH, int64_t SW, int64_t OH, int64_t OW, int64_t K, int64_t P,
+                        int interp, hipStream_t s) {
+  float *wp = (float *)scratch;
+  if (int rc = launch_pack_weights<TD>(w, wp, O, G, K, 0, s)) return rc;
+  return launch_gather_product<TD>(src, map, iw, wp, bias, y, B, G, O, SH, SW, OH, OW, K, P,
+                                   interp, nullptr, 0, s);
+}
+
+// ---- weight gradient ---------------------------------------------------------------
+size_t mfma_weight_grad_bytes(int64_t B, int64_t A, int64_t G, int64_t MH, int64_t MW,
+                              int64_t K) {
+  const PixelTiling t = make_tiling(B, MH, MW);
+  return align256((size_t)weight_grad_ranges(t.total, A, G, K) * (size_t)(A * G * K) *
+                  sizeof(float));
+}
+
+// scratch: mfma_weight_grad_bytes(...) bytes (per-range partial sums).
+template <typename TD>
+int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const float *iw, TD *gw,
+                     void *scratch, int64_t B, int64_t A, int64_t G, int64_t GH, int64_t GW,
+                     int64_t MH, int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s) {
+  float *part = (float *)scratch;
   const PixelTiling t = make_tiling(B, MH, MW);
   if (t.total > 0x7fffffffLL) return MCX_E_SHAPE;
   const int ranges = weight_grad_ranges(t.total, A, G, K);
   const int cgroups = (int)((G + kWgCB * kGC - 1) / (kWgCB * kGC));
   dim3 grid((unsigned)(ranges * cgroups), (unsigned)((A + kWgA - 1) / kWgA),
             (unsigned)((K + kWgKT - 1) / kWgKT));
-  const int mode = canonical_interp(interp);
-  const int weighted = P > 0 ? 1 : 0, wrap = mode == kInterpBispherical ? 1 : 0;
-  const int np = P > 0 ? (int)P : 1;
+  const ModeArgs m = mode_args(interp, P);
 #define MCX_LAUNCH(NCORN, NP)                                                                    \
-  hipLaunchKernelGGL((weight_grad_mfma_kernel<NCORN, NP>), grid, dim3(kThreads), 0, s, plain,    \
+  hipLaunchKernelGGL((weight_grad_mfma_kernel<TD, NCORN, NP>), grid, dim3(kThreads), 0, s, plain, \
                      gath, map, iw, part, (int)A, (int)G, (int)GH, (int)GW, (int)MH, (int)MW,    \
-                     (int)K, weighted, wrap, t.tiles_x, t.tiles_per_img, t.tw_shift,             \
+                     (int)K, m.weighted, m.wrap, t.tiles_x, t.tiles_per_img, t.tw_shift,         \
                      (int)t.total, ranges, cgroups)
-  if (mode == kInterpNearest) {
-    switch (np) {
-      case 1: MCX_LAUNCH(1, 1); break;
-      case 2: MCX_LAUNCH(1, 2); break;
-      case 3: MCX_LAUNCH(1, 3); break;
-      default: MCX_LAUNCH(1, 4); break;
-    }
-  } else {
-    switch (np) {
-      case 1: MCX_LAUNCH(4, 1); break;
-      case 2: MCX_LAUNCH(4, 2); break;
-      case 3: MCX_LAUNCH(4, 3); break;
-      default: MCX_LAUNCH(4, 4); break;
-    }
-  }
+  MCX_DISPATCH_TAPS(m, MCX_LAUNCH)
 #undef MCX_LAUNCH
   MCX_HIP_CHECK_LAUNCH();
   const int64_t n = A * G * K;
-  hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s,
-                     part, gw, ranges, n);
+  hipLaunchKernelGGL(reduce_partials_kernel<TD>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                     s, part, gw, ranges, n);
   MCX_HIP_CHECK_LAUNCH();
   return 0;
 }
 
-bool mfma_f32_product_scatter_supported(int64_t P) { return P >= 0 && P <= 4; }
-
+// ---- product-scatter ---------------------------------------------------------------
 namespace {
 
-// ---------------------------------------------------------------------------------
 // Transposed map.  A scatter through map[n,k] is a gather through the transposed
 // map: destination pixel p receives wt * col[., k, n] from every (n, corner) that
 // lands on it.  When no (p, k) receives more than kTransSlots contributions (true for
@@ -854,25 +944,49 @@ __global__ void build_transposed_map_kernel(const float *__restrict__ map,
   }
 }
 
+// dst[b,c,:] = bias[c] (or 0); runs only when the gate agrees (see above).
+template <typename TD>
+__global__ void init_planes_kernel(float *__restrict__ dst, const TD *__restrict__ bias, int C,
+                                   int64_t plane, int64_t total, const int *__restrict__ gate,
+                                   int run_if_zero) {
+  if (gate && ((*gate == 0) != (run_if_zero != 0))) return;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x)
+    dst[i] = bias ? to_f32(bias[(i / plane) % C]) : 0.f;
+}
+
+template <typename TD>
+__global__ void convert_planes_kernel(const float *__restrict__ src, TD *__restrict__ dst,
+                                      int64_t total, const int *__restrict__ gate,
+                                      int run_if_zero) {
+  if (gate && ((*gate == 0) != (run_if_zero != 0))) return;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x)
+    dst[i] = from_f32<TD>(src[i]);
+}
+
 struct ScatterScratch {
-  size_t wq, wpt, cnt, tmap, tiw, total;  // byte offsets; cnt holds the counters + the flag
+  size_t wq, wpt, cnt, tmap, tiw, acc32, total;  // byte offsets
   bool transposed_path;
 };
 
-inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
-
-ScatterScratch scatter_scratch(int64_t S, int64_t D, int64_t K, int64_t DH, int64_t DW) {
+// elem: bytes per data element; a non-fp32 destination needs an fp32 accumulation
+// image for the atomic path.
+ScatterScratch scatter_scratch(int64_t B, int64_t S, int64_t D, int64_t K, int64_t DH, int64_t DW,
+                               size_t elem) {
   ScatterScratch sc;
   size_t off = 0;
   sc.wq = off;
   off += align256((size_t)(K * ((D + kScDC - 1) / kScDC) * round_up(S, kScSC) * kScDC) * 4);
+  sc.acc32 = off;
+  if (elem != 4) off += align256((size_t)(B * D * DH * DW) * 4);
   const int64_t cells = DH * DW * K;
   sc.transposed_path = cells * kTransSlots * 2 <= 0x7fffffffLL;
   sc.wpt = sc.cnt = sc.tmap = sc.tiw = off;
   if (sc.transposed_path) {
     sc.wpt = off;
     off += align256((size_t)(K * round_up(S, kGC) * round_up(D, kOT)) * 4);
-    sc.cnt = off;
+    sc.cnt = off;  // counters, then the overflow flag; cleared together with tmap and tiw
     off += align256((size_t)(cells + 1) * 4);
     sc.tmap = off;
     off += align256((size_t)cells * kTransSlots * 2 * 4);
@@ -883,32 +997,25 @@ ScatterScratch scatter_scratch(int64_t S, int64_t D, int64_t K, int64_t DH, int6
   return sc;
 }
 
-int launch_gather_product(const float *src, const float *map, const float *iw, const float *wp,
-                          const float *bias, float *y, int64_t B, int64_t G, int64_t O, int64_t SH,
-                          int64_t SW, int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
-                          const int *gate, int run_if_zero, hipStream_t s);
-
 }  // namespace
 
-size_t mfma_f32_product_scatter_bytes(int64_t S, int64_t D, int64_t K, int64_t DH, int64_t DW) {
-  return scatter_scratch(S, D, K, DH, DW).total;
+size_t mfma_product_scatter_bytes(int64_t B, int64_t S, int64_t D, int64_t K, int64_t DH,
+                                  int64_t DW, size_t elem) {
+  return scatter_scratch(B, S, D, K, DH, DW, elem).total;
 }
 
-// dst must already hold its initial value (zeros or bias[d] broadcast); `bias` is
-// that per-channel initial value or NULL for zeros.  scratch: device memory of
-// mfma_f32_product_scatter_bytes(...) bytes.
-int mfma_f32_product_scatter(const float *src, const float *map, const float *iw, const float *w,
-                             const float *bias, float *dst, void *scratch, int64_t B, int64_t S,
-                             int64_t D, int64_t DH, int64_t DW, int64_t MH, int64_t MW, int64_t K,
-                             int64_t P, int interp, hipStream_t s) {
-  const ScatterScratch sc = scatter_scratch(S, D, K, DH, DW);
+// dst is fully overwritten: dst[b,d] = bias[d] (or 0) + scattered products.
+// scratch: mfma_product_scatter_bytes(...) bytes.
+template <typename TD>
+int mfma_product_scatter(const TD *src, const float *map, const float *iw, const TD *w,
+                         const TD *bias, TD *dst, void *scratch, int64_t B, int64_t S, int64_t D,
+                         int64_t DH, int64_t DW, int64_t MH, int64_t MW, int64_t K, int64_t P,
+                         int interp, hipStream_t s) {
+  const ScatterScratch sc = scatter_scratch(B, S, D, K, DH, DW, sizeof(TD));
   char *base = (char *)scratch;
   float *wq = (float *)(base + sc.wq);
   const int Spad = (int)round_up(S, kScSC), dchunks = (int)((D + kScDC - 1) / kScDC);
-  const int64_t packed = (int64_t)K * dchunks * Spad * kScDC;
-  const int mode = canonical_interp(interp);
-  const int weighted = P > 0 ? 1 : 0, wrap = mode == kInterpBispherical ? 1 : 0;
-  const int np = P > 0 ? (int)P : 1;
+  const ModeArgs m = mode_args(interp, P);
   const int *gate = nullptr;
 
   if (sc.transposed_path) {
@@ -919,30 +1026,33 @@ int mfma_f32_product_scatter(const float *src, const float *map, const float *iw
     const int64_t cells = DH * DW * K;
     int *flag = cnt + cells;
     gate = flag;
-    int rc = fill_f32((float *)cnt, (int64_t)((sc.total - sc.cnt) / 4), 0.f, s);
-    if (rc) return rc;
+    if (int rc = fill_f32((float *)cnt, (int64_t)((sc.total - sc.cnt) / 4), 0.f, s)) return rc;
     const int64_t entries = MH * MW * K;
     const unsigned blocks = (unsigned)((entries + 255) / 256);
-    if (mode == kInterpNearest)
+    if (m.mode == kInterpNearest)
       hipLaunchKernelGGL(build_transposed_map_kernel<1>, dim3(blocks), dim3(256), 0, s, map, iw,
-                         cnt, tmap, tiw, flag, np, weighted, wrap, (int)DH, (int)DW, (int)MW,
-                         (int)K, entries);
+                         cnt, tmap, tiw, flag, m.np, m.weighted, m.wrap, (int)DH, (int)DW,
+                         (int)MW, (int)K, entries);
     else
       hipLaunchKernelGGL(build_transposed_map_kernel<4>, dim3(blocks), dim3(256), 0, s, map, iw,
-                         cnt, tmap, tiw, flag, np, weighted, wrap, (int)DH, (int)DW, (int)MW,
-                         (int)K, entries);
+                         cnt, tmap, tiw, flag, m.np, m.weighted, m.wrap, (int)DH, (int)DW,
+                         (int)MW, (int)K, entries);
     MCX_HIP_CHECK_LAUNCH();
-    const int Opad = (int)round_up(D, kOT), Gpad = (int)round_up(S, kGC);
-    const int64_t pk = (int64_t)K * Gpad * Opad;
-    hipLaunchKernelGGL(pack_weights_kernel, dim3((unsigned)std::min<int64_t>((pk + 255) / 256, 4096)),
-                       dim3(256), 0, s, w, wpt, (int)D, (int)S, (int)K, Opad, Gpad, 1);
-    MCX_HIP_CHECK_LAUNCH();
-    rc = launch_gather_product(src, tmap, tiw, wpt, bias, dst, B, S, D, MH, MW, DH, DW, K,
-                               kTransSlots, kInterpNearest, gate, 1, s);
-    if (rc) return rc;
+    if (int rc = launch_pack_weights<TD>(w, wpt, D, S, K, 1, s)) return rc;
+    if (int rc = launch_gather_product<TD>(src, tmap, tiw, wpt, bias, dst, B, S, D, MH, MW, DH,
+                                           DW, K, kTransSlots, kInterpNearest, gate, 1, s))
+      return rc;
   }
 
-  hipLaunchKernelGGL(pack_scatter_weights_kernel,
+  // atomic path (runs when there is no transposed map or it overflowed)
+  const int64_t total_dst = B * D * DH * DW;
+  float *acc = sizeof(TD) == 4 ? (float *)dst : (float *)(base + sc.acc32);
+  const unsigned fill_blocks = (unsigned)std::min<int64_t>((total_dst + 1023) / 1024, 65536);
+  hipLaunchKernelGGL(init_planes_kernel<TD>, dim3(fill_blocks), dim3(256), 0, s, acc, bias, (int)D,
+                     DH * DW, total_dst, gate, 0);
+  MCX_HIP_CHECK_LAUNCH();
+  const int64_t packed = (int64_t)K * dchunks * Spad * kScDC;
+  hipLaunchKernelGGL(pack_scatter_weights_kernel<TD>,
                      dim3((unsigned)std::min<int64_t>((packed + 255) / 256, 4096)), dim3(256), 0, s,
                      w, wq, (int)S, (int)D, (int)K, Spad, dchunks);
   MCX_HIP_CHECK_LAUNCH();
@@ -952,90 +1062,91 @@ int mfma_f32_product_scatter(const float *src, const float *map, const float *iw
   if (total > 0x7fffffffLL) return MCX_E_SHAPE;
   dim3 grid((unsigned)total);
 #define MCX_LAUNCH(NCORN, NP)                                                                    \
-  hipLaunchKernelGGL((product_scatter_mfma_kernel<NCORN, NP>), grid, dim3(kScThreads), 0, s,     \
-                     src, map, iw, wq, dst, (int)S, (int)D, Spad, (int)DH, (int)DW, (int)MH,     \
-                     (int)MW, (int)K, weighted, wrap, tiles_x, (int)tiles_per_img, gate, 0)
-  if (mode == kInterpNearest) {
-    switch (np) {
-      case 1: MCX_LAUNCH(1, 1); break;
-      case 2: MCX_LAUNCH(1, 2); break;
-      case 3: MCX_LAUNCH(1, 3); break;
-      default: MCX_LAUNCH(1, 4); break;
-    }
-  } else {
-    switch (np) {
-      case 1: MCX_LAUNCH(4, 1); break;
-      case 2: MCX_LAUNCH(4, 2); break;
-      case 3: MCX_LAUNCH(4, 3); break;
-      default: MCX_LAUNCH(4, 4); break;
-    }
-  }
+  hipLaunchKernelGGL((product_scatter_mfma_kernel<TD, NCORN, NP>), grid, dim3(kScThreads), 0, s, \
+                     src, map, iw, wq, acc, (int)S, (int)D, Spad, (int)DH, (int)DW, (int)MH,     \
+                     (int)MW, (int)K, m.weighted, m.wrap, tiles_x, (int)tiles_per_img, gate, 0)
+  MCX_DISPATCH_TAPS(m, MCX_LAUNCH)
 #undef MCX_LAUNCH
+  MCX_HIP_CHECK_LAUNCH();
+  if (sizeof(TD) != 4) {
+    hipLaunchKernelGGL(convert_planes_kernel<TD>, dim3(fill_blocks), dim3(256), 0, s, acc, dst,
+                       total_dst, gate, 0);
+    MCX_HIP_CHECK_LAUNCH();
+  }
+  return 0;
+}
+
+// ---- bias gradient for bf16 (fp32 accumulation) ---------------------------------------
+namespace {
+template <typename TD>
+__global__ __launch_bounds__(256) void channel_sum_partial_td_kernel(const TD *__restrict__ g,
+                                                                     float *__restrict__ part,
+                                                                     int C, int N, int splits) {
+  const int c = blockIdx.x, b = blockIdx.y, sp = blockIdx.z;
+  const int per = (N + splits - 1) / splits;
+  const int n0 = sp * per, n1 = min(N, n0 + per);
+  const TD *p = g + ((int64_t)b * C + c) * N;
+  float acc = 0.f;
+  for (int n = n0 + threadIdx.x; n < n1; n += 256) acc += to_f32(p[n]);
+  __shared__ float red[256];
+  red[threadIdx.x] = acc;
+  __syncthreads();
+  for (int stride = 128; stride > 0; stride >>= 1) {
+    if ((int)threadIdx.x < stride) red[threadIdx.x] += red[threadIdx.x + stride];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) part[(int64_t)c * gridDim.y * splits + b * splits + sp] = red[0];
+}
+template <typename TD>
+__global__ void channel_sum_final_td_kernel(const float *__restrict__ part, TD *__restrict__ gb,
+                                            int C, int per_channel) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  float acc = 0.f;
+  for (int i = 0; i < per_channel; i++) acc += part[(int64_t)c * per_channel + i];
+  gb[c] = from_f32<TD>(acc);
+}
+inline int bias_splits(int64_t B, int64_t C, int64_t N) {
+  int splits = 1;
+  while (B * C * splits < 2048 && N / (splits * 2) >= 4096 && splits < 64) splits *= 2;
+  return splits;
+}
+}  // namespace
+
+size_t mfma_bias_grad_bytes(int64_t B, int64_t C, int64_t N) {
+  return align256((size_t)(B * C * bias_splits(B, C, N)) * sizeof(float));
+}
+
+template <typename TD>
+int mfma_bias_grad(const TD *g, TD *gb, void *scratch, int64_t B, int64_t C, int64_t N,
+                   hipStream_t s) {
+  const int splits = bias_splits(B, C, N);
+  float *part = (float *)scratch;
+  hipLaunchKernelGGL(channel_sum_partial_td_kernel<TD>, dim3((unsigned)C, (unsigned)B,
+                                                             (unsigned)splits),
+                     dim3(256), 0, s, g, part, (int)C, (int)N, splits);
+  MCX_HIP_CHECK_LAUNCH();
+  hipLaunchKernelGGL(channel_sum_final_td_kernel<TD>, dim3((unsigned)((C + 63) / 64)), dim3(64), 0,
+                     s, part, gb, (int)C, (int)(B * splits));
   MCX_HIP_CHECK_LAUNCH();
   return 0;
 }
 
-namespace {
-}  // namespace
-
-size_t mfma_f32_packed_weight_bytes(int64_t O, int64_t G, int64_t K) {
-  return (size_t)(K * round_up(G, kGC) * round_up(O, kOT)) * sizeof(float);
-}
-
-bool mfma_f32_gather_product_supported(int64_t P) { return P >= 0 && P <= 4; }
-
-namespace {
-int launch_gather_product(const float *src, const float *map, const float *iw, const float *wp,
-                          const float *bias, float *y, int64_t B, int64_t G, int64_t O, int64_t SH,
-                          int64_t SW, int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
-                          const int *gate, int run_if_zero, hipStream_t s) {
-  const int Opad = (int)round_up(O, kOT), Gpad = (int)round_up(G, kGC);
-  const PixelTiling t = make_tiling(B, OH, OW);
-  const int tw_shift = t.tw_shift, tiles_x = t.tiles_x, tiles_per_img = t.tiles_per_img;
-  const int64_t total = t.total;
-  if (total > 0x7fffffffLL) return MCX_E_SHAPE;
-  dim3 grid((unsigned)total, (unsigned)(Opad / kOT));
-  const int mode = canonical_interp(interp);
-  const int weighted = P > 0 ? 1 : 0, wrap = mode == kInterpBispherical ? 1 : 0;
-  const int np = P > 0 ? (int)P : 1;
-#define MCX_LAUNCH(NCORN, NP)                                                                    \
-  hipLaunchKernelGGL((gather_product_mfma_kernel<NCORN, NP>), grid, dim3(kThreads), 0, s, src,   \
-                     map, iw, wp, bias, y, (int)G, (int)O, Opad, Gpad, (int)SH, (int)SW,         \
-                     (int)OH, (int)OW, (int)K, weighted, wrap, tiles_x, tiles_per_img, tw_shift, \
-                     gate, run_if_zero)
-  if (mode == kInterpNearest) {
-    switch (np) {
-      case 1: MCX_LAUNCH(1, 1); break;
-      case 2: MCX_LAUNCH(1, 2); break;
-      case 3: MCX_LAUNCH(1, 3); break;
-      default: MCX_LAUNCH(1, 4); break;
-    }
-  } else {
-    switch (np) {
-      case 1: MCX_LAUNCH(4, 1); break;
-      case 2: MCX_LAUNCH(4, 2); break;
-      case 3: MCX_LAUNCH(4, 3); break;
-      default: MCX_LAUNCH(4, 4); break;
-    }
-  }
-#undef MCX_LAUNCH
-  MCX_HIP_CHECK_LAUNCH();
-  return 0;
-}
-}  // namespace
-
-// wp: scratch of mfma_f32_packed_weight_bytes(O, G, K) bytes.
-int mfma_f32_gather_product(const float *src, const float *map, const float *iw, const float *w,
-                            const float *bias, float *y, float *wp, int64_t B, int64_t G,
-                            int64_t O, int64_t SH, int64_t SW, int64_t OH, int64_t OW, int64_t K,
-                            int64_t P, int interp, hipStream_t s) {
-  const int Opad = (int)round_up(O, kOT), Gpad = (int)round_up(G, kGC);
-  const int64_t packed = (int64_t)K * Gpad * Opad;
-  hipLaunchKernelGGL(pack_weights_kernel, dim3((unsigned)std::min<int64_t>((packed + 255) / 256, 4096)),
-                     dim3(256), 0, s, w, wp, (int)O, (int)G, (int)K, Opad, Gpad, 0);
-  MCX_HIP_CHECK_LAUNCH();
-  return launch_gather_product(src, map, iw, wp, bias, y, B, G, O, SH, SW, OH, OW, K, P, interp,
-                               nullptr, 0, s);
-}
+#define MCX_INSTANTIATE_TD(TD)                                                                     \
+  template int mfma_gather_product<TD>(const TD *, const float *, const float *, const TD *,      \
+                                       const TD *, TD *, void *, int64_t, int64_t, int64_t,       \
+                                       int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int, \
+                                       hipStream_t);                                              \
+  template int mfma_weight_grad<TD>(const TD *, const TD *, const float *, const float *, TD *,   \
+                                    void *, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, \
+                                    int64_t, int64_t, int64_t, int, hipStream_t);                 \
+  template int mfma_product_scatter<TD>(const TD *, const float *, const float *, const TD *,     \
+                                        const TD *, TD *, void *, int64_t, int64_t, int64_t,      \
+                                        int64_t, int64_t, int64_t, int64_t, int64_t, int64_t,     \
+                                        int, hipStream_t);                                        \
+  template int mfma_bias_grad<TD>(const TD *, TD *, void *, int64_t, int64_t, int64_t,            \
+                                  hipStream_t);
+MCX_INSTANTIATE_TD(float)
+MCX_INSTANTIATE_TD(bf16_t)
 
 }  // namespace mcx

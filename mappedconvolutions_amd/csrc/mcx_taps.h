@@ -10,27 +10,50 @@
 
 namespace mcx {
 
-// off[] are BYTE offsets of fp32 elements, unsigned, so that a load from a
-// wave-uniform plane pointer compiles to "scalar base + 32-bit vector offset".
+// Storage types of the convolution data: fp32, or bf16 (converted to fp32 on load,
+// rounded to nearest-even on store; all arithmetic and accumulation is fp32).
+struct bf16_t {
+  uint16_t v;
+};
+__device__ inline float to_f32(float x) { return x; }
+__device__ inline float to_f32(bf16_t x) { return __builtin_bit_cast(float, (uint32_t)x.v << 16); }
+template <typename TD>
+__device__ inline TD from_f32(float x);
+template <>
+__device__ inline float from_f32<float>(float x) {
+  return x;
+}
+template <>
+__device__ inline bf16_t from_f32<bf16_t>(float x) {
+  uint32_t u = __builtin_bit_cast(uint32_t, x);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return bf16_t{(uint16_t)0x7fc0};  // NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return bf16_t{(uint16_t)(u >> 16)};
+}
+
+// off[] are BYTE offsets of elements, unsigned, so that a load from a wave-uniform
+// plane pointer compiles to "scalar base + 32-bit vector offset".
 template <int NCORN>
 struct PairTap {
   unsigned off[NCORN];
   float wt[NCORN];
 };
 
-__device__ inline float load_at(const float *plane, unsigned byte_off) {
-  return *reinterpret_cast<const float *>(reinterpret_cast<const char *>(plane) + byte_off);
+template <typename TD>
+__device__ inline float load_at(const TD *plane, unsigned byte_off) {
+  return to_f32(*reinterpret_cast<const TD *>(reinterpret_cast<const char *>(plane) + byte_off));
 }
 
 // NCORN == 1: nearest.  NCORN == 4: bilinear (wrap == false) or bispherical (wrap == true).
-template <int NCORN>
+// ESZ: bytes per data element.
+template <int NCORN, int ESZ>
 __device__ inline void resolve_pairs(float x, float y, int h, int w, bool wrap, float scale,
                                      PairTap<NCORN> &t) {
   if (NCORN == 1) {
     const int xi = to_int(round_half_away(x));
     const int yi = to_int(round_half_away(y));
     const bool ok = xi >= 0 && xi <= w - 1 && yi >= 0 && yi <= h - 1;
-    t.off[0] = ok ? (unsigned)(yi * w + xi) * 4u : 0u;
+    t.off[0] = ok ? (unsigned)(yi * w + xi) * (unsigned)ESZ : 0u;
     t.wt[0] = ok ? scale : 0.f;
   } else {
     const float x1f = floorf(x), y1f = floorf(y);
@@ -53,7 +76,7 @@ __device__ inline void resolve_pairs(float x, float y, int h, int w, bool wrap, 
     const float wv[4] = {A * B, A * C, D * B, D * C};
 #pragma unroll
     for (int i = 0; i < NCORN; i++) {
-      t.off[i] = ok[i] ? (unsigned)o[i] * 4u : 0u;
+      t.off[i] = ok[i] ? (unsigned)o[i] * (unsigned)ESZ : 0u;
       t.wt[i] = ok[i] ? wv[i] * scale : 0.f;
     }
   }

@@ -226,6 +226,73 @@ def test_conv_medium_fp32_vs_oracle(interp, device):
         assert rel_err(a, r) < 1e-5, nm
 
 
+# ------------------------------------------------------------------ bf16 storage
+@pytest.mark.parametrize("interp", [0, 1, 2])
+@pytest.mark.parametrize("p", [0, 4])
+def test_conv_bf16_vs_fp32_oracle(interp, p, device):
+    """bf16 data / weights (fp32 maps, fp32 accumulation) against the fp32 oracle fed
+    the same bf16-rounded values: within 2e-2 of the result's magnitude."""
+    g = torch.Generator().manual_seed(700 + interp + 10 * p)
+    B, Ci, Co, IH, IW, OH, OW, K = 2, 24, 40, 20, 36, 12, 40, 5
+    bf = lambda t: t.to(torch.bfloat16)
+    x = bf(torch.randn(B, Ci, IH, IW, generator=g))
+    smap, wts = helpers.random_map(g, OH, OW, K, p, IH, IW, torch.float32)
+    w = bf(torch.randn(Co, Ci, K, generator=g) / 8)
+    b = bf(torch.randn(Co, generator=g))
+    gy = bf(torch.randn(B, Co, OH, OW, generator=g))
+    y_o = O.weighted_mapped_conv_forward(x.float(), smap, wts, w.float(), b.float(), K, interp)
+    g_o = O.weighted_mapped_conv_backward(gy.float(), smap, wts, x.float(), w.float(), b.float(),
+                                          K, interp)
+    xd, sd, wd_, wgt, bd, gyd = dev(x, smap, wts, w, b, gy)
+    if p:
+        y = _C.weighted_mapped_conv_forward(xd, sd, wd_, wgt, bd, K, interp)
+        gr = _C.weighted_mapped_conv_backward(gyd, sd, wd_, xd, wgt, bd, K, interp)
+    else:
+        y = _C.mapped_conv_forward(xd, sd, wgt, bd, K, interp)
+        gr = _C.mapped_conv_backward(gyd, sd, xd, wgt, bd, K, interp)
+    assert y.dtype == torch.bfloat16 and all(t.dtype == torch.bfloat16 for t in gr)
+    assert rel_err(y.float(), y_o) < 2e-2
+    for a, r, nm in zip(gr, g_o, ("grad_input", "grad_weight", "grad_bias")):
+        assert rel_err(a.float(), r) < 2e-2, nm
+
+
+def test_transposed_conv_bf16(device):
+    g = torch.Generator().manual_seed(720)
+    B, Ci, Co, IH, IW, OH, OW, K = 2, 16, 24, 10, 33, 14, 40, 4
+    bf = lambda t: t.to(torch.bfloat16)
+    x = bf(torch.randn(B, Ci, IH, IW, generator=g))
+    smap, _ = helpers.random_map(g, IH, IW, K, 0, OH, OW, torch.float32)
+    w = bf(torch.randn(Ci, Co, K, generator=g) / 8)
+    b = bf(torch.randn(Co, generator=g))
+    gy = bf(torch.randn(B, Co, OH, OW, generator=g))
+    y_o = O.mapped_transposed_conv_forward(x.float(), smap, w.float(), b.float(), OH, OW, K, 1)
+    g_o = O.mapped_transposed_conv_backward(gy.float(), smap, x.float(), w.float(), b.float(), K, 1)
+    xd, sd, wgt, bd, gyd = dev(x, smap, w, b, gy)
+    y = _C.mapped_transposed_conv_forward(xd, sd, wgt, bd, OH, OW, K, 1)
+    gr = _C.mapped_transposed_conv_backward(gyd, sd, xd, wgt, bd, K, 1)
+    assert rel_err(y.float(), y_o) < 2e-2
+    for a, r, nm in zip(gr, g_o, ("grad_input", "grad_weight", "grad_bias")):
+        assert rel_err(a.float(), r) < 2e-2, nm
+
+
+def test_conv_bf16_latitude_map_uses_both_backward_paths(device):
+    """Latitude map (transposed-map gather path of the input gradient) in bf16."""
+    torch.manual_seed(5)
+    B, C, H, W = 2, 32, 32, 64
+    bf = lambda t: t.to(torch.bfloat16)
+    x, gy = bf(torch.randn(B, C, H, W)), bf(torch.randn(B, C, H, W))
+    w, b = bf(torch.randn(C, C, 9) / 17), bf(torch.randn(C))
+    smap = synthetic.latitude_map(H, W, 1)
+    y_o = O.mapped_conv_forward(x.float(), smap, w.float(), b.float(), 9, 1)
+    g_o = O.mapped_conv_backward(gy.float(), smap, x.float(), w.float(), b.float(), 9, 1)
+    xd, sd, wd_, bd, gyd = dev(x, smap, w, b, gy)
+    y = _C.mapped_conv_forward(xd, sd, wd_, bd, 9, 1)
+    gr = _C.mapped_conv_backward(gyd, sd, xd, wd_, bd, 9, 1)
+    assert rel_err(y.float(), y_o) < 2e-2
+    for a, r, nm in zip(gr, g_o, ("grad_input", "grad_weight", "grad_bias")):
+        assert rel_err(a.float(), r) < 2e-2, nm
+
+
 # ----------------------------------------------------- size-independent properties
 @pytest.mark.parametrize("interp", [0, 1])
 def test_identity_map_equals_conv2d_large(interp, device):
