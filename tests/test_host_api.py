@@ -35,8 +35,13 @@ def test_library_exports_every_declared_symbol():
 def test_rejected_arguments_return_codes_without_a_gpu():
     lib = _lib.load()
     # NULL pointers / bad sizes are rejected before any launch
-    assert lib.mcx_conv_forward(None, None, None, None, None, None, 1, 1, 1, 4, 4, 4, 4, 1, 0, 1,
-                                0, None) == -3
+    assert lib.mcx_conv_forward(None, None, None, None, None, None, None, 0, 1, 1, 1, 4, 4, 4, 4,
+                                1, 0, 1, 0, None) == -3
+    # a matrix-core path without its scratch buffer is refused, not run
+    assert lib.mcx_conv_forward(1, 1, None, 1, 1, 1, None, 0, 1, 1, 1, 4, 4, 4, 4, 1, 0, 1, 0,
+                                None) == -4
+    assert lib.mcx_conv_forward_workspace(1, 64, 64, 8, 8, 8, 8, 9, 0, 0) > 0
+    assert lib.mcx_conv_forward_workspace(1, 64, 64, 8, 8, 8, 8, 9, 0, 1) == 0  # fp64: scalar kernels
     assert lib.mcx_resample_from_map(1, 1, None, 1, 0, 1, 4, 4, 4, 4, 0, 1, 0, None) == -2
     assert lib.mcx_resample_from_map(1, 1, None, 1, 1, 1, 4, 4, 4, 4, 0, 1, 7, None) == -1
     assert lib.mcx_knn(1, 1, 1, 1, 1, 3, 10, 10, 65, 0, None) == -2
