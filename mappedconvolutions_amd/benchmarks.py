@@ -1,0 +1,139 @@
+"""Secondary workloads of the mapped-convolution hot path, timed on one GPU.
+
+    python -m mappedconvolutions_amd.benchmarks [name ...]
+
+Each workload is one of the reference configurations other than the headline one
+(which `bench.py` at the repository root measures): the weighted mesh convolution,
+the cube-to-equirectangular resampling with pooling, KNN, and the encoder-scale
+bf16 convolution.  For every op the script prints one JSON line with the time per
+call (events on the launch stream, inputs resident in HBM), the algorithmic bytes
+or flops of the call and the fraction of the MI355X roofline that bounds it.
+"""
+import json
+import sys
+
+import torch
+
+from . import _C
+from .util import synthetic
+
+HBM_GBS = 8000.0
+FP32_MFMA_TFLOPS = 157.3
+FP32_VALU_TFLOPS = 157.3  # vector fp32 FMA peak (packed); KNN is bound by it
+
+
+def _time(fn, iters=10, warmup=2):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / iters
+
+
+def _line(name, ms, nbytes=None, flops=None, peak_tflops=FP32_MFMA_TFLOPS, **extra):
+    out = {"workload": name, "ms": round(ms, 4)}
+    if nbytes is not None:
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        out.update(bound="hbm", algorithmic_MB=round(nbytes / 1e6, 1), achieved_GBs=round(gbs, 1),
+                   frac=round(gbs / HBM_GBS, 4))
+    if flops is not None:
+        tf = flops / (ms * 1e-3) / 1e12
+        out.update(bound="mfma" if peak_tflops == FP32_MFMA_TFLOPS else "valu",
+                   GFLOP=round(flops / 1e9, 2), achieved_TFLOPs=round(tf, 2),
+                   frac=round(tf / peak_tflops, 4))
+    out.update(extra)
+    print(json.dumps(out), flush=True)
+
+
+def config3(dev):
+    """Weighted mesh convolution: [4, 64, 1, 40962] -> 128 channels, K=7, P=4, nearest."""
+    B, Ci, Co, V, K, P = 4, 64, 128, 40962, 7, 4
+    smap, iw = synthetic.mesh_weighted_map(V, K, P)
+    smap, iw = smap.to(dev), iw.to(dev)
+    g = torch.Generator().manual_seed(0)
+    for dtype in (torch.float32, torch.bfloat16):
+        x = torch.randn(B, Ci, 1, V, generator=g).to(dev, dtype)
+        w = (torch.randn(Co, Ci, K, generator=g) / (Ci * K) ** 0.5).to(dev, dtype)
+        b = torch.zeros(Co, device=dev, dtype=dtype)
+        gy = torch.randn(B, Co, 1, V, generator=g).to(dev, dtype)
+        flop = 2.0 * B * V * Co * Ci * K
+        tag = "config3 weighted mesh conv %s" % str(dtype).split(".")[-1]
+        _line(tag + " forward",
+              _time(lambda: _C.weighted_mapped_conv_forward(x, smap, iw, w, b, K, 0)), flops=flop)
+        _line(tag + " backward",
+              _time(lambda: _C.weighted_mapped_conv_backward(gy, smap, iw, x, w, b, K, 0)),
+              flops=2 * flop)
+
+
+def config4(dev):
+    """Cube -> equirect resampling (scatter + gather), pools, unpools on 512x1024."""
+    B, C, F, H, W = 4, 64, 256, 512, 1024
+    g = torch.Generator().manual_seed(0)
+    cube = torch.rand(B, C, F, 6 * F, generator=g).to(dev)
+    cmap = synthetic.cube_to_equirect_map(F, H, W).to(dev)
+    eq = torch.rand(B, C, H, W, generator=g).to(dev)
+    lmap = synthetic.latitude_map(H, W, 1).to(dev)
+    fb = 4
+    n_cube, n_eq = cube.numel() * fb, eq.numel() * fb
+    for name, code in (("bilinear", 1), ("bispherical", 2)):
+        _line("config4 resample_to_map %s" % name,
+              _time(lambda: _C.resample_to_map(cube, cmap, H, W, code)),
+              nbytes=n_cube + n_eq + cmap.numel() * fb)
+        _line("config4 resample_from_map %s (Unresample forward)" % name,
+              _time(lambda: _C.resample_from_map(eq, cmap, code)),
+              nbytes=n_cube + n_eq + cmap.numel() * fb)
+    mbytes = lmap.numel() * fb
+    _line("config4 mapped_avg_pool K9", _time(lambda: _C.mapped_avg_pool(eq, lmap, 9, 1)),
+          nbytes=2 * n_eq + mbytes)
+    _line("config4 mapped_max_pool K9", _time(lambda: _C.mapped_max_pool(eq, lmap, 9, 1)),
+          nbytes=2 * n_eq + 2 * n_eq + mbytes)
+    pooled, idx = _C.mapped_max_pool(eq, lmap, 9, 1)
+    _line("config4 mapped_avg_unpool K9",
+          _time(lambda: _C.mapped_avg_unpool(eq, lmap, H, W, 9, 1)), nbytes=2 * n_eq + mbytes)
+    _line("config4 mapped_max_unpool K9",
+          _time(lambda: _C.mapped_max_unpool(eq, idx, lmap, H, W, 9, 1)),
+          nbytes=2 * n_eq + 2 * n_eq + mbytes)
+
+
+def knn(dev):
+    """k=8 nearest of 40962 reference points for 524288 queries on the unit sphere."""
+    ref = synthetic.sphere_points(40962, seed=1).to(dev)
+    qry = synthetic.sphere_points(524288, seed=2).to(dev)
+    _line("config4 knn k=8 Q=524288 R=40962", _time(lambda: _C.knn_forward(ref, qry, 8), iters=3, warmup=1),
+          flops=8.0 * 524288 * 40962, peak_tflops=FP32_VALU_TFLOPS)
+
+
+def config5(dev):
+    """Encoder-scale convolution, bf16 storage: B=16, 128->128, 512x1024, 5x5 bilinear."""
+    B, C, H, W, K = 16, 128, 512, 1024, 25
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(B, C, H, W, generator=g, dtype=torch.bfloat16).to(dev)
+    gy = torch.randn(B, C, H, W, generator=g, dtype=torch.bfloat16).to(dev)
+    w = (torch.randn(C, C, K, generator=g) / (C * K) ** 0.5).to(dev, torch.bfloat16)
+    b = torch.zeros(C, device=dev, dtype=torch.bfloat16)
+    smap = synthetic.latitude_map(H, W, 2).to(dev)
+    flop = 2.0 * B * H * W * C * C * K
+    _line("config5 bf16 conv forward (fp32 MFMA accumulate)",
+          _time(lambda: _C.mapped_conv_forward(x, smap, w, b, K, 1), iters=3, warmup=1), flops=flop)
+    _line("config5 bf16 conv backward (fp32 MFMA accumulate)",
+          _time(lambda: _C.mapped_conv_backward(gy, smap, x, w, b, K, 1), iters=3, warmup=1),
+          flops=2 * flop)
+
+
+WORKLOADS = {"config3": config3, "config4": config4, "knn": knn, "config5": config5}
+
+
+def main(argv):
+    names = argv or list(WORKLOADS)
+    dev = torch.device("cuda:0")
+    for n in names:
+        WORKLOADS[n](dev)
+
+
+if __name__ == "__main__":
+    main(sys.argv[1:])

@@ -23,6 +23,7 @@ constexpr int kTilePx = 128;  // output pixels per workgroup
 constexpr int kGC = 16;       // source channels per reduction chunk
 constexpr int kOT = 64;       // output channels per workgroup
 constexpr int kWtLd = kOT + 4;
+constexpr int kTapCache = 12;  // cached (offset, weight) pairs per tile pixel (12 KB of LDS)
 
 // Workgroups are dealt round-robin to the 8 XCDs; give every XCD one contiguous
 // run of tiles so that neighbouring tiles (which share source rows) share an L2.
@@ -50,15 +51,18 @@ __global__ void pack_weights_kernel(const TD *__restrict__ w, float *__restrict_
 }
 
 template <typename TD, int NCORN, int NP>
-__global__ __launch_bounds__(kThreads, 2) void gather_product_mfma_kernel(
+__global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
     const TD *__restrict__ src, const float *__restrict__ map, const float *__restrict__ iw,
     const float *__restrict__ wp, const TD *__restrict__ bias, TD *__restrict__ y, int G,
     int O, int Opad, int Gpad, int SH, int SW, int OH, int OW, int K, int weighted, int wrap,
     int tiles_x, int tiles_per_img, int tw_shift, const int *__restrict__ gate, int run_if_zero) {
+  constexpr int NE = NP * NCORN;         // (offset, weight) pairs per pixel and tap
+  constexpr int TG = kTapCache / NE > 0 ? kTapCache / NE : 1;  // taps cached in LDS at a time
   __shared__ __attribute__((aligned(16))) float S[2][kGC][kTilePx];
-  if (gate && ((*gate == 0) != (run_if_zero != 0))) return;  // device-side path selection
-
   __shared__ __attribute__((aligned(16))) float Wt[2][kGC][kWtLd];
+  __shared__ __attribute__((aligned(16))) unsigned TapOff[TG][kTilePx][NE];
+  __shared__ __attribute__((aligned(16))) float TapWt[TG][kTilePx][NE];
+  if (gate && ((*gate == 0) != (run_if_zero != 0))) return;  // device-side path selection
 
   const int tid = threadIdx.x;
   const int tile = xcd_contiguous_tile(blockIdx.x, gridDim.x);
@@ -80,28 +84,19 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_mfma_kernel(
 
   const TD *src_b = src + (int64_t)b * G * plane;
   const int chunks = Gpad / kGC;
-  const int iters = K * chunks;
 
-  PairTap<NCORN> taps[NP];
-  float mx[NP], my[NP], mw[NP];
-  float v[8][NP * NCORN];
+  unsigned off[NE];
+  float wt[NE];
+  float v[8][NE];
   float4 wv;
   const int w_off = (tid >> 4) * Opad + (tid & 15) * 4;
 
-  auto load_map = [&](int k) {
+  auto load_tap = [&](int kl) {  // cached pairs of tap kl of the group -> registers
 #pragma unroll
-    for (int sp = 0; sp < NP; sp++) {
-      const int64_t e = (n_g * K + k) * NP + sp;
-      mx[sp] = map[e * 2];
-      my[sp] = map[e * 2 + 1];
-      mw[sp] = weighted ? iw[e] : 1.f;
+    for (int i = 0; i < NE; i++) {
+      off[i] = TapOff[kl][p][i];
+      wt[i] = TapWt[kl][p][i];
     }
-  };
-  auto resolve = [&]() {
-#pragma unroll
-    for (int sp = 0; sp < NP; sp++)
-      resolve_pairs<NCORN, sizeof(TD)>(mx[sp], my[sp], SH, SW, wrap != 0, live ? mw[sp] : 0.f,
-                                       taps[sp]);
   };
   auto issue = [&](int k, int c) {
     const int g0 = c * kGC + half * 8;
@@ -110,9 +105,7 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_mfma_kernel(
       const int g = min(g0 + ch, G - 1);  // padded channels read a valid plane, weights are 0
       const TD *pl = src_b + (int64_t)g * plane;
 #pragma unroll
-      for (int sp = 0; sp < NP; sp++)
-#pragma unroll
-        for (int i = 0; i < NCORN; i++) v[ch][sp * NCORN + i] = load_at(pl, taps[sp].off[i]);
+      for (int i = 0; i < NE; i++) v[ch][i] = load_at(pl, off[i]);
     }
     // weights of this chunk: 16 rows x 64 floats, one float4 per thread
     const float *wchunk = wp + ((int64_t)k * Gpad + c * kGC) * Opad + o0;  // uniform
@@ -123,10 +116,7 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_mfma_kernel(
     for (int ch = 0; ch < 8; ch++) {
       float acc = 0.f;
 #pragma unroll
-      for (int sp = 0; sp < NP; sp++)
-#pragma unroll
-        for (int i = 0; i < NCORN; i++)
-          acc = __builtin_fmaf(taps[sp].wt[i], v[ch][sp * NCORN + i], acc);
+      for (int i = 0; i < NE; i++) acc = __builtin_fmaf(wt[i], v[ch][i], acc);
       S[buf][half * 8 + ch][p] = acc;
     }
     const int cc = tid >> 4, o4 = (tid & 15) * 4;
@@ -137,38 +127,60 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_mfma_kernel(
   const int lane = tid & 63, wave = tid >> 6;
   const int l31 = lane & 31, lhi = lane >> 5;
 
-  load_map(0);
-  resolve();
-  if (K > 1) load_map(1);
-  issue(0, 0);
-  int k = 0, c = 0;
-  for (int it = 0; it < iters; ++it) {
-    const int buf = it & 1;
-    stage(buf);
-    __syncthreads();
-    // advance to the next (tap, chunk) and put its loads in flight
-    if (++c == chunks) {
-      c = 0;
-      ++k;
-      if (k < K) {
-        resolve();  // from the map values fetched one tap ahead
-        if (k + 1 < K) load_map(k + 1);
+  int buf = 0;
+  for (int k0 = 0; k0 < K; k0 += TG) {  // tap groups
+    const int kn = min(TG, K - k0);
+    // Resolve the group's taps once per tile into LDS: thread (p, half) takes every
+    // other tap of pixel p.  All channel chunks reuse them.
+    __syncthreads();  // the previous group's units are done with the cache and with S/Wt
+    for (int kl = half; kl < kn; kl += 2) {
+#pragma unroll
+      for (int sp = 0; sp < NP; sp++) {
+        const int64_t e = (n_g * K + k0 + kl) * NP + sp;
+        PairTap<NCORN> t;
+        resolve_pairs<NCORN, sizeof(TD)>(map[e * 2], map[e * 2 + 1], SH, SW, wrap != 0,
+                                         live ? (weighted ? iw[e] : 1.f) : 0.f, t);
+#pragma unroll
+        for (int i = 0; i < NCORN; i++) {
+          TapOff[kl][p][sp * NCORN + i] = t.off[i];
+          TapWt[kl][p][sp * NCORN + i] = t.wt[i];
+        }
       }
     }
-    if (it + 1 < iters) issue(k, c);
-    // fetch every operand of the chunk first, then issue the MFMAs back to back
-    float bv[kGC / 2], a0[kGC / 2], a1[kGC / 2];
+    __syncthreads();
+
+    // Units run chunk-major with the tap fastest: the source rows a 16-channel chunk
+    // touches are reused by all taps of the group while they are still in cache.
+    const int units = chunks * kn;
+    load_tap(0);
+    issue(k0, 0);
+    int kl = 0, c = 0;
+    for (int u = 0; u < units; ++u) {
+      stage(buf);
+      __syncthreads();
+      if (++kl == kn) {
+        kl = 0;
+        ++c;
+      }
+      if (u + 1 < units) {  // next unit's taps and gathers in flight during the MFMAs
+        load_tap(kl);
+        issue(k0 + kl, c);
+      }
+      // fetch every operand of the chunk first, then issue the MFMAs back to back
+      float bv[kGC / 2], a0[kGC / 2], a1[kGC / 2];
 #pragma unroll
-    for (int s = 0; s < kGC / 2; s++) {
-      const int kk = 2 * s + lhi;
-      bv[s] = S[buf][kk][wave * 32 + l31];
-      a0[s] = Wt[buf][kk][l31];
-      a1[s] = Wt[buf][kk][32 + l31];
-    }
+      for (int s = 0; s < kGC / 2; s++) {
+        const int kk = 2 * s + lhi;
+        bv[s] = S[buf][kk][wave * 32 + l31];
+        a0[s] = Wt[buf][kk][l31];
+        a1[s] = Wt[buf][kk][32 + l31];
+      }
 #pragma unroll
-    for (int s = 0; s < kGC / 2; s++) {
-      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[s], bv[s], acc0, 0, 0, 0);
-      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[s], bv[s], acc1, 0, 0, 0);
+      for (int s = 0; s < kGC / 2; s++) {
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[s], bv[s], acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[s], bv[s], acc1, 0, 0, 0);
+      }
+      buf ^= 1;
     }
   }
 
