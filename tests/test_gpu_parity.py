@@ -293,6 +293,104 @@ def test_conv_bf16_latitude_map_uses_both_backward_paths(device):
         assert rel_err(a.float(), r) < 2e-2, nm
 
 
+# ------------------------------------------------- BASELINE configs 3, 4, 5 (scaled)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_config3_weighted_mesh_conv(dtype, device):
+    """Weighted conv on a mesh signal [B, C, 1, V]: K=7 taps x P=4 random vertices,
+    Dirichlet weights, nearest.  V and channels scaled so the oracle runs in seconds."""
+    B, Ci, Co, V, K, P = 2, 64, 128, 4098, 7, 4
+    smap, iw = synthetic.mesh_weighted_map(V, K, P, seed=3)
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(B, Ci, 1, V, generator=g).to(dtype)
+    w = (torch.randn(Co, Ci, K, generator=g) / (Ci * K) ** 0.5).to(dtype)
+    b = torch.randn(Co, generator=g).to(dtype)
+    gy = torch.randn(B, Co, 1, V, generator=g).to(dtype)
+    y_o = O.weighted_mapped_conv_forward(x.float(), smap, iw, w.float(), b.float(), K, 0)
+    g_o = O.weighted_mapped_conv_backward(gy.float(), smap, iw, x.float(), w.float(), b.float(),
+                                          K, 0)
+    xd, sd, id_, wd_, bd, gyd = dev(x, smap, iw, w, b, gy)
+    y = _C.weighted_mapped_conv_forward(xd, sd, id_, wd_, bd, K, 0)
+    gr = _C.weighted_mapped_conv_backward(gyd, sd, id_, xd, wd_, bd, K, 0)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    assert rel_err(y.float(), y_o) < tol
+    for a, r, nm in zip(gr, g_o, ("grad_input", "grad_weight", "grad_bias")):
+        assert rel_err(a.float(), r) < tol, nm
+
+
+@pytest.mark.parametrize("interp", [1, 2])
+def test_config4_cube_resample_and_pools(interp, device):
+    """Cube map [B, C, F, 6F] -> equirect [2F, 4F] through the exact gnomonic map:
+    resample_to_map (scatter), its adjoint gather, then mapped max / avg pooling with
+    the latitude map on the equirect image.  F scaled to 32."""
+    B, C, F = 2, 8, 32
+    H, W = 2 * F, 4 * F
+    g = torch.Generator().manual_seed(4)
+    cube = torch.rand(B, C, F, 6 * F, generator=g)
+    cmap = synthetic.cube_to_equirect_map(F, H, W)
+    eq_o = O.resample_to_map(cube, cmap, H, W, interp)
+    eq = _C.resample_to_map(cube.cuda(), cmap.cuda(), H, W, interp)
+    assert rel_err(eq, eq_o) < 1e-5
+    back_o = O.resample_from_map(eq_o, cmap, interp)
+    back = _C.resample_from_map(eq_o.cuda(), cmap.cuda(), interp)
+    assert torch.equal(back.cpu(), back_o)
+    lmap = synthetic.latitude_map(H, W, 1)
+    mo, mi = O.mapped_max_pool(eq_o, lmap, 9, 1)
+    m, i = _C.mapped_max_pool(eq_o.cuda(), lmap.cuda(), 9, 1)
+    assert torch.equal(m.cpu(), mo) and torch.equal(i.cpu(), mi)
+    assert torch.equal(_C.mapped_avg_pool(eq_o.cuda(), lmap.cuda(), 9, 1).cpu(),
+                       O.mapped_avg_pool(eq_o, lmap, 9, 1))
+    gy = torch.randn(B, C, H, W, generator=g)
+    assert rel_err(_C.mapped_max_unpool(gy.cuda(), i, lmap.cuda(), H, W, 9, 1),
+                   O.mapped_max_unpool(gy, mi, lmap, H, W, 9, 1)) < 1e-5
+    assert rel_err(_C.mapped_avg_unpool(gy.cuda(), lmap.cuda(), H, W, 9, 1),
+                   O.mapped_avg_unpool(gy, lmap, H, W, 9, 1)) < 1e-5
+
+
+def test_config5_bf16_5x5(device):
+    """Encoder-scale shape scaled down: 128 -> 128 channels, 5x5 latitude map (K=25),
+    bf16 storage with fp32 accumulation, against the fp32 oracle."""
+    B, C, H, W, K = 1, 128, 16, 64, 25
+    g = torch.Generator().manual_seed(5)
+    bf = lambda t: t.to(torch.bfloat16)
+    x, gy = bf(torch.randn(B, C, H, W, generator=g)), bf(torch.randn(B, C, H, W, generator=g))
+    w = bf(torch.randn(C, C, K, generator=g) / (C * K) ** 0.5)
+    b = bf(torch.randn(C, generator=g))
+    smap = synthetic.latitude_map(H, W, 2)
+    y_o = O.mapped_conv_forward(x.float(), smap, w.float(), b.float(), K, 1)
+    g_o = O.mapped_conv_backward(gy.float(), smap, x.float(), w.float(), b.float(), K, 1)
+    xd, sd, wd_, bd, gyd = dev(x, smap, w, b, gy)
+    y = _C.mapped_conv_forward(xd, sd, wd_, bd, K, 1)
+    gr = _C.mapped_conv_backward(gyd, sd, xd, wd_, bd, K, 1)
+    assert rel_err(y.float(), y_o) < 2e-2
+    for a, r, nm in zip(gr, g_o, ("grad_input", "grad_weight", "grad_bias")):
+        assert rel_err(a.float(), r) < 2e-2, nm
+
+
+def test_headline_shape_properties(device):
+    """B=8, 64->64, 256x512, 3x3 latitude map, fp32, at full size: linearity in the
+    input, adjointness of forward and input gradient, bias gradient = plain sum, and
+    the weight gradient as the derivative of <conv(x), g> along a random direction."""
+    torch.manual_seed(6)
+    B, C, H, W = 8, 64, 256, 512
+    x = torch.randn(B, C, H, W, device=device)
+    gy = torch.randn(B, C, H, W, device=device)
+    w = torch.randn(C, C, 9, device=device) / 24
+    zero = torch.zeros(C, device=device)
+    smap = synthetic.latitude_map(H, W, 1).to(device)
+    for interp in (0, 1):
+        y = _C.mapped_conv_forward(x, smap, w, zero, 9, interp)
+        gx, gw, gb = _C.mapped_conv_backward(gy, smap, x, w, zero, 9, interp)
+        lhs, rhs = (y.double() * gy.double()).sum(), (x.double() * gx.double()).sum()
+        assert abs(lhs - rhs) / abs(lhs) < 1e-5
+        assert rel_err(gb, gy.double().sum((0, 2, 3))) < 1e-5
+        dw = torch.randn_like(w)
+        y2 = _C.mapped_conv_forward(x, smap, dw, zero, 9, interp)  # linear in the weight
+        lhs, rhs = (y2.double() * gy.double()).sum(), (gw.double() * dw.double()).sum()
+        assert abs(lhs - rhs) / abs(lhs) < 1e-4
+        y3 = _C.mapped_conv_forward(2 * x, smap, w, zero, 9, interp)
+        assert rel_err(y3, 2 * y) < 1e-6
+
+
 # ----------------------------------------------------- size-independent properties
 @pytest.mark.parametrize("interp", [0, 1])
 def test_identity_map_equals_conv2d_large(interp, device):
