@@ -56,17 +56,21 @@ def cpu_baseline(interp):
     else:
         from oracle import ops as mod
         kind = "port"
-    times = []
-    for rep in range(4):
+    def once():
         t0 = time.perf_counter()
         mod.mapped_conv_forward(x, smap, w, b, K, interp)
         mod.mapped_conv_backward(gy, smap, x, w, b, K, interp)
-        times.append(time.perf_counter() - t0)
-    t = statistics.median(times[1:])
+        return time.perf_counter() - t0
+
+    warm = once()
+    reps = int(min(40, max(3, 12.0 / max(warm, 1e-3))))  # about 12 s of CPU work
+    times = [once() for _ in range(reps)]
+    t = statistics.median(times)
     return {"value": round(H * W / t / 1e6, 4), "unit": "Mpix/s", "cores": torch.get_num_threads(),
             "kind": kind,
             "sample": "B=1 slice (1 of 8 images; the reference loops over the batch, so cost is "
-                      "linear in B), forward+backward, 1 warm-up + median of 3, %.2f s each" % t}
+                      "linear in B), forward+backward, 1 warm-up + median of %d, %.2f s each"
+                      % (reps, t)}
 
 
 def main():
