@@ -218,13 +218,23 @@ constexpr int kWgKT = 9;            // taps per pass (accumulators in registers)
 constexpr int kLdPx = kTilePx + 4;  // LDS row stride (floats)
 
 template <typename TD, int NCORN, int NP>
-__global__ __launch_bounds__(kThreads, 2) void weight_grad_mfma_kernel(
+__global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad_mfma_kernel(
     const TD *__restrict__ plain, const TD *__restrict__ gath,
     const float *__restrict__ map, const float *__restrict__ iw, float *__restrict__ part, int A,
     int G, int GH, int GW, int MH, int MW, int K, int weighted, int wrap, int tiles_x,
     int tiles_per_img, int tw_shift, int total_tiles, int ranges, int cgroups) {
-  __shared__ __attribute__((aligned(16))) float Pt[kWgA][kLdPx];
+  constexpr int NE = NP * NCORN;  // (offset, weight) pairs per pixel and tap
+  // The plain tile is only needed until each wave has copied its rows into registers;
+  // the same LDS then holds the tile's resolved taps (offsets, then weights).
+  constexpr int kPtFloats = kWgA * kLdPx;
+  constexpr int kTapFloats = 2 * kWgKT * kTilePx * NE;
+  constexpr bool kCacheTaps = kTapFloats <= kPtFloats + 1024;
+  __shared__ __attribute__((aligned(16))) float PtMem[kCacheTaps && kTapFloats > kPtFloats ? kTapFloats : kPtFloats];
   __shared__ __attribute__((aligned(16))) float S[2][kGC][kLdPx];
+  float(*Pt)[kLdPx] = reinterpret_cast<float(*)[kLdPx]>(PtMem);
+  unsigned(*TapOff)[kTilePx][NE] = reinterpret_cast<unsigned(*)[kTilePx][NE]>(PtMem);
+  float(*TapWt)[kTilePx][NE] =
+      reinterpret_cast<float(*)[kTilePx][NE]>(PtMem + kWgKT * kTilePx * NE);
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l15 = lane & 15, lq = lane >> 4;
@@ -312,23 +322,33 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_mfma_kernel(
     const int64_t n_g = live ? (int64_t)gi * MW + gj : 0;
     const TD *gath_b = gath + (int64_t)b * G * gplane;
 
-    PairTap<NCORN> taps[NP];
-    float mx[NP], my[NP], mw[NP];
-    float v[8][NP * NCORN];
-    auto load_map = [&](int k) {
+    unsigned off[NE];
+    float wt[NE];
+    float v[8][NE];
+    auto resolve_tap = [&](int k, unsigned *o, float *w_) {  // tap k of this thread's pixel
 #pragma unroll
       for (int sp = 0; sp < NP; sp++) {
         const int64_t e = (n_g * K + k) * NP + sp;
-        mx[sp] = map[e * 2];
-        my[sp] = map[e * 2 + 1];
-        mw[sp] = weighted ? iw[e] : 1.f;
+        PairTap<NCORN> t;
+        resolve_pairs<NCORN, sizeof(TD)>(map[e * 2], map[e * 2 + 1], GH, GW, wrap != 0,
+                                         live ? (weighted ? iw[e] : 1.f) : 0.f, t);
+#pragma unroll
+        for (int i = 0; i < NCORN; i++) {
+          o[sp * NCORN + i] = t.off[i];
+          w_[sp * NCORN + i] = t.wt[i];
+        }
       }
     };
-    auto resolve = [&]() {
+    auto load_tap = [&](int k) {  // k: tap within this pass
+      if (kCacheTaps) {
 #pragma unroll
-      for (int sp = 0; sp < NP; sp++)
-        resolve_pairs<NCORN, sizeof(TD)>(mx[sp], my[sp], GH, GW, wrap != 0, live ? mw[sp] : 0.f,
-                                         taps[sp]);
+        for (int i = 0; i < NE; i++) {
+          off[i] = TapOff[k][p][i];
+          wt[i] = TapWt[k][p][i];
+        }
+      } else {
+        resolve_tap(k_base + k, off, wt);
+      }
     };
     auto issue = [&](int cb) {
       const int g0 = g_first + cb * kGC + half * 8;
@@ -336,9 +356,7 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_mfma_kernel(
       for (int ch = 0; ch < 8; ch++) {
         const TD *pl = gath_b + (int64_t)min(g0 + ch, G - 1) * gplane;
 #pragma unroll
-        for (int sp = 0; sp < NP; sp++)
-#pragma unroll
-          for (int i = 0; i < NCORN; i++) v[ch][sp * NCORN + i] = load_at(pl, taps[sp].off[i]);
+        for (int i = 0; i < NE; i++) v[ch][i] = load_at(pl, off[i]);
       }
     };
     auto stage = [&](int buf) {
@@ -346,32 +364,47 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_mfma_kernel(
       for (int ch = 0; ch < 8; ch++) {
         float s = 0.f;
 #pragma unroll
-        for (int sp = 0; sp < NP; sp++)
-#pragma unroll
-          for (int i = 0; i < NCORN; i++)
-            s = __builtin_fmaf(taps[sp].wt[i], v[ch][sp * NCORN + i], s);
+        for (int i = 0; i < NE; i++) s = __builtin_fmaf(wt[i], v[ch][i], s);
         S[buf][half * 8 + ch][p] = s;
       }
     };
 
-    load_map(k_base);
-    resolve();
-    if (ktaps > 1) load_map(k_base + 1);
+    if (kCacheTaps) {
+      // every wave has its A operands in registers: reuse the plain tile's LDS for the
+      // resolved taps of this tile (thread (p, half) takes every other tap of pixel p)
+      __syncthreads();
+      for (int k = half; k < ktaps; k += 2) {
+        unsigned o[NE];
+        float w_[NE];
+        resolve_tap(k_base + k, o, w_);
+#pragma unroll
+        for (int i = 0; i < NE; i++) {
+          TapOff[k][p][i] = o[i];
+          TapWt[k][p][i] = w_[i];
+        }
+      }
+      __syncthreads();
+    }
+
+    // Units run channel-block-major with the tap fastest: the rows a 16-channel block
+    // touches are reused by all taps while they are still in cache.
+    load_tap(0);
     issue(0);
+    int buf = 0;
 #pragma unroll
-    for (int k = 0; k < kWgKT; k++) {
-      if (k < ktaps) {
+    for (int cb = 0; cb < kWgCB; cb++) {
 #pragma unroll
-        for (int cb = 0; cb < kWgCB; cb++) {
-          const int buf = (k * kWgCB + cb) & 1;
+      for (int k = 0; k < kWgKT; k++) {
+        if (k < ktaps) {
+          buf ^= 1;
           stage(buf);
           __syncthreads();
-          if (cb + 1 < kWgCB) {
+          if (k + 1 < ktaps) {
+            load_tap(k + 1);
+            issue(cb);
+          } else if (cb + 1 < kWgCB) {
+            load_tap(0);
             issue(cb + 1);
-          } else if (k + 1 < ktaps) {
-            resolve();
-            if (k + 2 < ktaps) load_map(k_base + k + 2);
-            issue(0);
           }
 #pragma unroll
           for (int s4 = 0; s4 < 8; s4++) {
@@ -772,7 +805,7 @@ inline PixelTiling make_tiling(int64_t B, int64_t H, int64_t W) {
 inline int weight_grad_ranges(int64_t total_tiles, int64_t A, int64_t G, int64_t K) {
   const int64_t per_range = ((G + kWgCB * kGC - 1) / (kWgCB * kGC)) * ((A + kWgA - 1) / kWgA) *
                             ((K + kWgKT - 1) / kWgKT);
-  int64_t r = std::max<int64_t>(8, (512 / per_range) / 8 * 8);  // about two workgroups per CU
+  int64_t r = std::max<int64_t>(8, (768 / per_range) / 8 * 8);  // about three workgroups per CU
   return (int)std::min<int64_t>(r, std::max<int64_t>(total_tiles, 1));
 }
 
