@@ -80,6 +80,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--interp", default="bilinear", choices=["bilinear", "nearest"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="before the warm-up, run three plain copy kernels over the input "
+                         "(reads and writes B*Ci*H*W*4 bytes each) so that a counter run of this "
+                         "command holds a dispatch of known traffic to scale FETCH_SIZE/WRITE_SIZE by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
@@ -88,6 +92,13 @@ def main():
     interp = 1 if args.interp == "bilinear" else 0
     dev = torch.device("cuda:0")
     inputs = make_inputs(dev)
+
+    if args.calibration_copy:
+        dst = torch.empty_like(inputs[0])
+        for _ in range(3):
+            torch.mul(inputs[0], 1.0, out=dst)  # one elementwise kernel: 1 read + 1 write per element
+        torch.cuda.synchronize()
+        del dst
 
     for _ in range(args.warmup):
         step(*inputs, interp)
