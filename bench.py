@@ -29,6 +29,21 @@ B, CI, CO, H, W, K = 8, 64, 64, 256, 512, 9
 PEAK_FP32_MFMA_TFLOPS = 157.3
 GEMM_FLOP = 2.0 * B * H * W * CO * CI * K  # one of the three products
 
+# Bytes that cross the L2 boundary per launch (bilinear workload), from FETCH_SIZE and WRITE_SIZE
+# counter passes of this script scaled by a copy kernel of known size (x2.0 KiB and x1.0 KiB per
+# count); profiles/conv_fwd_bwd_headline_hbm_traffic.txt holds the runs.  Counters cannot be read
+# from inside the process, so the figures are the recorded ones; other workloads report null.
+MEASURED_TRAFFIC_BYTES = {
+    "conv_forward": 774.0e6 + 268.4e6,
+    "conv_backward_input": 2052.0e6 + 268.4e6,
+    "conv_backward_weight": 1897.1e6 + 82.8e6,
+}
+KERNEL_OF = {
+    "conv_forward": "gather_product_mfma_kernel<float,4,1>",
+    "conv_backward_input": "gather_product_mfma_kernel<float,1,4>",
+    "conv_backward_weight": "weight_grad_mfma_kernel<float,4,1>",
+}
+
 
 def make_inputs(device, batch=B):
     g = torch.Generator().manual_seed(0)
@@ -130,10 +145,12 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "MappedConvolution fwd+bwd B8 Ci64 Co64 256x512 K9 latitude map, "
                                + args.interp, "interpolation": args.interp},
-        "roofline": {"bound": "mfma", "kernel": dominant,
+        "roofline": {"bound": "mfma", "kernel": KERNEL_OF.get(dominant, dominant) if interp == 1
+                     else dominant,
                      "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
-                     "traffic": None},
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(dominant) if interp == 1 else None,
+                     "traffic_unit": "bytes per launch"},
         "kernel_ms": {k: round(v, 4) for k, v in kernel_ms.items()},
     }
     if not args.no_cpu_baseline:

@@ -35,17 +35,20 @@ _EXT_MODULES = {
 }
 
 
-def install_aliases():
+def install_aliases(ext_only=False):
     """Make `import mapped_convolution.nn` and
-    `import _mapped_convolution_ext._mapped_convolution` resolve to this package."""
-    pkg = types.ModuleType("mapped_convolution")
-    pkg.nn, pkg.util = nn, util
-    pkg.__path__ = []
-    sys.modules.setdefault("mapped_convolution", pkg)
-    sys.modules.setdefault("mapped_convolution.nn", nn)
-    sys.modules.setdefault("mapped_convolution.util", util)
-    sys.modules.setdefault("mapped_convolutions", sys.modules["mapped_convolution"])
-    sys.modules.setdefault("mapped_convolutions.nn", nn)
+    `import _mapped_convolution_ext._mapped_convolution` resolve to this package.
+    With `ext_only` only the extension-module names are registered, for use under
+    the reference's own pure-Python layer files."""
+    if not ext_only:
+        pkg = types.ModuleType("mapped_convolution")
+        pkg.nn, pkg.util = nn, util
+        pkg.__path__ = []
+        sys.modules.setdefault("mapped_convolution", pkg)
+        sys.modules.setdefault("mapped_convolution.nn", nn)
+        sys.modules.setdefault("mapped_convolution.util", util)
+        sys.modules.setdefault("mapped_convolutions", sys.modules["mapped_convolution"])
+        sys.modules.setdefault("mapped_convolutions.nn", nn)
     ext = types.ModuleType("_mapped_convolution_ext")
     ext.__path__ = []
     sys.modules.setdefault("_mapped_convolution_ext", ext)

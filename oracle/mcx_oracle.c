@@ -8,7 +8,7 @@
  * check and the bench's CPU-baseline leg may load the library built from this
  * file; the shipped HIP library never links, loads or falls back to it.
  *
- * How each function is pinned (see tests/test_oracle_*.py):
+ * How each function is pinned (see tests/test_oracle.py):
  *   - interpolators, resample, conv, transposed conv, pools: the reference's
  *     own hand-computed known answers (literals of the files under package/tests, transcribed
  *     as data), the reference's CPU build in oracle/_ref where present, and
