@@ -66,11 +66,17 @@ int mcx_resample_from_map(const void *src, const void *map, const void *iw, void
 /* resample_to_map (+ weighted_resample_to_map):
  * include/nn/layers/resample_layer.h:38-40,83 and weighted_resample_layer.h:49-54;
  * kernels include/nn/cuda/resample.cuh:14-26,85-99.
- * out (cleared here) accumulates every input pixel at map[y_in,x_in];
- * in [B,C,IH,IW], map [IH,IW,(P,)2], out [B,C,OH,OW]. */
+ * out accumulates every input pixel at map[y_in,x_in] (fully written here, the caller need
+ * not clear it); in [B,C,IH,IW], map [IH,IW,(P,)2], out [B,C,OH,OW].
+ * With a workspace of mcx_resample_to_map_workspace() bytes the map is turned around once and
+ * every output is gathered (no float atomics); with workspace == NULL the op scatters with
+ * atomics, as the reference does. */
+size_t mcx_resample_to_map_workspace(int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t P,
+                                     int interp, int dtype);
 int mcx_resample_to_map(const void *in, const void *map, const void *iw, void *out,
-                        int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t OH, int64_t OW,
-                        int64_t P, int interp, int dtype, void *stream);
+                        void *workspace, size_t workspace_bytes, int64_t B, int64_t C, int64_t IH,
+                        int64_t IW, int64_t OH, int64_t OW, int64_t P, int interp, int dtype,
+                        void *stream);
 
 /* ---- Pooling --------------------------------------------------------------- */
 
@@ -84,10 +90,14 @@ int mcx_max_pool(const void *in, const void *map, const void *iw, void *out, int
 
 /* mapped_max_unpool (+ weighted): mapped_max_pooling_layer.h:69-73,103,
  * weighted_mapped_max_pooling_layer.h:67-70; kernels mapped_max_pool.cuh:56-70,144-159.
- * gout, idx [B,C,OH,OW] -> gin [B,C,IH,IW] (cleared here). */
+ * gout, idx [B,C,OH,OW] -> gin [B,C,IH,IW] (fully written here).  Workspace as for
+ * mcx_resample_to_map: mcx_unpool_workspace() bytes select the gather form, NULL the atomics. */
+size_t mcx_unpool_workspace(int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P,
+                            int interp, int dtype);
 int mcx_max_unpool(const void *gout, const int64_t *idx, const void *map, const void *iw,
-                   void *gin, int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t OH,
-                   int64_t OW, int64_t K, int64_t P, int interp, int dtype, void *stream);
+                   void *gin, void *workspace, size_t workspace_bytes, int64_t B, int64_t C,
+                   int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
+                   int dtype, void *stream);
 
 /* mapped_avg_pool (+ weighted): include/nn/layers/mapped_avg_pooling_layer.h:42-44,91-94,
  * weighted_mapped_avg_pooling_layer.h:48-52; kernels include/nn/cuda/mapped_avg_pool.cuh:15-27,91-106. */
@@ -96,10 +106,11 @@ int mcx_avg_pool(const void *in, const void *map, const void *iw, void *out, int
                  int64_t P, int interp, int dtype, void *stream);
 
 /* mapped_avg_unpool (+ weighted): mapped_avg_pooling_layer.h:64-67,
- * weighted_mapped_avg_pooling_layer.h:75-78; kernels mapped_avg_pool.cuh:50-63,131-145. */
-int mcx_avg_unpool(const void *gout, const void *map, const void *iw, void *gin, int64_t B,
-                   int64_t C, int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
-                   int64_t P, int interp, int dtype, void *stream);
+ * weighted_mapped_avg_pooling_layer.h:75-78; kernels mapped_avg_pool.cuh:50-63,131-145.
+ * Workspace: mcx_unpool_workspace() bytes, or NULL for the atomic form. */
+int mcx_avg_unpool(const void *gout, const void *map, const void *iw, void *gin, void *workspace,
+                   size_t workspace_bytes, int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t OH,
+                   int64_t OW, int64_t K, int64_t P, int interp, int dtype, void *stream);
 
 /* ---- Mapped convolution ---------------------------------------------------- */
 

@@ -20,6 +20,10 @@ _DTYPES = {torch.float32: MCX_F32, torch.float64: MCX_F64, torch.bfloat16: MCX_B
 # are enqueued on.  Used by the benchmark to time individual kernels.
 profile_events = None
 
+# resample_to_map and the unpoolings run as gathers through a transposed map when
+# given a workspace; False selects the library's atomic-scatter form instead.
+scatter_as_gather = True
+
 
 def _timed(label, device, fn):
     if profile_events is None:
@@ -306,10 +310,14 @@ def _max_unpool(grad_output, idx_mask, sample_map, interp_weights, input_height,
     B, C, OH, OW = grad_output.shape
     IH, IW = int(input_height), int(input_width)
     gin = torch.empty((B, C, IH, IW), dtype=grad_output.dtype, device=grad_output.device)
+    lib = _lib.load()
+    ws_bytes = lib.mcx_unpool_workspace(IH, IW, OH, OW, K, P, int(interpolation), dt) \
+        if scatter_as_gather else 0
+    ws = _workspace(ws_bytes, grad_output.device)
     with torch.cuda.device(grad_output.device):
-        rc = _lib.load().mcx_max_unpool(_ptr(grad_output), _ptr(idx_mask), _ptr(sample_map),
-                                        _ptr(interp_weights), _ptr(gin), B, C, IH, IW, OH, OW, K,
-                                        P, int(interpolation), dt, _stream(grad_output))
+        rc = lib.mcx_max_unpool(_ptr(grad_output), _ptr(idx_mask), _ptr(sample_map),
+                                _ptr(interp_weights), _ptr(gin), _ptr(ws), ws_bytes, B, C, IH, IW,
+                                OH, OW, K, P, int(interpolation), dt, _stream(grad_output))
     _lib.check(rc, "mapped_max_unpool")
     return gin
 
@@ -341,10 +349,14 @@ def _avg_unpool(grad_output, sample_map, interp_weights, input_height, input_wid
         raise RuntimeError("sample_map spatial size must match grad_output")
     IH, IW = int(input_height), int(input_width)
     gin = torch.empty((B, C, IH, IW), dtype=grad_output.dtype, device=grad_output.device)
+    lib = _lib.load()
+    ws_bytes = lib.mcx_unpool_workspace(IH, IW, OH, OW, K, P, int(interpolation), dt) \
+        if scatter_as_gather else 0
+    ws = _workspace(ws_bytes, grad_output.device)
     with torch.cuda.device(grad_output.device):
-        rc = _lib.load().mcx_avg_unpool(_ptr(grad_output), _ptr(sample_map), _ptr(interp_weights),
-                                        _ptr(gin), B, C, IH, IW, OH, OW, K, P, int(interpolation),
-                                        dt, _stream(grad_output))
+        rc = lib.mcx_avg_unpool(_ptr(grad_output), _ptr(sample_map), _ptr(interp_weights),
+                                _ptr(gin), _ptr(ws), ws_bytes, B, C, IH, IW, OH, OW, K, P,
+                                int(interpolation), dt, _stream(grad_output))
     _lib.check(rc, "mapped_avg_unpool")
     return gin
 
@@ -409,10 +421,14 @@ def _resample_to_map(input, sample_map, interp_weights, output_height, output_wi
         raise RuntimeError("sample_map spatial size must match the input")
     OH, OW = int(output_height), int(output_width)
     out = torch.empty((B, C, OH, OW), dtype=input.dtype, device=input.device)
+    lib = _lib.load()
+    ws_bytes = lib.mcx_resample_to_map_workspace(IH, IW, OH, OW, P, int(interpolation), dt) \
+        if scatter_as_gather else 0
+    ws = _workspace(ws_bytes, input.device)
     with torch.cuda.device(input.device):
-        rc = _lib.load().mcx_resample_to_map(_ptr(input), _ptr(sample_map), _ptr(interp_weights),
-                                             _ptr(out), B, C, IH, IW, OH, OW, P,
-                                             int(interpolation), dt, _stream(input))
+        rc = lib.mcx_resample_to_map(_ptr(input), _ptr(sample_map), _ptr(interp_weights),
+                                     _ptr(out), _ptr(ws), ws_bytes, B, C, IH, IW, OH, OW, P,
+                                     int(interpolation), dt, _stream(input))
     _lib.check(rc, "resample_to_map")
     return out
 

@@ -21,11 +21,13 @@ SIGNATURES = {
     "mcx_abi_version": (_i, []),
     "mcx_error_string": (ctypes.c_char_p, [_i]),
     "mcx_resample_from_map": (_i, [_p] * 4 + [_i64] * 7 + [_i, _i, _p]),
-    "mcx_resample_to_map": (_i, [_p] * 4 + [_i64] * 7 + [_i, _i, _p]),
+    "mcx_resample_to_map_workspace": (_sz, [_i64] * 5 + [_i, _i]),
+    "mcx_resample_to_map": (_i, [_p] * 5 + [_sz] + [_i64] * 7 + [_i, _i, _p]),
     "mcx_max_pool": (_i, [_p] * 5 + [_i64] * 8 + [_i, _i, _p]),
-    "mcx_max_unpool": (_i, [_p] * 5 + [_i64] * 8 + [_i, _i, _p]),
+    "mcx_unpool_workspace": (_sz, [_i64] * 6 + [_i, _i]),
+    "mcx_max_unpool": (_i, [_p] * 6 + [_sz] + [_i64] * 8 + [_i, _i, _p]),
     "mcx_avg_pool": (_i, [_p] * 4 + [_i64] * 8 + [_i, _i, _p]),
-    "mcx_avg_unpool": (_i, [_p] * 4 + [_i64] * 8 + [_i, _i, _p]),
+    "mcx_avg_unpool": (_i, [_p] * 5 + [_sz] + [_i64] * 8 + [_i, _i, _p]),
     "mcx_conv_forward": (_i, [_p] * 7 + [_sz] + [_i64] * 9 + [_i, _i, _p]),
     "mcx_conv_forward_workspace": (_sz, [_i64] * 9 + [_i]),
     "mcx_conv_backward_workspace": (_sz, [_i64] * 9 + [_i]),

@@ -386,7 +386,7 @@ extern "C" int mcx_tconv_backward(const void *gy, const void *map, const void *i
                                                 workspace_bytes, d, interp, s));
 }
 
-extern "C" int mcx_abi_version(void) { return 3; }
+extern "C" int mcx_abi_version(void) { return 4; }
 
 extern "C" const char *mcx_error_string(int code) {
   switch (code) {

@@ -51,6 +51,9 @@ __device__ inline T round_half_away(T v) {
 __device__ inline int to_int(float v) { return (int)fminf(fmaxf(v, -2.0e9f), 2.0e9f); }
 __device__ inline int to_int(double v) { return (int)fmin(fmax(v, -2.0e9), 2.0e9); }
 
+__device__ inline float mcx_fma(float a, float b, float c) { return fmaf(a, b, c); }
+__device__ inline double mcx_fma(double a, double b, double c) { return fma(a, b, c); }
+
 __device__ inline int wrap_index(int v, int n) {
   int r = v % n;
   return r < 0 ? r + n : r;
@@ -88,6 +91,9 @@ struct Tap<T, kInterpNearest> {
   __device__ inline void scatter(T *plane, T v) const {
     if (off >= 0) atomic_add(plane + off, v);
   }
+  static constexpr int kCorners = 1;
+  __device__ inline int corner_off(int) const { return off; }
+  __device__ inline T corner_wt(int) const { return T(1); }
 };
 
 // Bilinear (zero padding on both axes) and bispherical (x wraps, y zero-padded).
@@ -136,6 +142,9 @@ struct Tap {
     for (int i = 0; i < 4; i++)
       if (off[i] >= 0) atomic_add(plane + off[i], wt[i] * v);
   }
+  static constexpr int kCorners = 4;
+  __device__ inline int corner_off(int i) const { return off[i]; }
+  __device__ inline T corner_wt(int i) const { return wt[i]; }
 };
 
 // ---- launch helpers ---------------------------------------------------------

@@ -162,6 +162,140 @@ __global__ __launch_bounds__(kThreads) void max_unpool_kernel(
   }
 }
 
+
+// ---- scatter ops as gathers through a transposed map -------------------------
+// resample_to_map and the two unpoolings push every source value to the
+// destination pixels its taps touch.  The map is shared by all B*C planes, so it
+// pays to turn it around once per call: a compressed list, per destination pixel,
+// of the (source location, weight) pairs that land on it (count -> prefix sum ->
+// fill), after which every destination element is a plain weighted gather: no
+// float atomics, no zero fill, each output written once.  Contributions whose
+// weight is exactly zero are left out (they add 0 to any finite value).
+constexpr int kScanItems = 8;                      // counts per thread of the block scan
+constexpr int kScanBlock = kThreads * kScanItems;  // counts per block
+
+enum { UN_RESAMPLE = 0, UN_AVG = 1, UN_MAX = 2 };
+
+// One thread per map sample i = (n*K + k)*Pm + p.  FILL == false counts the
+// contributions of each destination pixel; FILL == true writes them to their place.
+template <typename T, int MODE, bool FILL>
+__global__ __launch_bounds__(kThreads) void transposed_map_kernel(
+    const T *__restrict__ map, const T *__restrict__ iw, int64_t samples, int per_code, int DH,
+    int DW, uint32_t *__restrict__ local, uint32_t *__restrict__ cursor,
+    const uint32_t *__restrict__ bsum, uint32_t *__restrict__ e_src, T *__restrict__ e_wt) {
+  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i >= samples) return;
+  Tap<T, MODE> tap;
+  tap.set(map[i * 2], map[i * 2 + 1], DH, DW);
+  const T w = iw ? iw[i] : T(1);
+  const uint32_t code = (uint32_t)(i / per_code);
+#pragma unroll
+  for (int c = 0; c < Tap<T, MODE>::kCorners; c++) {
+    const int off = tap.corner_off(c);
+    const T ww = iw ? tap.corner_wt(c) * w : tap.corner_wt(c);
+    if (off < 0 || ww == T(0)) continue;
+    if (!FILL) {
+      atomicAdd(&local[off], 1u);
+    } else {
+      const uint32_t pos = local[off] + bsum[off / kScanBlock] + atomicAdd(&cursor[off], 1u);
+      e_src[pos] = code;
+      e_wt[pos] = ww;
+    }
+  }
+}
+
+// Exclusive prefix sum of counts, two levels: within blocks of kScanBlock (in
+// place), then over the block totals (one workgroup).  The prefix of element i is
+// local[i] + bsum[i / kScanBlock].
+__global__ __launch_bounds__(kThreads) void scan_blocks_kernel(uint32_t *__restrict__ local,
+                                                               uint32_t *__restrict__ bsum,
+                                                               int64_t n) {
+  __shared__ uint32_t part[kThreads];
+  const int64_t base = (int64_t)blockIdx.x * kScanBlock + (int64_t)threadIdx.x * kScanItems;
+  uint32_t v[kScanItems], sum = 0;
+#pragma unroll
+  for (int j = 0; j < kScanItems; j++) {
+    v[j] = base + j < n ? local[base + j] : 0u;
+    sum += v[j];
+  }
+  part[threadIdx.x] = sum;
+  __syncthreads();
+  for (int d = 1; d < kThreads; d <<= 1) {
+    const uint32_t add = threadIdx.x >= (unsigned)d ? part[threadIdx.x - d] : 0u;
+    __syncthreads();
+    part[threadIdx.x] += add;
+    __syncthreads();
+  }
+  uint32_t run = part[threadIdx.x] - sum;  // exclusive prefix of this thread
+#pragma unroll
+  for (int j = 0; j < kScanItems; j++) {
+    if (base + j < n) local[base + j] = run;
+    run += v[j];
+  }
+  if (threadIdx.x == kThreads - 1) bsum[blockIdx.x] = part[threadIdx.x];
+}
+
+__global__ __launch_bounds__(kThreads) void scan_sums_kernel(uint32_t *__restrict__ bsum, int n) {
+  __shared__ uint32_t part[kThreads];
+  uint32_t carry = 0;
+  for (int base = 0; base < n; base += kThreads) {
+    const int i = base + (int)threadIdx.x;
+    const uint32_t v = i < n ? bsum[i] : 0u;
+    part[threadIdx.x] = v;
+    __syncthreads();
+    for (int d = 1; d < kThreads; d <<= 1) {
+      const uint32_t add = threadIdx.x >= (unsigned)d ? part[threadIdx.x - d] : 0u;
+      __syncthreads();
+      part[threadIdx.x] += add;
+      __syncthreads();
+    }
+    if (i < n) bsum[i] = carry + part[threadIdx.x] - v;
+    carry += part[kThreads - 1];
+    __syncthreads();
+  }
+}
+
+// One thread per destination pixel and kCH planes.  UN_MAX keeps a contribution
+// only where the recorded winner of that source element is this tap.
+template <typename T, int OP>
+__global__ __launch_bounds__(kThreads) void transposed_gather_kernel(
+    const T *__restrict__ src, const int64_t *__restrict__ idx, T *__restrict__ dst,
+    const uint32_t *__restrict__ local, const uint32_t *__restrict__ bsum,
+    const uint32_t *__restrict__ e_src, const T *__restrict__ e_wt, int64_t planes, int nsrc,
+    int ndst, int K, int idx_scale, int groups) {
+  const int pg = blockIdx.x % groups;
+  const int p = (blockIdx.x / groups) * kThreads + threadIdx.x;
+  if (p >= ndst) return;
+  const int64_t plane0 = (int64_t)pg * kCH;
+  const int nc = (int)min((int64_t)kCH, planes - plane0);
+  const uint32_t start = local[p] + bsum[p / kScanBlock];
+  const uint32_t end = local[p + 1] + bsum[(p + 1) / kScanBlock];
+  const T *s0 = src + plane0 * nsrc;
+  const int64_t *i0 = OP == UN_MAX ? idx + plane0 * nsrc : nullptr;
+  T acc[kCH];
+#pragma unroll
+  for (int c = 0; c < kCH; c++) acc[c] = T(0);
+  for (uint32_t e = start; e < end; e++) {
+    const uint32_t code = e_src[e];
+    const T w = e_wt[e];
+    const uint32_t n = OP == UN_MAX ? code / (uint32_t)K : code;
+    const int64_t want = (int64_t)code * idx_scale;
+#pragma unroll
+    for (int c = 0; c < kCH; c++) {
+      if (c >= nc) continue;
+      if (OP == UN_MAX) {
+        if (i0[(int64_t)c * nsrc + n] == want) acc[c] = mcx_fma(w, s0[(int64_t)c * nsrc + n], acc[c]);
+      } else {
+        acc[c] = mcx_fma(w, s0[(int64_t)c * nsrc + n], acc[c]);
+      }
+    }
+  }
+  T *d0 = dst + plane0 * ndst + p;
+#pragma unroll
+  for (int c = 0; c < kCH; c++)
+    if (c < nc) d0[(int64_t)c * ndst] = OP == UN_AVG ? acc[c] / (T)K : acc[c];
+}
+
 bool bad_dims(std::initializer_list<int64_t> dims) {
   for (int64_t d : dims)
     if (d <= 0 || d > 0x7fffffffLL) return true;
@@ -186,6 +320,80 @@ int launch_gather(const void *in, const void *map, const void *iw, void *out, in
                                                0, s, (const T *)in, (const T *)map,
                                                (const T *)iw, (T *)out, idx, (int)C, (int)IH,
                                                (int)IW, (int)N, (int)K, (int)P));
+  MCX_HIP_CHECK_LAUNCH();
+  return 0;
+}
+
+
+// Workspace of the transposed-map form.  `samples` = source locations x taps x
+// points; every sample can land on `corners` destination pixels.
+struct TransposedLayout {
+  size_t local, cursor, bsum, e_src, e_wt, total;
+  int nblocks;
+  bool ok;
+};
+
+inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+TransposedLayout transposed_layout(int64_t ndst, int64_t samples, int corners, size_t elem) {
+  TransposedLayout l{};
+  const int64_t cap = samples * corners;
+  l.ok = ndst > 0 && samples > 0 && cap <= 0x7fffffffLL && ndst < 0x7fffffffLL;
+  if (!l.ok) return l;
+  l.nblocks = (int)((ndst + 1 + kScanBlock - 1) / kScanBlock);
+  size_t off = 0;
+  l.local = off;  off += align256((size_t)(ndst + 1) * 4);
+  l.cursor = off; off += align256((size_t)ndst * 4);
+  l.bsum = off;   off += align256((size_t)l.nblocks * 4);
+  l.e_src = off;  off += align256((size_t)cap * 4);
+  l.e_wt = off;   off += align256((size_t)cap * elem);
+  l.total = off;
+  return l;
+}
+
+inline int corners_of(int interp) { return canonical_interp(interp) == kInterpNearest ? 1 : 4; }
+
+// Returns -1000 when the form does not apply (no or short workspace, sizes beyond
+// 32-bit entry indices): the caller then runs the atomic scatter instead.
+constexpr int kNotApplicable = -1000;
+
+template <typename T, int OP>
+int launch_transposed(const void *src, const int64_t *idx, const void *map, const void *iw,
+                      void *dst, void *ws, size_t ws_bytes, int64_t planes, int64_t nsrc,
+                      int64_t K, int64_t P, int64_t DH, int64_t DW, int interp, hipStream_t s) {
+  const int64_t pm = P ? P : 1;
+  const int64_t samples = nsrc * K * pm, ndst = DH * DW;
+  const TransposedLayout l = transposed_layout(ndst, samples, corners_of(interp), sizeof(T));
+  if (!ws || !l.ok || ws_bytes < l.total || nsrc * K > 0xffffffffLL) return kNotApplicable;
+  const int64_t groups = (planes + kCH - 1) / kCH;
+  const int64_t blocks = groups * ((ndst + kThreads - 1) / kThreads);
+  if (blocks > 0x7fffffffLL) return kNotApplicable;
+  char *base = (char *)ws;
+  uint32_t *local = (uint32_t *)(base + l.local), *cursor = (uint32_t *)(base + l.cursor);
+  uint32_t *bsum = (uint32_t *)(base + l.bsum), *e_src = (uint32_t *)(base + l.e_src);
+  T *e_wt = (T *)(base + l.e_wt);
+  int rc = fill<uint32_t>(local, ndst + 1, 0u, s);
+  if (rc) return rc;
+  if ((rc = fill<uint32_t>(cursor, ndst, 0u, s))) return rc;
+  const int per_code = (int)(OP == UN_MAX ? pm : pm * K);
+  const dim3 sgrid(div_up(samples, kThreads)), blk(kThreads);
+  MCX_DISPATCH_MODE(interp, hipLaunchKernelGGL((transposed_map_kernel<T, MODE, false>), sgrid, blk,
+                                               0, s, (const T *)map, (const T *)iw, samples,
+                                               per_code, (int)DH, (int)DW, local, cursor, bsum,
+                                               e_src, e_wt));
+  MCX_HIP_CHECK_LAUNCH();
+  hipLaunchKernelGGL(scan_blocks_kernel, dim3(l.nblocks), blk, 0, s, local, bsum, ndst + 1);
+  MCX_HIP_CHECK_LAUNCH();
+  hipLaunchKernelGGL(scan_sums_kernel, dim3(1), blk, 0, s, bsum, l.nblocks);
+  MCX_HIP_CHECK_LAUNCH();
+  MCX_DISPATCH_MODE(interp, hipLaunchKernelGGL((transposed_map_kernel<T, MODE, true>), sgrid, blk,
+                                               0, s, (const T *)map, (const T *)iw, samples,
+                                               per_code, (int)DH, (int)DW, local, cursor, bsum,
+                                               e_src, e_wt));
+  MCX_HIP_CHECK_LAUNCH();
+  hipLaunchKernelGGL((transposed_gather_kernel<T, OP>), dim3((unsigned)blocks), blk, 0, s,
+                     (const T *)src, idx, (T *)dst, local, bsum, e_src, e_wt, planes, (int)nsrc,
+                     (int)ndst, (int)K, (int)(pm * 2), (int)groups);
   MCX_HIP_CHECK_LAUNCH();
   return 0;
 }
@@ -238,18 +446,52 @@ extern "C" int mcx_resample_from_map(const void *src, const void *map, const voi
                                             P, interp, s);
 }
 
+namespace {
+template <typename T>
+int resample_to_map_t(const void *in, const void *map, const void *iw, void *out, void *ws,
+                      size_t ws_bytes, int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t OH,
+                      int64_t OW, int64_t P, int interp, hipStream_t s) {
+  const int rc = launch_transposed<T, UN_RESAMPLE>(in, nullptr, map, iw, out, ws, ws_bytes, B * C,
+                                                   IH * IW, 1, P, OH, OW, interp, s);
+  if (rc != kNotApplicable) return rc;
+  return launch_scatter<T, OP_RESAMPLE>(in, map, iw, out, B, C, OH, OW, IH * IW, 1, P, interp, s);
+}
+
+size_t transposed_workspace(int64_t nsrc, int64_t K, int64_t P, int64_t DH, int64_t DW, int interp,
+                            int dtype) {
+  if (dtype != MCX_F32 && dtype != MCX_F64) return 0;
+  if (bad_dims({nsrc, K, DH, DW, DH * DW}) || P < 0) return 0;
+  const TransposedLayout l = transposed_layout(DH * DW, nsrc * K * (P ? P : 1), corners_of(interp),
+                                               dtype == MCX_F32 ? 4 : 8);
+  return l.ok ? l.total : 0;
+}
+}  // namespace
+
+extern "C" size_t mcx_resample_to_map_workspace(int64_t IH, int64_t IW, int64_t OH, int64_t OW,
+                                                int64_t P, int interp, int dtype) {
+  if (bad_dims({IH, IW, IH * IW})) return 0;
+  return transposed_workspace(IH * IW, 1, P, OH, OW, interp, dtype);
+}
+
+extern "C" size_t mcx_unpool_workspace(int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
+                                       int64_t P, int interp, int dtype) {
+  if (bad_dims({OH, OW, OH * OW})) return 0;
+  return transposed_workspace(OH * OW, K, P, IH, IW, interp, dtype);
+}
+
 extern "C" int mcx_resample_to_map(const void *in, const void *map, const void *iw, void *out,
-                                   int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t OH,
-                                   int64_t OW, int64_t P, int interp, int dtype, void *stream) {
+                                   void *workspace, size_t workspace_bytes, int64_t B, int64_t C,
+                                   int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t P,
+                                   int interp, int dtype, void *stream) {
   if (int rc = check_common(in, map, iw, out, P, dtype)) return rc;
   if (bad_dims({B, C, IH, IW, OH, OW, IH * IW, OH * OW, IH * IW * (P ? P : 1) * 2}) || B > 65535)
     return MCX_E_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == MCX_F32)
-    return launch_scatter<float, OP_RESAMPLE>(in, map, iw, out, B, C, OH, OW, IH * IW, 1, P,
-                                              interp, s);
-  return launch_scatter<double, OP_RESAMPLE>(in, map, iw, out, B, C, OH, OW, IH * IW, 1, P, interp,
-                                             s);
+    return resample_to_map_t<float>(in, map, iw, out, workspace, workspace_bytes, B, C, IH, IW, OH,
+                                    OW, P, interp, s);
+  return resample_to_map_t<double>(in, map, iw, out, workspace, workspace_bytes, B, C, IH, IW, OH,
+                                   OW, P, interp, s);
 }
 
 extern "C" int mcx_max_pool(const void *in, const void *map, const void *iw, void *out,
@@ -280,24 +522,41 @@ extern "C" int mcx_avg_pool(const void *in, const void *map, const void *iw, voi
                                        interp, s);
 }
 
+namespace {
+template <typename T>
+int avg_unpool_t(const void *gout, const void *map, const void *iw, void *gin, void *ws,
+                 size_t ws_bytes, int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t OH,
+                 int64_t OW, int64_t K, int64_t P, int interp, hipStream_t s) {
+  const int rc = launch_transposed<T, UN_AVG>(gout, nullptr, map, iw, gin, ws, ws_bytes, B * C,
+                                              OH * OW, K, P, IH, IW, interp, s);
+  if (rc != kNotApplicable) return rc;
+  return launch_scatter<T, OP_AVG>(gout, map, iw, gin, B, C, IH, IW, OH * OW, K, P, interp, s);
+}
+}  // namespace
+
 extern "C" int mcx_avg_unpool(const void *gout, const void *map, const void *iw, void *gin,
-                              int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t OH, int64_t OW,
-                              int64_t K, int64_t P, int interp, int dtype, void *stream) {
+                              void *workspace, size_t workspace_bytes, int64_t B, int64_t C,
+                              int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P,
+                              int interp, int dtype, void *stream) {
   if (int rc = check_common(gout, map, iw, gin, P, dtype)) return rc;
   if (bad_dims({B, C, IH, IW, OH, OW, K, IH * IW, OH * OW}) || B > 65535) return MCX_E_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == MCX_F32)
-    return launch_scatter<float, OP_AVG>(gout, map, iw, gin, B, C, IH, IW, OH * OW, K, P, interp,
-                                         s);
-  return launch_scatter<double, OP_AVG>(gout, map, iw, gin, B, C, IH, IW, OH * OW, K, P, interp, s);
+    return avg_unpool_t<float>(gout, map, iw, gin, workspace, workspace_bytes, B, C, IH, IW, OH, OW,
+                               K, P, interp, s);
+  return avg_unpool_t<double>(gout, map, iw, gin, workspace, workspace_bytes, B, C, IH, IW, OH, OW,
+                              K, P, interp, s);
 }
 
 namespace {
 template <typename T>
 int launch_max_unpool(const void *gout, const int64_t *idx, const void *map, const void *iw,
-                      void *gin, int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t N,
-                      int64_t K, int64_t P, int interp, hipStream_t s) {
-  int rc = mcx::fill<T>((T *)gin, B * C * IH * IW, T(0), s);
+                      void *gin, void *ws, size_t ws_bytes, int64_t B, int64_t C, int64_t IH,
+                      int64_t IW, int64_t N, int64_t K, int64_t P, int interp, hipStream_t s) {
+  int rc = launch_transposed<T, UN_MAX>(gout, idx, map, iw, gin, ws, ws_bytes, B * C, N, K, P, IH,
+                                        IW, interp, s);
+  if (rc != kNotApplicable) return rc;
+  rc = mcx::fill<T>((T *)gin, B * C * IH * IW, T(0), s);
   if (rc) return rc;
   const int64_t total = B * C * N;
   const int64_t map_elems = N * K * (P ? P : 1) * 2;
@@ -312,9 +571,9 @@ int launch_max_unpool(const void *gout, const int64_t *idx, const void *map, con
 }  // namespace
 
 extern "C" int mcx_max_unpool(const void *gout, const int64_t *idx, const void *map,
-                              const void *iw, void *gin, int64_t B, int64_t C, int64_t IH,
-                              int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
-                              int dtype, void *stream) {
+                              const void *iw, void *gin, void *workspace, size_t workspace_bytes,
+                              int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t OH, int64_t OW,
+                              int64_t K, int64_t P, int interp, int dtype, void *stream) {
   if (int rc = check_common(gout, map, iw, gin, P, dtype)) return rc;
   if (!idx) return MCX_E_NULL;
   if (bad_dims({B, C, IH, IW, OH, OW, K, IH * IW, OH * OW}) ||
@@ -322,7 +581,8 @@ extern "C" int mcx_max_unpool(const void *gout, const int64_t *idx, const void *
     return MCX_E_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == MCX_F32)
-    return launch_max_unpool<float>(gout, idx, map, iw, gin, B, C, IH, IW, OH * OW, K, P, interp,
-                                    s);
-  return launch_max_unpool<double>(gout, idx, map, iw, gin, B, C, IH, IW, OH * OW, K, P, interp, s);
+    return launch_max_unpool<float>(gout, idx, map, iw, gin, workspace, workspace_bytes, B, C, IH,
+                                    IW, OH * OW, K, P, interp, s);
+  return launch_max_unpool<double>(gout, idx, map, iw, gin, workspace, workspace_bytes, B, C, IH,
+                                   IW, OH * OW, K, P, interp, s);
 }

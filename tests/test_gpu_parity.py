@@ -124,7 +124,9 @@ def test_transposed_conv_forward_backward(dtype, interp, p, device):
 @pytest.mark.parametrize("interp", [0, 1, 2])
 @pytest.mark.parametrize("p", [0, 3])
 @pytest.mark.parametrize("half", [False, True])
-def test_pools(dtype, interp, p, half, device):
+@pytest.mark.parametrize("form", ["gather", "atomic"])
+def test_pools(dtype, interp, p, half, form, device, monkeypatch):
+    monkeypatch.setattr(_C, "scatter_as_gather", form == "gather")
     g = torch.Generator().manual_seed(300 + interp + 10 * p)
     B, C, IH, IW, OH, OW, K = 2, 11, 9, 13, 7, 9, 5   # C=11: a ragged channel chunk
     x = torch.randn(B, C, IH, IW, generator=g, dtype=torch.float64).to(dtype)
@@ -156,7 +158,9 @@ def test_pools(dtype, interp, p, half, device):
 @pytest.mark.parametrize("interp", [0, 1, 2])
 @pytest.mark.parametrize("p", [0, 4])
 @pytest.mark.parametrize("half", [False, True])
-def test_resample(dtype, interp, p, half, device):
+@pytest.mark.parametrize("form", ["gather", "atomic"])
+def test_resample(dtype, interp, p, half, form, device, monkeypatch):
+    monkeypatch.setattr(_C, "scatter_as_gather", form == "gather")
     g = torch.Generator().manual_seed(400 + interp + 10 * p)
     B, C, IH, IW, OH, OW = 2, 9, 10, 12, 8, 15
     x = torch.randn(B, C, IH, IW, generator=g, dtype=torch.float64).to(dtype)
@@ -344,6 +348,43 @@ def test_config4_cube_resample_and_pools(interp, device):
                    O.mapped_max_unpool(gy, mi, lmap, H, W, 9, 1)) < 1e-5
     assert rel_err(_C.mapped_avg_unpool(gy.cuda(), lmap.cuda(), H, W, 9, 1),
                    O.mapped_avg_unpool(gy, lmap, H, W, 9, 1)) < 1e-5
+
+
+def test_config4_full_size_scatter_properties(device):
+    """Full spatial size of the cube -> equirect resampling (256x1536 -> 512x1024) and of the
+    512x1024 unpoolings, fewer planes: the gather form against the atomic form, and
+    adjointness <R_to(x), y> == <x, R_from(y)> (the oracle would take minutes here)."""
+    F, H, W, B, C = 256, 512, 1024, 1, 16
+    g = torch.Generator().manual_seed(44)
+    cube = torch.rand(B, C, F, 6 * F, generator=g).cuda()
+    y = torch.randn(B, C, H, W, generator=g).cuda()
+    cmap = synthetic.cube_to_equirect_map(F, H, W).cuda()
+    lmap = synthetic.latitude_map(H, W, 1).cuda()
+    for interp in (1, 2):
+        _C.scatter_as_gather = True
+        to = _C.resample_to_map(cube, cmap, H, W, interp)
+        lhs = (to.double() * y.double()).sum()
+        rhs = (cube.double() * _C.resample_from_map(y, cmap, interp).double()).sum()
+        assert abs(lhs - rhs) < 1e-6 * abs(rhs)
+        _C.scatter_as_gather = False
+        try:
+            to_atomic = _C.resample_to_map(cube, cmap, H, W, interp)
+        finally:
+            _C.scatter_as_gather = True
+        assert rel_err(to, to_atomic.cpu()) < 1e-5
+    m, i = _C.mapped_max_pool(y, lmap, 9, 1)
+    au, mu = _C.mapped_avg_unpool(y, lmap, H, W, 9, 1), _C.mapped_max_unpool(y, i, lmap, H, W, 9, 1)
+    _C.scatter_as_gather = False
+    try:
+        au_a = _C.mapped_avg_unpool(y, lmap, H, W, 9, 1)
+        mu_a = _C.mapped_max_unpool(y, i, lmap, H, W, 9, 1)
+    finally:
+        _C.scatter_as_gather = True
+    assert rel_err(au, au_a.cpu()) < 1e-5 and rel_err(mu, mu_a.cpu()) < 1e-5
+    x = torch.randn(B, C, H, W, generator=g).cuda()
+    lhs = (_C.mapped_avg_pool(x, lmap, 9, 1).double() * y.double()).sum()
+    rhs = (x.double() * au.double()).sum()
+    assert abs(lhs - rhs) < 1e-6 * abs(rhs)
 
 
 def test_config5_bf16_5x5(device):
