@@ -120,14 +120,16 @@ struct Tap {
     const bool y1ok = y1 >= 0 && y1 <= h - 1;
     const bool y2ok = y2 >= 0 && y2 <= h - 1;
     const T A = y2f - y, B = x2f - x, C = x - x1f, D = y - y1f;
-    off[0] = (x1ok && y1ok) ? y1 * w + x1 : -1;
-    off[1] = (x2ok && y1ok) ? y1 * w + x2 : -1;
-    off[2] = (x1ok && y2ok) ? y2 * w + x1 : -1;
-    off[3] = (x2ok && y2ok) ? y2 * w + x2 : -1;
     wt[0] = A * B;
     wt[1] = A * C;
     wt[2] = D * B;
     wt[3] = D * C;
+    // A corner of weight exactly zero (integral coordinates) is treated like one outside
+    // the plane: it adds 0 to any finite value, and its load or atomic is saved.
+    off[0] = (x1ok && y1ok && wt[0] != T(0)) ? y1 * w + x1 : -1;
+    off[1] = (x2ok && y1ok && wt[1] != T(0)) ? y1 * w + x2 : -1;
+    off[2] = (x1ok && y2ok && wt[2] != T(0)) ? y2 * w + x1 : -1;
+    off[3] = (x2ok && y2ok && wt[3] != T(0)) ? y2 * w + x2 : -1;
   }
   template <typename TD>
   __device__ inline T gather(const TD *plane) const {

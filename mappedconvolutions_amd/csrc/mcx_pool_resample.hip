@@ -46,12 +46,22 @@ __global__ __launch_bounds__(kThreads) void gather_kernel(
     acc[c] = OP == OP_MAX ? T(-3.402823466e+38F) : T(0);
     best[c] = -1;
   }
+  // Unweighted: the next tap's coordinates are fetched while this tap's samples are.
+  T nx = T(0), ny = T(0);
+  if (P == 0) {
+    nx = map[(int64_t)n * K * 2];
+    ny = map[(int64_t)n * K * 2 + 1];
+  }
   for (int k = 0; k < K; k++) {
     const int64_t e = ((int64_t)n * K + k) * pm;
     T val[kCH];
     if (P == 0) {
       Tap<T, MODE> tap;
-      tap.set(map[e * 2], map[e * 2 + 1], IH, IW);
+      tap.set(nx, ny, IH, IW);
+      if (k + 1 < K) {
+        nx = map[(e + 1) * 2];
+        ny = map[(e + 1) * 2 + 1];
+      }
 #pragma unroll
       for (int c = 0; c < kCH; c++)
         if (c < nc) val[c] = tap.gather(src + c * plane);
@@ -255,7 +265,43 @@ __global__ __launch_bounds__(kThreads) void scan_sums_kernel(uint32_t *__restric
   }
 }
 
-// One thread per destination pixel and kCH planes.  UN_MAX keeps a contribution
+// Orders the entries of every destination pixel by source location (insertion sort,
+// one thread per pixel; lists are short).  The fill kernel places entries in the
+// order its atomics happen to retire: sorted lists make the result independent of
+// that order, and neighbouring lanes of the gather then read neighbouring sources
+// at the same step.  Lists longer than kSortMax stay as filled.
+constexpr uint32_t kSortMax = 512;
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void sort_entries_kernel(
+    const uint32_t *__restrict__ local, const uint32_t *__restrict__ bsum,
+    uint32_t *__restrict__ e_src, T *__restrict__ e_wt, int ndst) {
+  const int p = blockIdx.x * kThreads + threadIdx.x;
+  if (p >= ndst) return;
+  const uint32_t start = local[p] + bsum[p / kScanBlock];
+  const uint32_t end = local[p + 1] + bsum[(p + 1) / kScanBlock];
+  if (end - start > kSortMax) return;
+  for (uint32_t i = start + 1; i < end; i++) {
+    const uint32_t code = e_src[i];
+    const T w = e_wt[i];
+    uint32_t j = i;
+    while (j > start) {
+      const uint32_t pc = e_src[j - 1];
+      const T pw = e_wt[j - 1];
+      // ties (one source reaching the pixel through two corners or points) by weight bits
+      if (pc < code || (pc == code && !(pw > w))) break;
+      e_src[j] = pc;
+      e_wt[j] = pw;
+      j--;
+    }
+    e_src[j] = code;
+    e_wt[j] = w;
+  }
+}
+
+constexpr int kTCH = 8;  // planes per thread of the transposed gather
+
+// One thread per destination pixel and kTCH planes.  UN_MAX keeps a contribution
 // only where the recorded winner of that source element is this tap.
 template <typename T, int OP>
 __global__ __launch_bounds__(kThreads) void transposed_gather_kernel(
@@ -266,33 +312,47 @@ __global__ __launch_bounds__(kThreads) void transposed_gather_kernel(
   const int pg = blockIdx.x % groups;
   const int p = (blockIdx.x / groups) * kThreads + threadIdx.x;
   if (p >= ndst) return;
-  const int64_t plane0 = (int64_t)pg * kCH;
-  const int nc = (int)min((int64_t)kCH, planes - plane0);
+  const int64_t plane0 = (int64_t)pg * kTCH;
+  const int nc = (int)min((int64_t)kTCH, planes - plane0);
   const uint32_t start = local[p] + bsum[p / kScanBlock];
   const uint32_t end = local[p + 1] + bsum[(p + 1) / kScanBlock];
   const T *s0 = src + plane0 * nsrc;
   const int64_t *i0 = OP == UN_MAX ? idx + plane0 * nsrc : nullptr;
-  T acc[kCH];
+  T acc[kTCH];
 #pragma unroll
-  for (int c = 0; c < kCH; c++) acc[c] = T(0);
-  for (uint32_t e = start; e < end; e++) {
-    const uint32_t code = e_src[e];
-    const T w = e_wt[e];
-    const uint32_t n = OP == UN_MAX ? code / (uint32_t)K : code;
-    const int64_t want = (int64_t)code * idx_scale;
+  for (int c = 0; c < kTCH; c++) acc[c] = T(0);
+  // kUnroll entries per trip so that their loads are in flight together; entries past
+  // the end repeat the last valid one with weight zero.
+  constexpr int kUnroll = OP == UN_RESAMPLE ? 2 : 4;
+  for (uint32_t e = start; e < end; e += kUnroll) {
+    uint32_t code[kUnroll];
+    T w[kUnroll];
 #pragma unroll
-    for (int c = 0; c < kCH; c++) {
-      if (c >= nc) continue;
-      if (OP == UN_MAX) {
-        if (i0[(int64_t)c * nsrc + n] == want) acc[c] = mcx_fma(w, s0[(int64_t)c * nsrc + n], acc[c]);
-      } else {
-        acc[c] = mcx_fma(w, s0[(int64_t)c * nsrc + n], acc[c]);
+    for (int u = 0; u < kUnroll; u++) {
+      const bool in = e + u < end;
+      const uint32_t ee = in ? e + u : e;
+      code[u] = e_src[ee];
+      w[u] = in ? e_wt[ee] : T(0);
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+      const uint32_t n = OP == UN_MAX ? code[u] / (uint32_t)K : code[u];
+      const int64_t want = (int64_t)code[u] * idx_scale;
+#pragma unroll
+      for (int c = 0; c < kTCH; c++) {
+        if (c >= nc) continue;
+        if (OP == UN_MAX) {
+          if (i0[(int64_t)c * nsrc + n] == want)
+            acc[c] = mcx_fma(w[u], s0[(int64_t)c * nsrc + n], acc[c]);
+        } else {
+          acc[c] = mcx_fma(w[u], s0[(int64_t)c * nsrc + n], acc[c]);
+        }
       }
     }
   }
   T *d0 = dst + plane0 * ndst + p;
 #pragma unroll
-  for (int c = 0; c < kCH; c++)
+  for (int c = 0; c < kTCH; c++)
     if (c < nc) d0[(int64_t)c * ndst] = OP == UN_AVG ? acc[c] / (T)K : acc[c];
 }
 
@@ -365,7 +425,7 @@ int launch_transposed(const void *src, const int64_t *idx, const void *map, cons
   const int64_t samples = nsrc * K * pm, ndst = DH * DW;
   const TransposedLayout l = transposed_layout(ndst, samples, corners_of(interp), sizeof(T));
   if (!ws || !l.ok || ws_bytes < l.total || nsrc * K > 0xffffffffLL) return kNotApplicable;
-  const int64_t groups = (planes + kCH - 1) / kCH;
+  const int64_t groups = (planes + kTCH - 1) / kTCH;
   const int64_t blocks = groups * ((ndst + kThreads - 1) / kThreads);
   if (blocks > 0x7fffffffLL) return kNotApplicable;
   char *base = (char *)ws;
@@ -390,6 +450,9 @@ int launch_transposed(const void *src, const int64_t *idx, const void *map, cons
                                                0, s, (const T *)map, (const T *)iw, samples,
                                                per_code, (int)DH, (int)DW, local, cursor, bsum,
                                                e_src, e_wt));
+  MCX_HIP_CHECK_LAUNCH();
+  hipLaunchKernelGGL((sort_entries_kernel<T>), dim3(div_up(ndst, kThreads)), blk, 0, s, local, bsum,
+                     e_src, e_wt, (int)ndst);
   MCX_HIP_CHECK_LAUNCH();
   hipLaunchKernelGGL((transposed_gather_kernel<T, OP>), dim3((unsigned)blocks), blk, 0, s,
                      (const T *)src, idx, (T *)dst, local, bsum, e_src, e_wt, planes, (int)nsrc,
