@@ -11,6 +11,15 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kCH = 8;  // channels per thread
+// Map locations per workgroup: a 32 x 8 patch for resampling (arbitrary maps: neighbouring
+// rows of the map read neighbouring source pixels), one 256-long row segment for pooling
+// (taps already reach into the rows above and below; longer rows mean fewer cache lines
+// per wave-wide load).
+template <int OP>
+struct Patch {
+  static constexpr int kW = OP == 0 ? 32 : kThreads;
+  static constexpr int kH = kThreads / kW;
+};
 
 enum { OP_RESAMPLE = 0, OP_AVG = 1, OP_MAX = 2 };
 
@@ -29,9 +38,14 @@ __global__ void fill_kernel(T *p, int64_t n, T v) {
 template <typename T, int MODE, int OP>
 __global__ __launch_bounds__(kThreads) void gather_kernel(
     const T *__restrict__ in, const T *__restrict__ map, const T *__restrict__ iw,
-    T *__restrict__ out, int64_t *__restrict__ idx, int C, int IH, int IW, int N, int K, int P) {
-  const int n = blockIdx.x * kThreads + threadIdx.x;
-  if (n >= N) return;
+    T *__restrict__ out, int64_t *__restrict__ idx, int C, int IH, int IW, int N, int MW, int K,
+    int P) {
+  constexpr int kTileW = Patch<OP>::kW, kTileH = Patch<OP>::kH;
+  const int tiles_x = (MW + kTileW - 1) / kTileW;
+  const int tx = (blockIdx.x % tiles_x) * kTileW + threadIdx.x % kTileW;
+  const int ty = (blockIdx.x / tiles_x) * kTileH + threadIdx.x / kTileW;
+  const int n = ty * MW + tx;
+  if (tx >= MW || n >= N) return;
   const int c0 = blockIdx.y * kCH;
   const int b = blockIdx.z;
   const int64_t plane = (int64_t)IH * IW;
@@ -373,13 +387,14 @@ int fill(T *p, int64_t n, T v, hipStream_t s) {
 
 template <typename T, int OP>
 int launch_gather(const void *in, const void *map, const void *iw, void *out, int64_t *idx,
-                  int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t N, int64_t K, int64_t P,
-                  int interp, hipStream_t s) {
-  dim3 grid(div_up(N, kThreads), div_up(C, kCH), (unsigned)B);
+                  int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t MH, int64_t MW, int64_t K,
+                  int64_t P, int interp, hipStream_t s) {
+  const int64_t N = MH * MW;
+  dim3 grid(div_up(MW, Patch<OP>::kW) * div_up(MH, Patch<OP>::kH), div_up(C, kCH), (unsigned)B);
   MCX_DISPATCH_MODE(interp, hipLaunchKernelGGL((gather_kernel<T, MODE, OP>), grid, dim3(kThreads),
                                                0, s, (const T *)in, (const T *)map,
                                                (const T *)iw, (T *)out, idx, (int)C, (int)IH,
-                                               (int)IW, (int)N, (int)K, (int)P));
+                                               (int)IW, (int)N, (int)MW, (int)K, (int)P));
   MCX_HIP_CHECK_LAUNCH();
   return 0;
 }
@@ -503,9 +518,9 @@ extern "C" int mcx_resample_from_map(const void *src, const void *map, const voi
     return MCX_E_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == MCX_F32)
-    return launch_gather<float, OP_RESAMPLE>(src, map, iw, dst, nullptr, B, C, SH, SW, MH * MW, 1,
+    return launch_gather<float, OP_RESAMPLE>(src, map, iw, dst, nullptr, B, C, SH, SW, MH, MW, 1,
                                              P, interp, s);
-  return launch_gather<double, OP_RESAMPLE>(src, map, iw, dst, nullptr, B, C, SH, SW, MH * MW, 1,
+  return launch_gather<double, OP_RESAMPLE>(src, map, iw, dst, nullptr, B, C, SH, SW, MH, MW, 1,
                                             P, interp, s);
 }
 
@@ -566,9 +581,9 @@ extern "C" int mcx_max_pool(const void *in, const void *map, const void *iw, voi
   if (bad_dims({B, C, IH, IW, OH, OW, K, IH * IW, OH * OW}) || B > 65535) return MCX_E_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == MCX_F32)
-    return launch_gather<float, OP_MAX>(in, map, iw, out, idx, B, C, IH, IW, OH * OW, K, P, interp,
+    return launch_gather<float, OP_MAX>(in, map, iw, out, idx, B, C, IH, IW, OH, OW, K, P, interp,
                                         s);
-  return launch_gather<double, OP_MAX>(in, map, iw, out, idx, B, C, IH, IW, OH * OW, K, P, interp,
+  return launch_gather<double, OP_MAX>(in, map, iw, out, idx, B, C, IH, IW, OH, OW, K, P, interp,
                                        s);
 }
 
@@ -579,9 +594,9 @@ extern "C" int mcx_avg_pool(const void *in, const void *map, const void *iw, voi
   if (bad_dims({B, C, IH, IW, OH, OW, K, IH * IW, OH * OW}) || B > 65535) return MCX_E_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == MCX_F32)
-    return launch_gather<float, OP_AVG>(in, map, iw, out, nullptr, B, C, IH, IW, OH * OW, K, P,
+    return launch_gather<float, OP_AVG>(in, map, iw, out, nullptr, B, C, IH, IW, OH, OW, K, P,
                                         interp, s);
-  return launch_gather<double, OP_AVG>(in, map, iw, out, nullptr, B, C, IH, IW, OH * OW, K, P,
+  return launch_gather<double, OP_AVG>(in, map, iw, out, nullptr, B, C, IH, IW, OH, OW, K, P,
                                        interp, s);
 }
 
