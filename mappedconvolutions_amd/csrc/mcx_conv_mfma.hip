@@ -62,6 +62,11 @@ __global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
   __shared__ __attribute__((aligned(16))) float Wt[2][kGC][kWtLd];
   __shared__ __attribute__((aligned(16))) unsigned TapOff[TG][kTilePx][NE];
   __shared__ __attribute__((aligned(16))) float TapWt[TG][kTilePx][NE];
+  // Bit e of TapMask[kl][h]: some pixel of the half-tile resolved by wave pair h has a
+  // nonzero weight in pair e of tap kl.  Pairs that are zero across the whole tile
+  // (bilinear corners of integral coordinates, unused slots) are neither loaded nor
+  // accumulated.
+  __shared__ unsigned TapMask[TG][2][2];
   if (gate && ((*gate == 0) != (run_if_zero != 0))) return;  // device-side path selection
 
   const int tid = threadIdx.x;
@@ -88,37 +93,51 @@ __global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
   unsigned off[NE];
   float wt[NE];
   float v[8][NE];
+  unsigned tmask = 0;
   float4 wv;
   const int w_off = (tid >> 4) * Opad + (tid & 15) * 4;
 
   auto load_tap = [&](int kl) {  // cached pairs of tap kl of the group -> registers
+    tmask = __builtin_amdgcn_readfirstlane(TapMask[kl][0][0] | TapMask[kl][0][1] |
+                                           TapMask[kl][1][0] | TapMask[kl][1][1]);
 #pragma unroll
     for (int i = 0; i < NE; i++) {
       off[i] = TapOff[kl][p][i];
       wt[i] = TapWt[kl][p][i];
     }
   };
-  auto issue = [&](int k, int c) {
+  // Plane bases of this thread's 8 channels of a chunk (scalar registers); they change
+  // only when the chunk does, not with every tap.
+  const TD *pl[8];
+  auto set_chunk = [&](int c) {
     const int g0 = c * kGC + half * 8;
 #pragma unroll
-    for (int ch = 0; ch < 8; ch++) {
-      const int g = min(g0 + ch, G - 1);  // padded channels read a valid plane, weights are 0
-      const TD *pl = src_b + (int64_t)g * plane;
+    for (int ch = 0; ch < 8; ch++)  // padded channels read a valid plane, weights are 0
+      pl[ch] = src_b + (int64_t)min(g0 + ch, G - 1) * plane;
+  };
+  auto issue = [&](int k, int c) {
 #pragma unroll
-      for (int i = 0; i < NE; i++) v[ch][i] = load_at(pl, off[i]);
+    for (int i = 0; i < NE; i++) {
+      if (!((tmask >> i) & 1u)) continue;  // wave-uniform
+#pragma unroll
+      for (int ch = 0; ch < 8; ch++) v[ch][i] = load_at(pl[ch], off[i]);
     }
     // weights of this chunk: 16 rows x 64 floats, one float4 per thread
     const float *wchunk = wp + ((int64_t)k * Gpad + c * kGC) * Opad + o0;  // uniform
     wv = *reinterpret_cast<const float4 *>(wchunk + w_off);
   };
   auto stage = [&](int buf) {
+    float sv[8];
 #pragma unroll
-    for (int ch = 0; ch < 8; ch++) {
-      float acc = 0.f;
+    for (int ch = 0; ch < 8; ch++) sv[ch] = 0.f;
 #pragma unroll
-      for (int i = 0; i < NE; i++) acc = __builtin_fmaf(wt[i], v[ch][i], acc);
-      S[buf][half * 8 + ch][p] = acc;
+    for (int i = 0; i < NE; i++) {
+      if (!((tmask >> i) & 1u)) continue;
+#pragma unroll
+      for (int ch = 0; ch < 8; ch++) sv[ch] = __builtin_fmaf(wt[i], v[ch][i], sv[ch]);
     }
+#pragma unroll
+    for (int ch = 0; ch < 8; ch++) S[buf][half * 8 + ch][p] = sv[ch];
     const int cc = tid >> 4, o4 = (tid & 15) * 4;
     *reinterpret_cast<float4 *>(&Wt[buf][cc][o4]) = wv;
   };
@@ -133,7 +152,10 @@ __global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
     // Resolve the group's taps once per tile into LDS: thread (p, half) takes every
     // other tap of pixel p.  All channel chunks reuse them.
     __syncthreads();  // the previous group's units are done with the cache and with S/Wt
+    if (tid < TG * 4) (&TapMask[0][0][0])[tid] = 0u;  // slots no wave writes below
+    __syncthreads();
     for (int kl = half; kl < kn; kl += 2) {
+      unsigned m = 0;
 #pragma unroll
       for (int sp = 0; sp < NP; sp++) {
         const int64_t e = (n_g * K + k0 + kl) * NP + sp;
@@ -144,8 +166,10 @@ __global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
         for (int i = 0; i < NCORN; i++) {
           TapOff[kl][p][sp * NCORN + i] = t.off[i];
           TapWt[kl][p][sp * NCORN + i] = t.wt[i];
+          if (__builtin_amdgcn_ballot_w64(t.wt[i] != 0.f)) m |= 1u << (sp * NCORN + i);
         }
       }
+      if ((tid & 63) == 0) TapMask[kl][half][(tid >> 6) & 1] = m;
     }
     __syncthreads();
 
@@ -153,6 +177,7 @@ __global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
     // touches are reused by all taps of the group while they are still in cache.
     const int units = chunks * kn;
     load_tap(0);
+    set_chunk(0);
     issue(k0, 0);
     int kl = 0, c = 0;
     for (int u = 0; u < units; ++u) {
@@ -161,6 +186,7 @@ __global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
       if (++kl == kn) {
         kl = 0;
         ++c;
+        set_chunk(c);
       }
       if (u + 1 < units) {  // next unit's taps and gathers in flight during the MFMAs
         load_tap(kl);
