@@ -50,6 +50,46 @@ __global__ void pack_weights_kernel(const TD *__restrict__ w, float *__restrict_
   }
 }
 
+// bf16 storage feeds v_mfma_f32_32x32x16_bf16: one instruction multiplies a 32 x 16 block
+// of weights by a 16 x 32 block of samples, a lane holding 8 consecutive reduction
+// elements (channels kg*8 .. kg*8+7, kg = lane / 32) of its row or column in 16 bytes.
+// Weights are therefore packed as Wb[k][chunk][kg][o][8] bf16: the 64 x 16 slice of a
+// (tap, chunk) is two runs of 64 x 16 bytes that are copied linearly into LDS.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+
+template <typename TD>
+__global__ void pack_weights_bf16_kernel(const TD *__restrict__ w, uint16_t *__restrict__ wb,
+                                         int O, int G, int K, int Opad, int Gpad,
+                                         int transposed) {
+  const int chunks = Gpad / kGC;
+  const int64_t total = (int64_t)K * Gpad * Opad;
+  for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total;
+       e += (int64_t)gridDim.x * blockDim.x) {
+    const int j = (int)(e & 7);
+    const int o = (int)((e >> 3) % Opad);
+    const int kg = (int)((e / ((int64_t)8 * Opad)) & 1);
+    const int c = (int)((e / ((int64_t)16 * Opad)) % chunks);
+    const int k = (int)(e / ((int64_t)16 * Opad * chunks));
+    const int g = c * kGC + kg * 8 + j;
+    const int64_t wi = transposed ? ((int64_t)g * O + o) * K + k : ((int64_t)o * G + g) * K + k;
+    wb[e] = (o < O && g < G) ? from_f32<bf16_t>(to_f32(w[wi])).v : (uint16_t)0;
+  }
+}
+
+// LDS operand tiles of the gather-product kernel, double-buffered.
+template <typename TD>
+struct OperandTiles {  // fp32: samples S[chunk channel][pixel], weights Wt[chunk channel][o]
+  float S[2][kGC][kTilePx];
+  float Wt[2][kGC][kWtLd];
+};
+template <>
+struct OperandTiles<bf16_t> {  // bf16: 16-byte groups of 8 channels, [kg][pixel] and [kg][o]
+  uint4 S[2][2][kTilePx];
+  uint4 Wt[2][2][kOT];
+};
+
 template <typename TD, int NCORN, int NP>
 __global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
     const TD *__restrict__ src, const float *__restrict__ map, const float *__restrict__ iw,
@@ -58,8 +98,8 @@ __global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
     int tiles_x, int tiles_per_img, int tw_shift, const int *__restrict__ gate, int run_if_zero) {
   constexpr int NE = NP * NCORN;         // (offset, weight) pairs per pixel and tap
   constexpr int TG = kTapCache / NE > 0 ? kTapCache / NE : 1;  // taps cached in LDS at a time
-  __shared__ __attribute__((aligned(16))) float S[2][kGC][kTilePx];
-  __shared__ __attribute__((aligned(16))) float Wt[2][kGC][kWtLd];
+  constexpr bool kBf16 = sizeof(TD) == 2;
+  __shared__ __attribute__((aligned(16))) OperandTiles<TD> T;
   __shared__ __attribute__((aligned(16))) unsigned TapOff[TG][kTilePx][NE];
   __shared__ __attribute__((aligned(16))) float TapWt[TG][kTilePx][NE];
   // Bit e of TapMask[kl][h]: some pixel of the half-tile resolved by wave pair h has a
@@ -94,7 +134,8 @@ __global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
   float wt[NE];
   float v[8][NE];
   unsigned tmask = 0;
-  float4 wv;
+  float4 wv;   // fp32: this thread's share of the next weight chunk
+  uint2 wb8;   // bf16: likewise, 8 bytes
   const int w_off = (tid >> 4) * Opad + (tid & 15) * 4;
 
   auto load_tap = [&](int kl) {  // cached pairs of tap kl of the group -> registers
@@ -122,9 +163,16 @@ __global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
 #pragma unroll
       for (int ch = 0; ch < 8; ch++) v[ch][i] = load_at(pl[ch], off[i]);
     }
-    // weights of this chunk: 16 rows x 64 floats, one float4 per thread
-    const float *wchunk = wp + ((int64_t)k * Gpad + c * kGC) * Opad + o0;  // uniform
-    wv = *reinterpret_cast<const float4 *>(wchunk + w_off);
+    if constexpr (kBf16) {
+      // weights of this chunk: two runs (kg = 0, 1) of 64 x 16 bytes, 8 bytes per thread
+      const char *wchunk = reinterpret_cast<const char *>(wp) +
+                           ((((int64_t)k * chunks + c) * 2 + (tid >> 7)) * Opad + o0) * 16;
+      wb8 = *reinterpret_cast<const uint2 *>(wchunk + (tid & 127) * 8);
+    } else {
+      // weights of this chunk: 16 rows x 64 floats, one float4 per thread
+      const float *wchunk = wp + ((int64_t)k * Gpad + c * kGC) * Opad + o0;  // uniform
+      wv = *reinterpret_cast<const float4 *>(wchunk + w_off);
+    }
   };
   auto stage = [&](int buf) {
     float sv[8];
@@ -136,10 +184,20 @@ __global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
 #pragma unroll
       for (int ch = 0; ch < 8; ch++) sv[ch] = __builtin_fmaf(wt[i], v[ch][i], sv[ch]);
     }
+    if constexpr (kBf16) {
+      uint4 q;
+      q.x = __builtin_bit_cast(unsigned, __builtin_convertvector(floatx2{sv[0], sv[1]}, bf16x2));
+      q.y = __builtin_bit_cast(unsigned, __builtin_convertvector(floatx2{sv[2], sv[3]}, bf16x2));
+      q.z = __builtin_bit_cast(unsigned, __builtin_convertvector(floatx2{sv[4], sv[5]}, bf16x2));
+      q.w = __builtin_bit_cast(unsigned, __builtin_convertvector(floatx2{sv[6], sv[7]}, bf16x2));
+      T.S[buf][half][p] = q;
+      reinterpret_cast<uint2 *>(&T.Wt[buf][tid >> 7][0])[tid & 127] = wb8;
+    } else {
 #pragma unroll
-    for (int ch = 0; ch < 8; ch++) S[buf][half * 8 + ch][p] = sv[ch];
-    const int cc = tid >> 4, o4 = (tid & 15) * 4;
-    *reinterpret_cast<float4 *>(&Wt[buf][cc][o4]) = wv;
+      for (int ch = 0; ch < 8; ch++) T.S[buf][half * 8 + ch][p] = sv[ch];
+      const int cc = tid >> 4, o4 = (tid & 15) * 4;
+      *reinterpret_cast<float4 *>(&T.Wt[buf][cc][o4]) = wv;
+    }
   };
 
   floatx16 acc0 = {0}, acc1 = {0};
@@ -193,18 +251,26 @@ __global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
         issue(k0 + kl, c);
       }
       // fetch every operand of the chunk first, then issue the MFMAs back to back
-      float bv[kGC / 2], a0[kGC / 2], a1[kGC / 2];
+      if constexpr (kBf16) {
+        const bf16x8 bq = __builtin_bit_cast(bf16x8, T.S[buf][lhi][wave * 32 + l31]);
+        const bf16x8 aq0 = __builtin_bit_cast(bf16x8, T.Wt[buf][lhi][l31]);
+        const bf16x8 aq1 = __builtin_bit_cast(bf16x8, T.Wt[buf][lhi][32 + l31]);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aq0, bq, acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aq1, bq, acc1, 0, 0, 0);
+      } else {
+        float bv[kGC / 2], a0[kGC / 2], a1[kGC / 2];
 #pragma unroll
-      for (int s = 0; s < kGC / 2; s++) {
-        const int kk = 2 * s + lhi;
-        bv[s] = S[buf][kk][wave * 32 + l31];
-        a0[s] = Wt[buf][kk][l31];
-        a1[s] = Wt[buf][kk][32 + l31];
-      }
+        for (int s = 0; s < kGC / 2; s++) {
+          const int kk = 2 * s + lhi;
+          bv[s] = T.S[buf][kk][wave * 32 + l31];
+          a0[s] = T.Wt[buf][kk][l31];
+          a1[s] = T.Wt[buf][kk][32 + l31];
+        }
 #pragma unroll
-      for (int s = 0; s < kGC / 2; s++) {
-        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[s], bv[s], acc0, 0, 0, 0);
-        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[s], bv[s], acc1, 0, 0, 0);
+        for (int s = 0; s < kGC / 2; s++) {
+          acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[s], bv[s], acc0, 0, 0, 0);
+          acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[s], bv[s], acc1, 0, 0, 0);
+        }
       }
       buf ^= 1;
     }
@@ -906,9 +972,14 @@ int launch_pack_weights(const TD *w, float *wp, int64_t O, int64_t G, int64_t K,
                         hipStream_t s) {
   const int Opad = (int)round_up(O, kOT), Gpad = (int)round_up(G, kGC);
   const int64_t packed = (int64_t)K * Gpad * Opad;
-  hipLaunchKernelGGL(pack_weights_kernel<TD>,
-                     dim3((unsigned)std::min<int64_t>((packed + 255) / 256, 4096)), dim3(256), 0, s,
-                     w, wp, (int)O, (int)G, (int)K, Opad, Gpad, transposed);
+  const dim3 grid((unsigned)std::min<int64_t>((packed + 255) / 256, 4096));
+  if (sizeof(TD) == 2)  // bf16 storage: bf16 MFMA operand layout (same scratch, half the bytes)
+    hipLaunchKernelGGL(pack_weights_bf16_kernel<TD>, grid, dim3(256), 0, s, w,
+                       reinterpret_cast<uint16_t *>(wp), (int)O, (int)G, (int)K, Opad, Gpad,
+                       transposed);
+  else
+    hipLaunchKernelGGL(pack_weights_kernel<TD>, grid, dim3(256), 0, s, w, wp, (int)O, (int)G,
+                       (int)K, Opad, Gpad, transposed);
   MCX_HIP_CHECK_LAUNCH();
   return 0;
 }
