@@ -87,11 +87,13 @@ struct OperandTiles {  // fp32: samples S[chunk channel][pixel], weights Wt[chun
 template <>
 struct OperandTiles<bf16_t> {  // bf16: 16-byte groups of 8 channels, [kg][pixel] and [kg][o]
   uint4 S[2][2][kTilePx];
-  uint4 Wt[2][2][kOT];
+  uint4 Wt[2][2][2 * kOT];
 };
 
-template <typename TD, int NCORN, int NP>
-__global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
+// OG: groups of 64 output channels per workgroup (2 only with bf16 storage, where the
+// gather, not the MFMA, bounds the kernel and is shared by twice the outputs).
+template <typename TD, int NCORN, int NP, int OG>
+__global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma_kernel(
     const TD *__restrict__ src, const float *__restrict__ map, const float *__restrict__ iw,
     const float *__restrict__ wp, const TD *__restrict__ bias, TD *__restrict__ y, int G,
     int O, int Opad, int Gpad, int SH, int SW, int OH, int OW, int K, int weighted, int wrap,
@@ -116,7 +118,7 @@ __global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
   const int tile_y = t_in / tiles_x, tile_x = t_in - tile_y * tiles_x;
   const int tw_mask = (1 << tw_shift) - 1;
   const int th = kTilePx >> tw_shift;
-  const int o0 = blockIdx.y * kOT;
+  const int o0 = blockIdx.y * (kOT * OG);
   const int N = OH * OW;
   const int64_t plane = (int64_t)SH * SW;
 
@@ -135,7 +137,7 @@ __global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
   float v[8][NE];
   unsigned tmask = 0;
   float4 wv;   // fp32: this thread's share of the next weight chunk
-  uint2 wb8;   // bf16: likewise, 8 bytes
+  unsigned wb8[2 * OG];  // bf16: likewise, 8 * OG bytes
   const int w_off = (tid >> 4) * Opad + (tid & 15) * 4;
 
   auto load_tap = [&](int kl) {  // cached pairs of tap kl of the group -> registers
@@ -164,10 +166,16 @@ __global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
       for (int ch = 0; ch < 8; ch++) v[ch][i] = load_at(pl[ch], off[i]);
     }
     if constexpr (kBf16) {
-      // weights of this chunk: two runs (kg = 0, 1) of 64 x 16 bytes, 8 bytes per thread
+      // weights of this chunk: two runs (kg = 0, 1) of 64*OG x 16 bytes, 8*OG bytes per thread
       const char *wchunk = reinterpret_cast<const char *>(wp) +
                            ((((int64_t)k * chunks + c) * 2 + (tid >> 7)) * Opad + o0) * 16;
-      wb8 = *reinterpret_cast<const uint2 *>(wchunk + (tid & 127) * 8);
+      if constexpr (OG == 1) {
+        const uint2 t2 = *reinterpret_cast<const uint2 *>(wchunk + (tid & 127) * 8);
+        wb8[0] = t2.x; wb8[1] = t2.y;
+      } else {
+        const uint4 t4 = *reinterpret_cast<const uint4 *>(wchunk + (tid & 127) * 16);
+        wb8[0] = t4.x; wb8[1] = t4.y; wb8[2 % (2 * OG)] = t4.z; wb8[3 % (2 * OG)] = t4.w;
+      }
     } else {
       // weights of this chunk: 16 rows x 64 floats, one float4 per thread
       const float *wchunk = wp + ((int64_t)k * Gpad + c * kGC) * Opad + o0;  // uniform
@@ -191,7 +199,11 @@ __global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
       q.z = __builtin_bit_cast(unsigned, __builtin_convertvector(floatx2{sv[4], sv[5]}, bf16x2));
       q.w = __builtin_bit_cast(unsigned, __builtin_convertvector(floatx2{sv[6], sv[7]}, bf16x2));
       T.S[buf][half][p] = q;
-      reinterpret_cast<uint2 *>(&T.Wt[buf][tid >> 7][0])[tid & 127] = wb8;
+      if constexpr (OG == 1)
+        reinterpret_cast<uint2 *>(&T.Wt[buf][tid >> 7][0])[tid & 127] = uint2{wb8[0], wb8[1]};
+      else
+        T.Wt[buf][tid >> 7][tid & 127] =
+            uint4{wb8[0], wb8[1], wb8[2 % (2 * OG)], wb8[3 % (2 * OG)]};
     } else {
 #pragma unroll
       for (int ch = 0; ch < 8; ch++) T.S[buf][half * 8 + ch][p] = sv[ch];
@@ -200,7 +212,11 @@ __global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
     }
   };
 
-  floatx16 acc0 = {0}, acc1 = {0};
+  floatx16 acc[2 * OG];
+#pragma unroll
+  for (int m = 0; m < 2 * OG; m++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[m][i] = 0.f;
   const int lane = tid & 63, wave = tid >> 6;
   const int l31 = lane & 31, lhi = lane >> 5;
 
@@ -253,10 +269,13 @@ __global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
       // fetch every operand of the chunk first, then issue the MFMAs back to back
       if constexpr (kBf16) {
         const bf16x8 bq = __builtin_bit_cast(bf16x8, T.S[buf][lhi][wave * 32 + l31]);
-        const bf16x8 aq0 = __builtin_bit_cast(bf16x8, T.Wt[buf][lhi][l31]);
-        const bf16x8 aq1 = __builtin_bit_cast(bf16x8, T.Wt[buf][lhi][32 + l31]);
-        acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aq0, bq, acc0, 0, 0, 0);
-        acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aq1, bq, acc1, 0, 0, 0);
+        bf16x8 aq[2 * OG];
+#pragma unroll
+        for (int m = 0; m < 2 * OG; m++)
+          aq[m] = __builtin_bit_cast(bf16x8, T.Wt[buf][lhi][32 * m + l31]);
+#pragma unroll
+        for (int m = 0; m < 2 * OG; m++)
+          acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aq[m], bq, acc[m], 0, 0, 0);
       } else {
         float bv[kGC / 2], a0[kGC / 2], a1[kGC / 2];
 #pragma unroll
@@ -268,8 +287,8 @@ __global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
         }
 #pragma unroll
         for (int s = 0; s < kGC / 2; s++) {
-          acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[s], bv[s], acc0, 0, 0, 0);
-          acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[s], bv[s], acc1, 0, 0, 0);
+          acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[s], bv[s], acc[0], 0, 0, 0);
+          acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[s], bv[s], acc[1], 0, 0, 0);
         }
       }
       buf ^= 1;
@@ -282,12 +301,12 @@ __global__ __launch_bounds__(kThreads, 4) void gather_product_mfma_kernel(
   if (ei < OH && ej < OW) {
     TD *yb = y + (int64_t)b * O * N + (int64_t)ei * OW + ej;
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-      const int o = o0 + (i >> 2) * 8 + lhi * 4 + (i & 3);
-      if (o < O) yb[(int64_t)o * N] = from_f32<TD>(acc0[i] + (bias ? to_f32(bias[o]) : 0.f));
-      if (o + 32 < O)
-        yb[(int64_t)(o + 32) * N] = from_f32<TD>(acc1[i] + (bias ? to_f32(bias[o + 32]) : 0.f));
-    }
+    for (int m = 0; m < 2 * OG; m++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        const int o = o0 + 32 * m + (i >> 2) * 8 + lhi * 4 + (i & 3);
+        if (o < O) yb[(int64_t)o * N] = from_f32<TD>(acc[m][i] + (bias ? to_f32(bias[o]) : 0.f));
+      }
   }
 }
 
@@ -954,15 +973,28 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
   const int Opad = (int)round_up(O, kOT), Gpad = (int)round_up(G, kGC);
   const PixelTiling t = make_tiling(B, OH, OW);
   if (t.total > 0x7fffffffLL) return MCX_E_SHAPE;
-  dim3 grid((unsigned)t.total, (unsigned)(Opad / kOT));
+  // bf16 storage with at least 128 output channels: 128 outputs per workgroup
+  const bool wide = sizeof(TD) == 2 && Opad % (2 * kOT) == 0;
+  dim3 grid((unsigned)t.total, (unsigned)(Opad / (wide ? 2 * kOT : kOT)));
   const ModeArgs m = mode_args(interp, P);
-#define MCX_LAUNCH(NCORN, NP)                                                                    \
-  hipLaunchKernelGGL((gather_product_mfma_kernel<TD, NCORN, NP>), grid, dim3(kThreads), 0, s,    \
-                     src, map, iw, wp, bias, y, (int)G, (int)O, Opad, Gpad, (int)SH, (int)SW,    \
+#define MCX_LAUNCH_OG(NCORN, NP, OG)                                                             \
+  hipLaunchKernelGGL((gather_product_mfma_kernel<TD, NCORN, NP, OG>), grid, dim3(kThreads), 0,   \
+                     s, src, map, iw, wp, bias, y, (int)G, (int)O, Opad, Gpad, (int)SH, (int)SW, \
                      (int)OH, (int)OW, (int)K, m.weighted, m.wrap, t.tiles_x, t.tiles_per_img,   \
                      t.tw_shift, gate, run_if_zero)
+#define MCX_LAUNCH(NCORN, NP)                               \
+  if constexpr (sizeof(TD) == 2) {                          \
+    if (wide) {                                             \
+      MCX_LAUNCH_OG(NCORN, NP, 2);                          \
+    } else {                                                \
+      MCX_LAUNCH_OG(NCORN, NP, 1);                          \
+    }                                                       \
+  } else {                                                  \
+    MCX_LAUNCH_OG(NCORN, NP, 1);                            \
+  }
   MCX_DISPATCH_TAPS(m, MCX_LAUNCH)
 #undef MCX_LAUNCH
+#undef MCX_LAUNCH_OG
   MCX_HIP_CHECK_LAUNCH();
   return 0;
 }
