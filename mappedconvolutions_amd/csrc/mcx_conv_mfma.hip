@@ -343,6 +343,13 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
   __shared__ __attribute__((aligned(16))) float PtMem[kCacheTaps && kTapFloats > kPtFloats ? kTapFloats : kPtFloats];
   __shared__ __attribute__((aligned(16))) float S[2][kGC][kLdPx];
   float(*Pt)[kLdPx] = reinterpret_cast<float(*)[kLdPx]>(PtMem);
+  // bf16 storage: both tiles hold bf16 (row stride kLdPxB keeps 16-byte row reads of 16
+  // different rows on different banks) and feed v_mfma_f32_16x16x32_bf16, whose lanes take
+  // 8 consecutive pixels of their row.
+  constexpr bool kBf16 = sizeof(TD) == 2;
+  constexpr int kLdPxB = kTilePx + 8;
+  uint16_t(*PtB)[kLdPxB] = reinterpret_cast<uint16_t(*)[kLdPxB]>(PtMem);
+  uint16_t(*SB)[kGC][kLdPxB] = reinterpret_cast<uint16_t(*)[kGC][kLdPxB]>(&S[0][0][0]);
   unsigned(*TapOff)[kTilePx][NE] = reinterpret_cast<unsigned(*)[kTilePx][NE]>(PtMem);
   float(*TapWt)[kTilePx][NE] =
       reinterpret_cast<float(*)[kTilePx][NE]>(PtMem + kWgKT * kTilePx * NE);
@@ -394,38 +401,67 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
       const bool row_ok = (a0 + a) < A && si < MH;
       const TD *prow = plain + ((int64_t)b * A + min(a0 + a, A - 1)) * N +
                        (int64_t)min(si, MH - 1) * MW;
-      float t[32];
-      if (vec_ok && row_ok && sj + 32 <= MW) {
-        constexpr int kPer = 16 / (int)sizeof(TD);  // elements per 16-byte load
-        const uint4 *srcv = reinterpret_cast<const uint4 *>(prow + sj);
-        uint4 raw[32 / kPer];
+      if constexpr (kBf16) {
+        uint4 raw[4];
+        if (vec_ok && row_ok && sj + 32 <= MW) {
+          const uint4 *srcv = reinterpret_cast<const uint4 *>(prow + sj);
 #pragma unroll
-        for (int r = 0; r < 32 / kPer; r++) raw[r] = srcv[r];
+          for (int r = 0; r < 4; r++) raw[r] = srcv[r];
+        } else {
+          uint16_t *e = reinterpret_cast<uint16_t *>(raw);
 #pragma unroll
-        for (int r = 0; r < 32 / kPer; r++) {
-          const TD *e = reinterpret_cast<const TD *>(&raw[r]);
-#pragma unroll
-          for (int q = 0; q < kPer; q++) t[r * kPer + q] = to_f32(e[q]);
+          for (int r = 0; r < 32; r++) {
+            const uint16_t bits = prow[min(sj + r, MW - 1)].v;
+            e[r] = (row_ok && sj + r < MW) ? bits : (uint16_t)0;
+          }
         }
+        uint4 *dstv = reinterpret_cast<uint4 *>(&PtB[a][px0]);
+#pragma unroll
+        for (int r = 0; r < 4; r++) dstv[r] = raw[r];
       } else {
+        float t[32];
+        if (vec_ok && row_ok && sj + 32 <= MW) {
+          constexpr int kPer = 16 / (int)sizeof(TD);  // elements per 16-byte load
+          const uint4 *srcv = reinterpret_cast<const uint4 *>(prow + sj);
+          uint4 raw[32 / kPer];
 #pragma unroll
-        for (int r = 0; r < 32; r++) t[r] = to_f32(prow[min(sj + r, MW - 1)]);
+          for (int r = 0; r < 32 / kPer; r++) raw[r] = srcv[r];
 #pragma unroll
-        for (int r = 0; r < 32; r++) t[r] = (row_ok && sj + r < MW) ? t[r] : 0.f;
+          for (int r = 0; r < 32 / kPer; r++) {
+            const TD *e = reinterpret_cast<const TD *>(&raw[r]);
+#pragma unroll
+            for (int q = 0; q < kPer; q++) t[r * kPer + q] = to_f32(e[q]);
+          }
+        } else {
+#pragma unroll
+          for (int r = 0; r < 32; r++) t[r] = to_f32(prow[min(sj + r, MW - 1)]);
+#pragma unroll
+          for (int r = 0; r < 32; r++) t[r] = (row_ok && sj + r < MW) ? t[r] : 0.f;
+        }
+        float4 *dstv = reinterpret_cast<float4 *>(&Pt[a][px0]);
+#pragma unroll
+        for (int r = 0; r < 8; r++)
+          dstv[r] = float4{t[4 * r], t[4 * r + 1], t[4 * r + 2], t[4 * r + 3]};
       }
-      float4 *dstv = reinterpret_cast<float4 *>(&Pt[a][px0]);
-#pragma unroll
-      for (int r = 0; r < 8; r++) dstv[r] = float4{t[4 * r], t[4 * r + 1], t[4 * r + 2], t[4 * r + 3]};
     }
     __syncthreads();
-    float areg[32];
+    float areg[kBf16 ? 1 : 32];
+    bf16x8 aregb[kBf16 ? 4 : 1];
+    if constexpr (kBf16) {
 #pragma unroll
-    for (int s4 = 0; s4 < 8; s4++) {
-      const float4 t = *reinterpret_cast<const float4 *>(&Pt[wave * 16 + l15][16 * s4 + 4 * lq]);
-      areg[4 * s4 + 0] = t.x;
-      areg[4 * s4 + 1] = t.y;
-      areg[4 * s4 + 2] = t.z;
-      areg[4 * s4 + 3] = t.w;
+      for (int s = 0; s < 4; s++)
+        aregb[s] = __builtin_bit_cast(
+            bf16x8, *reinterpret_cast<const uint4 *>(&PtB[wave * 16 + l15][32 * s + 8 * lq]));
+    } else {
+#pragma unroll
+      for (int s4 = 0; s4 < 8; s4++) {
+        const float4 t =
+            *reinterpret_cast<const float4 *>(&Pt[wave * 16 + l15][16 * s4 + 4 * lq]);
+        areg[4 * s4 + 0] = t.x;
+        areg[4 * s4 + 1] = t.y;
+        areg[4 * s4 + 2] = t.z;
+        areg[4 * s4 + 3] = t.w;
+      }
     }
 
     const int gi = i0 + (p >> tw_shift), gj = j0 + (p & tw_mask);
@@ -476,7 +512,10 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
         float s = 0.f;
 #pragma unroll
         for (int i = 0; i < NE; i++) s = __builtin_fmaf(wt[i], v[ch][i], s);
-        S[buf][half * 8 + ch][p] = s;
+        if constexpr (kBf16)
+          SB[buf][half * 8 + ch][p] = from_f32<bf16_t>(s).v;
+        else
+          S[buf][half * 8 + ch][p] = s;
       }
     };
 
@@ -517,6 +556,15 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
             load_tap(0);
             issue(cb + 1);
           }
+          if constexpr (kBf16) {
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+              const bf16x8 bq = __builtin_bit_cast(
+                  bf16x8, *reinterpret_cast<const uint4 *>(&SB[buf][l15][32 * s + 8 * lq]));
+              acc[k][cb] =
+                  __builtin_amdgcn_mfma_f32_16x16x32_bf16(aregb[s], bq, acc[k][cb], 0, 0, 0);
+            }
+          } else
 #pragma unroll
           for (int s4 = 0; s4 < 8; s4++) {
             const float4 bq = *reinterpret_cast<const float4 *>(&S[buf][l15][16 * s4 + 4 * lq]);
