@@ -19,6 +19,7 @@ from .util import synthetic
 
 HBM_GBS = 8000.0
 FP32_MFMA_TFLOPS = 157.3
+BF16_MFMA_TFLOPS = 2500.0
 FP32_VALU_TFLOPS = 157.3  # vector fp32 FMA peak (packed); KNN is bound by it
 
 
@@ -35,7 +36,7 @@ def _time(fn, iters=10, warmup=2):
     return start.elapsed_time(end) / iters
 
 
-def _line(name, ms, nbytes=None, flops=None, peak_tflops=FP32_MFMA_TFLOPS, **extra):
+def _line(name, ms, nbytes=None, flops=None, peak_tflops=FP32_MFMA_TFLOPS, bound="mfma", **extra):
     out = {"workload": name, "ms": round(ms, 4)}
     if nbytes is not None:
         gbs = nbytes / (ms * 1e-3) / 1e9
@@ -43,9 +44,8 @@ def _line(name, ms, nbytes=None, flops=None, peak_tflops=FP32_MFMA_TFLOPS, **ext
                    frac=round(gbs / HBM_GBS, 4))
     if flops is not None:
         tf = flops / (ms * 1e-3) / 1e12
-        out.update(bound="mfma" if peak_tflops == FP32_MFMA_TFLOPS else "valu",
-                   GFLOP=round(flops / 1e9, 2), achieved_TFLOPs=round(tf, 2),
-                   frac=round(tf / peak_tflops, 4))
+        out.update(bound=bound, peak_TFLOPs=peak_tflops, GFLOP=round(flops / 1e9, 2),
+                   achieved_TFLOPs=round(tf, 2), frac=round(tf / peak_tflops, 4))
     out.update(extra)
     print(json.dumps(out), flush=True)
 
@@ -63,11 +63,13 @@ def config3(dev):
         gy = torch.randn(B, Co, 1, V, generator=g).to(dev, dtype)
         flop = 2.0 * B * V * Co * Ci * K
         tag = "config3 weighted mesh conv %s" % str(dtype).split(".")[-1]
+        peak = BF16_MFMA_TFLOPS if dtype == torch.bfloat16 else FP32_MFMA_TFLOPS
         _line(tag + " forward",
-              _time(lambda: _C.weighted_mapped_conv_forward(x, smap, iw, w, b, K, 0)), flops=flop)
+              _time(lambda: _C.weighted_mapped_conv_forward(x, smap, iw, w, b, K, 0)), flops=flop,
+              peak_tflops=peak)
         _line(tag + " backward",
               _time(lambda: _C.weighted_mapped_conv_backward(gy, smap, iw, x, w, b, K, 0)),
-              flops=2 * flop)
+              flops=2 * flop, peak_tflops=peak)
 
 
 def config4(dev):
@@ -105,7 +107,7 @@ def knn(dev):
     ref = synthetic.sphere_points(40962, seed=1).to(dev)
     qry = synthetic.sphere_points(524288, seed=2).to(dev)
     _line("config4 knn k=8 Q=524288 R=40962", _time(lambda: _C.knn_forward(ref, qry, 8), iters=3, warmup=1),
-          flops=8.0 * 524288 * 40962, peak_tflops=FP32_VALU_TFLOPS)
+          flops=8.0 * 524288 * 40962, peak_tflops=FP32_VALU_TFLOPS, bound="valu")
 
 
 def config5(dev):
@@ -118,11 +120,12 @@ def config5(dev):
     b = torch.zeros(C, device=dev, dtype=torch.bfloat16)
     smap = synthetic.latitude_map(H, W, 2).to(dev)
     flop = 2.0 * B * H * W * C * C * K
-    _line("config5 bf16 conv forward (fp32 MFMA accumulate)",
-          _time(lambda: _C.mapped_conv_forward(x, smap, w, b, K, 1), iters=3, warmup=1), flops=flop)
-    _line("config5 bf16 conv backward (fp32 MFMA accumulate)",
+    _line("config5 bf16 conv forward (bf16 MFMA, fp32 accumulate)",
+          _time(lambda: _C.mapped_conv_forward(x, smap, w, b, K, 1), iters=3, warmup=1), flops=flop,
+          peak_tflops=BF16_MFMA_TFLOPS)
+    _line("config5 bf16 conv backward (bf16 MFMA, fp32 accumulate)",
           _time(lambda: _C.mapped_conv_backward(gy, smap, x, w, b, K, 1), iters=3, warmup=1),
-          flops=2 * flop)
+          flops=2 * flop, peak_tflops=BF16_MFMA_TFLOPS)
 
 
 WORKLOADS = {"config3": config3, "config4": config4, "knn": knn, "config5": config5}
