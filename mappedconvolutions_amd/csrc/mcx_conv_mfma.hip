@@ -394,54 +394,39 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
 
     __syncthreads();  // everyone is done with the previous tile's LDS contents
     {
-      // Each thread stages 32 consecutive tile pixels of one plain channel: with
-      // either tile shape (4 x 32 or 1 x 128) they are contiguous in memory.
-      const int a = tid >> 2, px0 = (tid & 3) * 32;
+      // A row of the plain tile is kLanesPerRow 16-byte pieces; consecutive lanes take
+      // consecutive pieces of a row, so the loads coalesce and the LDS stores of a wave
+      // fall into consecutive banks.  A piece never straddles two image rows (either
+      // tile shape, 4 x 32 or 1 x 128, is made of 32-pixel runs).
+      constexpr int kPer = 16 / (int)sizeof(TD);
+      constexpr int kLanesPerRow = kTilePx / kPer, kRowsPerPass = kThreads / kLanesPerRow;
+      constexpr int kPasses = kWgA / kRowsPerPass;
+      const int px0 = (tid % kLanesPerRow) * kPer;
       const int si = i0 + (px0 >> tw_shift), sj = j0 + (px0 & tw_mask);
-      const bool row_ok = (a0 + a) < A && si < MH;
-      const TD *prow = plain + ((int64_t)b * A + min(a0 + a, A - 1)) * N +
-                       (int64_t)min(si, MH - 1) * MW;
-      if constexpr (kBf16) {
-        uint4 raw[4];
-        if (vec_ok && row_ok && sj + 32 <= MW) {
-          const uint4 *srcv = reinterpret_cast<const uint4 *>(prow + sj);
+      uint4 raw[kPasses];
 #pragma unroll
-          for (int r = 0; r < 4; r++) raw[r] = srcv[r];
+      for (int r = 0; r < kPasses; r++) {
+        const int a = tid / kLanesPerRow + r * kRowsPerPass;
+        const bool row_ok = (a0 + a) < A && si < MH;
+        const TD *prow = plain + ((int64_t)b * A + min(a0 + a, A - 1)) * N +
+                         (int64_t)min(si, MH - 1) * MW;
+        if (vec_ok && row_ok && sj + kPer <= MW) {
+          raw[r] = *reinterpret_cast<const uint4 *>(prow + sj);
         } else {
-          uint16_t *e = reinterpret_cast<uint16_t *>(raw);
+          TD e[kPer];
 #pragma unroll
-          for (int r = 0; r < 32; r++) {
-            const uint16_t bits = prow[min(sj + r, MW - 1)].v;
-            e[r] = (row_ok && sj + r < MW) ? bits : (uint16_t)0;
-          }
+          for (int q = 0; q < kPer; q++)
+            e[q] = (row_ok && sj + q < MW) ? prow[min(sj + q, MW - 1)] : TD{};
+          raw[r] = *reinterpret_cast<const uint4 *>(e);
         }
-        uint4 *dstv = reinterpret_cast<uint4 *>(&PtB[a][px0]);
+      }
 #pragma unroll
-        for (int r = 0; r < 4; r++) dstv[r] = raw[r];
-      } else {
-        float t[32];
-        if (vec_ok && row_ok && sj + 32 <= MW) {
-          constexpr int kPer = 16 / (int)sizeof(TD);  // elements per 16-byte load
-          const uint4 *srcv = reinterpret_cast<const uint4 *>(prow + sj);
-          uint4 raw[32 / kPer];
-#pragma unroll
-          for (int r = 0; r < 32 / kPer; r++) raw[r] = srcv[r];
-#pragma unroll
-          for (int r = 0; r < 32 / kPer; r++) {
-            const TD *e = reinterpret_cast<const TD *>(&raw[r]);
-#pragma unroll
-            for (int q = 0; q < kPer; q++) t[r * kPer + q] = to_f32(e[q]);
-          }
-        } else {
-#pragma unroll
-          for (int r = 0; r < 32; r++) t[r] = to_f32(prow[min(sj + r, MW - 1)]);
-#pragma unroll
-          for (int r = 0; r < 32; r++) t[r] = (row_ok && sj + r < MW) ? t[r] : 0.f;
-        }
-        float4 *dstv = reinterpret_cast<float4 *>(&Pt[a][px0]);
-#pragma unroll
-        for (int r = 0; r < 8; r++)
-          dstv[r] = float4{t[4 * r], t[4 * r + 1], t[4 * r + 2], t[4 * r + 3]};
+      for (int r = 0; r < kPasses; r++) {
+        const int a = tid / kLanesPerRow + r * kRowsPerPass;
+        if constexpr (kBf16)
+          *reinterpret_cast<uint4 *>(&PtB[a][px0]) = raw[r];
+        else
+          *reinterpret_cast<uint4 *>(&Pt[a][px0]) = raw[r];
       }
     }
     __syncthreads();
