@@ -50,8 +50,9 @@ template <>
 int fill_zero<double>(double *p, int64_t n, hipStream_t s) { return fill_f64(p, n, 0.0, s); }
 
 // ---- scratch sizes of the three operators -------------------------------------------
-size_t gather_product_ws(int dtype, int64_t G, int64_t O, int64_t K, int64_t P) {
-  return use_mfma(dtype, P) ? mfma_gather_product_bytes(O, G, K) : 0;
+size_t gather_product_ws(int dtype, int64_t G, int64_t O, int64_t K, int64_t P, int64_t B,
+                         int64_t SH, int64_t SW) {
+  return use_mfma(dtype, P) ? mfma_gather_product_bytes(O, G, K, B, SH, SW) : 0;
 }
 size_t weight_grad_ws(int dtype, int64_t B, int64_t A, int64_t G, int64_t MH, int64_t MW,
                       int64_t K, int64_t P) {
@@ -146,7 +147,7 @@ int gather_product<float>(bool mfma, const void *src, const void *map, const voi
     return generic_gather_product<float>((const float *)src, (const float *)map,
                                          (const float *)iw, (const float *)w, (const float *)bias,
                                          (float *)y, B, G, O, SH, SW, MH * MW, K, P, interp, s);
-  if (!ws || ws_bytes < mfma_gather_product_bytes(O, G, K)) return MCX_E_WORKSPACE;
+  if (!ws || ws_bytes < mfma_gather_product_bytes(O, G, K, B, SH, SW)) return MCX_E_WORKSPACE;
   return mfma_gather_product<float>((const float *)src, (const float *)map, (const float *)iw,
                                     (const float *)w, (const float *)bias, (float *)y, ws, B, G, O,
                                     SH, SW, MH, MW, K, P, interp, s);
@@ -201,7 +202,7 @@ int gather_product<bf16_t>(bool mfma, const void *src, const void *map, const vo
                            int64_t B, int64_t G, int64_t O, int64_t SH, int64_t SW, int64_t MH,
                            int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s) {
   if (!mfma) return MCX_E_DTYPE;
-  if (!ws || ws_bytes < mfma_gather_product_bytes(O, G, K)) return MCX_E_WORKSPACE;
+  if (!ws || ws_bytes < mfma_gather_product_bytes(O, G, K, B, SH, SW)) return MCX_E_WORKSPACE;
   return mfma_gather_product<bf16_t>((const bf16_t *)src, (const float *)map, (const float *)iw,
                                      (const bf16_t *)w, (const bf16_t *)bias, (bf16_t *)y, ws, B,
                                      G, O, SH, SW, MH, MW, K, P, interp, s);
@@ -296,9 +297,10 @@ int tconv_backward_t(bool mfma, const void *gy, const void *map, const void *iw,
 
 }  // namespace
 
-extern "C" size_t mcx_conv_forward_workspace(int64_t, int64_t Ci, int64_t Co, int64_t, int64_t,
-                                             int64_t, int64_t, int64_t K, int64_t P, int dtype) {
-  return gather_product_ws(dtype, Ci, Co, K, P);
+extern "C" size_t mcx_conv_forward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t IH,
+                                             int64_t IW, int64_t, int64_t, int64_t K, int64_t P,
+                                             int dtype) {
+  return gather_product_ws(dtype, Ci, Co, K, P, B, IH, IW);
 }
 
 extern "C" int mcx_conv_forward(const void *x, const void *map, const void *iw, const void *w,
@@ -366,7 +368,7 @@ extern "C" size_t mcx_tconv_backward_workspace(int64_t B, int64_t Ci, int64_t Co
                                                int64_t P, int dtype) {
   // backward-input is a gather-product with the channel roles swapped; the
   // gradients run one after the other and share the scratch
-  return std::max({gather_product_ws(dtype, Co, Ci, K, P),
+  return std::max({gather_product_ws(dtype, Co, Ci, K, P, B, OH, OW),
                    weight_grad_ws(dtype, B, Ci, Co, IH, IW, K, P),
                    bias_grad_ws(dtype, B, Co, OH * OW)});
 }

@@ -78,6 +78,31 @@ __global__ void pack_weights_bf16_kernel(const TD *__restrict__ w, uint16_t *__r
   }
 }
 
+// x[b][g][n] -> xt[b][n][Gpad] (channels past G zero): 64 pixels x 64 channels per
+// workgroup through LDS, coalesced on both sides.
+template <typename TD>
+__global__ __launch_bounds__(256) void to_channel_last_kernel(const TD *__restrict__ x,
+                                                              TD *__restrict__ xt, int G, int Gpad,
+                                                              int64_t plane) {
+  __shared__ TD tile[64][65];
+  const int64_t n0 = (int64_t)blockIdx.x * 64;
+  const int g0 = blockIdx.y * 64, b = blockIdx.z;
+  const int lx = threadIdx.x & 63, ly = threadIdx.x >> 6;
+#pragma unroll
+  for (int r = 0; r < 16; r++) {
+    const int g = g0 + ly + 4 * r;
+    const int64_t n = n0 + lx;
+    tile[ly + 4 * r][lx] = (g < G && n < plane) ? x[((int64_t)b * G + g) * plane + n] : TD{};
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < 16; r++) {
+    const int64_t n = n0 + ly + 4 * r;
+    const int g = g0 + lx;
+    if (n < plane && g < Gpad) xt[((int64_t)b * plane + n) * Gpad + g] = tile[lx][ly + 4 * r];
+  }
+}
+
 // LDS operand tiles of the gather-product kernel, double-buffered.
 template <typename TD>
 struct OperandTiles {  // fp32: samples S[chunk channel][pixel], weights Wt[chunk channel][o]
@@ -92,7 +117,11 @@ struct OperandTiles<bf16_t> {  // bf16: 16-byte groups of 8 channels, [kg][pixel
 
 // OG: groups of 64 output channels per workgroup (2 only with bf16 storage, where the
 // gather, not the MFMA, bounds the kernel and is shared by twice the outputs).
-template <typename TD, int NCORN, int NP, int OG>
+// CL: `src` is a channel-last copy [B][SH*SW][Gpad] of the source (made by
+// to_channel_last_kernel): a sample's 8 channels are then one or two 16-byte loads from
+// one cache line instead of 8 loads from 8 lines.  Used for single-row sources (mesh
+// signals), whose maps point anywhere.
+template <typename TD, int NCORN, int NP, int OG, bool CL>
 __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma_kernel(
     const TD *__restrict__ src, const float *__restrict__ map, const float *__restrict__ iw,
     const float *__restrict__ wp, const TD *__restrict__ bias, TD *__restrict__ y, int G,
@@ -129,7 +158,7 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
   const bool live = gi < OH && gj < OW;
   const int64_t n_g = live ? (int64_t)gi * OW + gj : 0;
 
-  const TD *src_b = src + (int64_t)b * G * plane;
+  const TD *src_b = src + (int64_t)b * (CL ? Gpad : G) * plane;
   const int chunks = Gpad / kGC;
 
   unsigned off[NE];
@@ -154,16 +183,38 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
   const TD *pl[8];
   auto set_chunk = [&](int c) {
     const int g0 = c * kGC + half * 8;
+    if constexpr (CL) {
+      pl[0] = src_b + g0;  // the 8 channels are contiguous; offsets select the pixel row
+    } else {
 #pragma unroll
-    for (int ch = 0; ch < 8; ch++)  // padded channels read a valid plane, weights are 0
-      pl[ch] = src_b + (int64_t)min(g0 + ch, G - 1) * plane;
+      for (int ch = 0; ch < 8; ch++)  // padded channels read a valid plane, weights are 0
+        pl[ch] = src_b + (int64_t)min(g0 + ch, G - 1) * plane;
+    }
   };
   auto issue = [&](int k, int c) {
 #pragma unroll
     for (int i = 0; i < NE; i++) {
       if (!((tmask >> i) & 1u)) continue;  // wave-uniform
+      if constexpr (CL) {
+        const char *row = reinterpret_cast<const char *>(pl[0]) + off[i];
+        if constexpr (kBf16) {
+          const uint4 q = *reinterpret_cast<const uint4 *>(row);
+          const unsigned w4[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
-      for (int ch = 0; ch < 8; ch++) v[ch][i] = load_at(pl[ch], off[i]);
+          for (int j = 0; j < 4; j++) {
+            v[2 * j][i] = __builtin_bit_cast(float, w4[j] << 16);
+            v[2 * j + 1][i] = __builtin_bit_cast(float, w4[j] & 0xffff0000u);
+          }
+        } else {
+          const float4 q0 = reinterpret_cast<const float4 *>(row)[0];
+          const float4 q1 = reinterpret_cast<const float4 *>(row)[1];
+          v[0][i] = q0.x; v[1][i] = q0.y; v[2][i] = q0.z; v[3][i] = q0.w;
+          v[4][i] = q1.x; v[5][i] = q1.y; v[6][i] = q1.z; v[7][i] = q1.w;
+        }
+      } else {
+#pragma unroll
+        for (int ch = 0; ch < 8; ch++) v[ch][i] = load_at(pl[ch], off[i]);
+      }
     }
     if constexpr (kBf16) {
       // weights of this chunk: two runs (kg = 0, 1) of 64*OG x 16 bytes, 8*OG bytes per thread
@@ -238,7 +289,7 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
                                          live ? (weighted ? iw[e] : 1.f) : 0.f, t);
 #pragma unroll
         for (int i = 0; i < NCORN; i++) {
-          TapOff[kl][p][sp * NCORN + i] = t.off[i];
+          TapOff[kl][p][sp * NCORN + i] = CL ? t.off[i] * (unsigned)Gpad : t.off[i];
           TapWt[kl][p][sp * NCORN + i] = t.wt[i];
           if (__builtin_amdgcn_ballot_w64(t.wt[i] != 0.f)) m |= 1u << (sp * NCORN + i);
         }
@@ -998,23 +1049,51 @@ inline ModeArgs mode_args(int interp, int64_t P) {
     }                                  \
   }
 
+// Channel-last staging of the source pays when neighbouring map entries point to unrelated
+// source pixels; that is taken to be the case for single-row sources (mesh signals stored
+// as [1, V] images) sampled with nearest interpolation.
+inline bool use_channel_last(int64_t SH, int interp) {
+  return SH == 1 && canonical_interp(interp) == kInterpNearest;
+}
+
+// `stage`: room for the channel-last copy (B * SH * SW * Gpad elements) when
+// use_channel_last(SH, interp), unused otherwise.
 template <typename TD>
 int launch_gather_product(const TD *src, const float *map, const float *iw, const float *wp,
-                          const TD *bias, TD *y, int64_t B, int64_t G, int64_t O, int64_t SH,
-                          int64_t SW, int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
-                          const int *gate, int run_if_zero, hipStream_t s) {
+                          const TD *bias, TD *y, TD *stage, int64_t B, int64_t G, int64_t O,
+                          int64_t SH, int64_t SW, int64_t OH, int64_t OW, int64_t K, int64_t P,
+                          int interp, const int *gate, int run_if_zero, hipStream_t s) {
   const int Opad = (int)round_up(O, kOT), Gpad = (int)round_up(G, kGC);
+  const bool cl = stage != nullptr && use_channel_last(SH, interp) &&
+                  SH * SW * Gpad * (int64_t)sizeof(TD) <= 0xffffffffLL;
+  if (cl) {
+    dim3 tg((unsigned)((SH * SW + 63) / 64), (unsigned)((Gpad + 63) / 64), (unsigned)B);
+    hipLaunchKernelGGL(to_channel_last_kernel<TD>, tg, dim3(256), 0, s, src, stage, (int)G, Gpad,
+                       SH * SW);
+    MCX_HIP_CHECK_LAUNCH();
+    src = stage;
+  }
   const PixelTiling t = make_tiling(B, OH, OW);
   if (t.total > 0x7fffffffLL) return MCX_E_SHAPE;
   // bf16 storage with at least 128 output channels: 128 outputs per workgroup
   const bool wide = sizeof(TD) == 2 && Opad % (2 * kOT) == 0;
   dim3 grid((unsigned)t.total, (unsigned)(Opad / (wide ? 2 * kOT : kOT)));
   const ModeArgs m = mode_args(interp, P);
-#define MCX_LAUNCH_OG(NCORN, NP, OG)                                                             \
-  hipLaunchKernelGGL((gather_product_mfma_kernel<TD, NCORN, NP, OG>), grid, dim3(kThreads), 0,   \
-                     s, src, map, iw, wp, bias, y, (int)G, (int)O, Opad, Gpad, (int)SH, (int)SW, \
-                     (int)OH, (int)OW, (int)K, m.weighted, m.wrap, t.tiles_x, t.tiles_per_img,   \
-                     t.tw_shift, gate, run_if_zero)
+#define MCX_LAUNCH_CL(NCORN, NP, OG, CL)                                                         \
+  hipLaunchKernelGGL((gather_product_mfma_kernel<TD, NCORN, NP, OG, CL>), grid, dim3(kThreads),  \
+                     0, s, src, map, iw, wp, bias, y, (int)G, (int)O, Opad, Gpad, (int)SH,       \
+                     (int)SW, (int)OH, (int)OW, (int)K, m.weighted, m.wrap, t.tiles_x,           \
+                     t.tiles_per_img, t.tw_shift, gate, run_if_zero)
+#define MCX_LAUNCH_OG(NCORN, NP, OG)           \
+  if constexpr (NCORN == 1) {                  \
+    if (cl) {                                  \
+      MCX_LAUNCH_CL(NCORN, NP, OG, true);      \
+    } else {                                   \
+      MCX_LAUNCH_CL(NCORN, NP, OG, false);     \
+    }                                          \
+  } else {                                     \
+    MCX_LAUNCH_CL(NCORN, NP, OG, false);       \
+  }
 #define MCX_LAUNCH(NCORN, NP)                               \
   if constexpr (sizeof(TD) == 2) {                          \
     if (wide) {                                             \
@@ -1028,6 +1107,7 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
   MCX_DISPATCH_TAPS(m, MCX_LAUNCH)
 #undef MCX_LAUNCH
 #undef MCX_LAUNCH_OG
+#undef MCX_LAUNCH_CL
   MCX_HIP_CHECK_LAUNCH();
   return 0;
 }
@@ -1052,20 +1132,29 @@ int launch_pack_weights(const TD *w, float *wp, int64_t O, int64_t G, int64_t K,
 }  // namespace
 
 // ---- gather-product --------------------------------------------------------------
-size_t mfma_gather_product_bytes(int64_t O, int64_t G, int64_t K) {
-  return align256((size_t)(K * round_up(G, kGC) * round_up(O, kOT)) * sizeof(float));
+// Packed weights, then (single-row sources) the channel-last copy of the source, sized
+// for 4-byte elements.
+size_t mfma_gather_product_bytes(int64_t O, int64_t G, int64_t K, int64_t B, int64_t SH,
+                                 int64_t SW) {
+  size_t n = align256((size_t)(K * round_up(G, kGC) * round_up(O, kOT)) * sizeof(float));
+  if (SH == 1) n += align256((size_t)(B * SH * SW * round_up(G, kGC)) * sizeof(float));
+  return n;
 }
 
-// scratch: mfma_gather_product_bytes(O, G, K) bytes (packed weights).
+// scratch: mfma_gather_product_bytes(...) bytes.
 template <typename TD>
 int mfma_gather_product(const TD *src, const float *map, const float *iw, const TD *w,
                         const TD *bias, TD *y, void *scratch, int64_t B, int64_t G, int64_t O,
                         int64_t SH, int64_t SW, int64_t OH, int64_t OW, int64_t K, int64_t P,
                         int interp, hipStream_t s) {
   float *wp = (float *)scratch;
+  TD *stage = SH == 1 ? reinterpret_cast<TD *>(
+                            (char *)scratch +
+                            align256((size_t)(K * round_up(G, kGC) * round_up(O, kOT)) * 4))
+                      : nullptr;
   if (int rc = launch_pack_weights<TD>(w, wp, O, G, K, 0, s)) return rc;
-  return launch_gather_product<TD>(src, map, iw, wp, bias, y, B, G, O, SH, SW, OH, OW, K, P,
-                                   interp, nullptr, 0, s);
+  return launch_gather_product<TD>(src, map, iw, wp, bias, y, stage, B, G, O, SH, SW, OH, OW, K,
+                                   P, interp, nullptr, 0, s);
 }
 
 // ---- weight gradient ---------------------------------------------------------------
@@ -1246,7 +1335,8 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
                          (int)MW, (int)K, entries);
     MCX_HIP_CHECK_LAUNCH();
     if (int rc = launch_pack_weights<TD>(w, wpt, D, S, K, 1, s)) return rc;
-    if (int rc = launch_gather_product<TD>(src, tmap, tiw, wpt, bias, dst, B, S, D, MH, MW, DH,
+    if (int rc = launch_gather_product<TD>(src, tmap, tiw, wpt, bias, dst, (TD *)nullptr, B, S, D,
+                                           MH, MW, DH,
                                            DW, K, kTransSlots, kInterpNearest, gate, 1, s))
       return rc;
   }
