@@ -54,7 +54,7 @@ __global__ __launch_bounds__(kThreads) void knn_kernel(const T *__restrict__ ref
     bi[j] = 0;
   }
 
-  for (int r = 0; r < R; r++) {
+  auto ssd_of = [&](int r) {
     T ssd = T(0);
     if (DT > 0) {
 #pragma unroll
@@ -68,6 +68,9 @@ __global__ __launch_bounds__(kThreads) void knn_kernel(const T *__restrict__ ref
         ssd = fma_t(t, t, ssd);
       }
     }
+    return ssd;
+  };
+  auto insert = [&](T ssd, int r) {
     if (ssd < bd[KMAX - 1]) {
       T cd = ssd;
       int ci = r + 1;
@@ -85,7 +88,25 @@ __global__ __launch_bounds__(kThreads) void knn_kernel(const T *__restrict__ ref
         }
       }
     }
+  };
+  // Reference points are taken kBatch at a time: their distances are independent work
+  // (the wave-uniform loads of the next points overlap the arithmetic), and a single
+  // comparison of the batch minimum decides whether any lane has to insert at all.
+  constexpr int kBatch = 8;
+  int r = 0;
+  for (; r + kBatch <= R; r += kBatch) {
+    T ssd[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; u++) ssd[u] = ssd_of(r + u);
+    T m = ssd[0];
+#pragma unroll
+    for (int u = 1; u < kBatch; u++) m = ssd[u] < m ? ssd[u] : m;
+    if (m < bd[KMAX - 1]) {
+#pragma unroll
+      for (int u = 0; u < kBatch; u++) insert(ssd[u], r + u);  // in index order: ties keep it
+    }
   }
+  for (; r < R; r++) insert(ssd_of(r), r);
   if (!live) return;
 #pragma unroll
   for (int j = 0; j < KMAX; j++) {
