@@ -638,8 +638,17 @@ __global__ void reduce_partials_kernel(const float *__restrict__ part, TD *__res
                                        int ranges, int64_t n) {
   const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (e >= n) return;
+  // eight loads in flight per thread; the order of the additions is fixed
   float s = 0.f;
-  for (int r = 0; r < ranges; r++) s += part[(int64_t)r * n + e];
+  int r = 0;
+  for (; r + 8 <= ranges; r += 8) {
+    float t[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) t[u] = part[(int64_t)(r + u) * n + e];
+#pragma unroll
+    for (int u = 0; u < 8; u++) s += t[u];
+  }
+  for (; r < ranges; r++) s += part[(int64_t)r * n + e];
   out[e] = from_f32<TD>(s);
 }
 
@@ -1187,8 +1196,8 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
 #undef MCX_LAUNCH
   MCX_HIP_CHECK_LAUNCH();
   const int64_t n = A * G * K;
-  hipLaunchKernelGGL(reduce_partials_kernel<TD>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
-                     s, part, gw, ranges, n);
+  hipLaunchKernelGGL(reduce_partials_kernel<TD>, dim3((unsigned)((n + 63) / 64)), dim3(64), 0, s,
+                     part, gw, ranges, n);
   MCX_HIP_CHECK_LAUNCH();
   return 0;
 }
