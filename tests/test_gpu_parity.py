@@ -321,6 +321,87 @@ def test_config3_weighted_mesh_conv(dtype, device):
         assert rel_err(a.float(), r) < tol, nm
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("p", [0, 3])
+def test_mesh_conv_ragged_channels(dtype, p, device):
+    """Single-row (mesh) source with channel counts that are no multiple of 16 and an output
+    count past one 64-channel group: the channel-last staging pads with zeros, taps outside
+    [0, V) contribute nothing.  Forward, backward and the transposed convolution."""
+    B, Ci, Co, V, K = 2, 20, 70, 777, 5
+    g = torch.Generator().manual_seed(31 + p)
+    smap, iw = helpers.random_map(g, 1, V, K, p, 1, V, torch.float32, integer=True)
+    x = torch.randn(B, Ci, 1, V, generator=g).to(dtype)
+    w = (torch.randn(Co, Ci, K, generator=g) / (Ci * K) ** 0.5).to(dtype)
+    b = torch.randn(Co, generator=g).to(dtype)
+    gy = torch.randn(B, Co, 1, V, generator=g).to(dtype)
+    y_o = O.weighted_mapped_conv_forward(x.float(), smap, iw, w.float(), b.float(), K, 0)
+    g_o = O.weighted_mapped_conv_backward(gy.float(), smap, iw, x.float(), w.float(), b.float(),
+                                          K, 0)
+    xd, sd, id_, wd_, bd, gyd = dev(x, smap, iw, w, b, gy)
+    if p:
+        y = _C.weighted_mapped_conv_forward(xd, sd, id_, wd_, bd, K, 0)
+        gr = _C.weighted_mapped_conv_backward(gyd, sd, id_, xd, wd_, bd, K, 0)
+    else:
+        y = _C.mapped_conv_forward(xd, sd, wd_, bd, K, 0)
+        gr = _C.mapped_conv_backward(gyd, sd, xd, wd_, bd, K, 0)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    assert rel_err(y.float(), y_o) < tol
+    for a, r, nm in zip(gr, g_o, ("grad_input", "grad_weight", "grad_bias")):
+        assert rel_err(a.float(), r) < tol, nm
+    # transposed convolution: its backward-input is the gather-product over grad_output
+    wt = (torch.randn(Ci, Co, K, generator=g) / (Ci * K) ** 0.5).to(dtype)
+    t_o = O.weighted_mapped_transposed_conv_backward(gy.float(), smap, iw, x.float(), wt.float(),
+                                                     b.float(), K, 0)
+    if p:
+        t = _C.weighted_mapped_transposed_conv_backward(gyd, sd, id_, xd, wt.cuda(), bd, K, 0)
+    else:
+        t = _C.mapped_transposed_conv_backward(gyd, sd, xd, wt.cuda(), bd, K, 0)
+    for a, r, nm in zip(t, t_o, ("grad_input", "grad_weight", "grad_bias")):
+        assert rel_err(a.float(), r) < tol, "transposed " + nm
+
+
+@pytest.mark.parametrize("co", [128, 192, 130])
+def test_conv_bf16_wide_outputs(co, device):
+    """bf16 storage with 128 output channels per workgroup (Co = 128), with Co padded to a
+    multiple of 64 but not of 128 (192) and ragged (130), input channels ragged too."""
+    B, Ci, H, W, K = 1, 40, 12, 40, 9
+    g = torch.Generator().manual_seed(co)
+    smap = synthetic.latitude_map(H, W, 1)
+    x = torch.randn(B, Ci, H, W, generator=g).bfloat16()
+    w = (torch.randn(co, Ci, K, generator=g) / (Ci * K) ** 0.5).bfloat16()
+    b = torch.randn(co, generator=g).bfloat16()
+    gy = torch.randn(B, co, H, W, generator=g).bfloat16()
+    y_o = O.mapped_conv_forward(x.float(), smap, w.float(), b.float(), K, 1)
+    g_o = O.mapped_conv_backward(gy.float(), smap, x.float(), w.float(), b.float(), K, 1)
+    y = _C.mapped_conv_forward(x.cuda(), smap.cuda(), w.cuda(), b.cuda(), K, 1)
+    gr = _C.mapped_conv_backward(gy.cuda(), smap.cuda(), x.cuda(), w.cuda(), b.cuda(), K, 1)
+    assert rel_err(y.float(), y_o) < 2e-2
+    for a, r, nm in zip(gr, g_o, ("grad_input", "grad_weight", "grad_bias")):
+        assert rel_err(a.float(), r) < 2e-2, nm
+
+
+def test_scatter_forms_many_to_one(device):
+    """Every source pixel lands on the same few destination pixels: destination lists far
+    longer than the length up to which they are sorted, empty lists everywhere else."""
+    B, C, IH, IW, OH, OW = 2, 5, 40, 50, 6, 7
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(B, C, IH, IW, generator=g)
+    smap = torch.zeros(IH, IW, 2)
+    smap[..., 0] = 2.25
+    smap[..., 1] = 3.5
+    smap[::7, ::5, 0] = 5.0   # a few land elsewhere, some outside
+    smap[::9, ::4, 1] = 40.0
+    for interp in (0, 1, 2):
+        want = O.resample_to_map(x, smap, OH, OW, interp)
+        got = _C.resample_to_map(x.cuda(), smap.cuda(), OH, OW, interp)
+        assert rel_err(got, want) < 1e-5
+    K = 3
+    pmap = smap[:, :, None, :].repeat(1, 1, K, 1).contiguous()
+    gy = torch.randn(B, C, IH, IW, generator=g)
+    want = O.mapped_avg_unpool(gy, pmap, OH, OW, K, 1)
+    assert rel_err(_C.mapped_avg_unpool(gy.cuda(), pmap.cuda(), OH, OW, K, 1), want) < 1e-5
+
+
 @pytest.mark.parametrize("interp", [1, 2])
 def test_config4_cube_resample_and_pools(interp, device):
     """Cube map [B, C, F, 6F] -> equirect [2F, 4F] through the exact gnomonic map:
@@ -510,7 +591,7 @@ def test_knn_vs_oracle(dtype, k, device):
 def test_knn_other_dimensions(device):
     for D in (1, 2, 4, 6):
         g = torch.Generator().manual_seed(D)
-        ref = torch.randn(1, D, 300, generator=g)
+        ref = torch.randn(1, D, 299 + D, generator=g)   # not a multiple of the batch of 8
         qry = torch.randn(1, D, 260, generator=g)
         io, do = O.knn_forward(ref, qry, 5)
         i, d = knn(ref.cuda(), qry.cuda(), 5)
