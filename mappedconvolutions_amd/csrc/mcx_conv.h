@@ -47,7 +47,7 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
                      void *scratch, int64_t B, int64_t A, int64_t G, int64_t GH, int64_t GW,
                      int64_t MH, int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s);
 size_t mfma_product_scatter_bytes(int64_t B, int64_t S, int64_t D, int64_t K, int64_t DH,
-                                  int64_t DW, size_t elem);
+                                  int64_t DW, size_t elem, int64_t MH, int64_t MW, int64_t P);
 template <typename TD>
 int mfma_product_scatter(const TD *src, const float *map, const float *iw, const TD *w,
                          const TD *bias, TD *dst, void *scratch, int64_t B, int64_t S, int64_t D,

@@ -59,8 +59,10 @@ size_t weight_grad_ws(int dtype, int64_t B, int64_t A, int64_t G, int64_t MH, in
   return use_mfma(dtype, P) ? mfma_weight_grad_bytes(B, A, G, MH, MW, K) : 0;
 }
 size_t product_scatter_ws(int dtype, int64_t B, int64_t S, int64_t D, int64_t K, int64_t P,
-                          int64_t DH, int64_t DW) {
-  return use_mfma(dtype, P) ? mfma_product_scatter_bytes(B, S, D, K, DH, DW, elem_size(dtype)) : 0;
+                          int64_t DH, int64_t DW, int64_t MH, int64_t MW) {
+  return use_mfma(dtype, P)
+             ? mfma_product_scatter_bytes(B, S, D, K, DH, DW, elem_size(dtype), MH, MW, P)
+             : 0;
 }
 size_t bias_grad_ws(int dtype, int64_t B, int64_t C, int64_t N) {
   if (dtype == MCX_BF16) return mfma_bias_grad_bytes(B, C, N);
@@ -166,7 +168,8 @@ int product_scatter<float>(bool mfma, const void *src, const void *map, const vo
                                           (const float *)iw, (const float *)w, (float *)dst, B, S,
                                           D, DH, DW, MH * MW, K, P, interp, s);
   }
-  if (!ws || ws_bytes < mfma_product_scatter_bytes(B, S, D, K, DH, DW, 4)) return MCX_E_WORKSPACE;
+  if (!ws || ws_bytes < mfma_product_scatter_bytes(B, S, D, K, DH, DW, 4, MH, MW, P))
+    return MCX_E_WORKSPACE;
   return mfma_product_scatter<float>((const float *)src, (const float *)map, (const float *)iw,
                                      (const float *)w, (const float *)bias, (float *)dst, ws, B, S,
                                      D, DH, DW, MH, MW, K, P, interp, s);
@@ -214,7 +217,8 @@ int product_scatter<bf16_t>(bool mfma, const void *src, const void *map, const v
                             int64_t B, int64_t S, int64_t D, int64_t DH, int64_t DW, int64_t MH,
                             int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s) {
   if (!mfma) return MCX_E_DTYPE;
-  if (!ws || ws_bytes < mfma_product_scatter_bytes(B, S, D, K, DH, DW, 2)) return MCX_E_WORKSPACE;
+  if (!ws || ws_bytes < mfma_product_scatter_bytes(B, S, D, K, DH, DW, 2, MH, MW, P))
+    return MCX_E_WORKSPACE;
   return mfma_product_scatter<bf16_t>((const bf16_t *)src, (const float *)map, (const float *)iw,
                                       (const bf16_t *)w, (const bf16_t *)bias, (bf16_t *)dst, ws,
                                       B, S, D, DH, DW, MH, MW, K, P, interp, s);
@@ -323,7 +327,7 @@ extern "C" size_t mcx_conv_backward_workspace(int64_t B, int64_t Ci, int64_t Co,
                                               int64_t P, int dtype) {
   // the gradients run one after the other on the stream and share the scratch
   return std::max({weight_grad_ws(dtype, B, Co, Ci, OH, OW, K, P),
-                   product_scatter_ws(dtype, B, Co, Ci, K, P, IH, IW),
+                   product_scatter_ws(dtype, B, Co, Ci, K, P, IH, IW, OH, OW),
                    bias_grad_ws(dtype, B, Co, OH * OW)});
 }
 
@@ -342,10 +346,10 @@ extern "C" int mcx_conv_backward(const void *gy, const void *map, const void *iw
                                                workspace_bytes, d, interp, s));
 }
 
-extern "C" size_t mcx_tconv_forward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t, int64_t,
-                                              int64_t OH, int64_t OW, int64_t K, int64_t P,
-                                              int dtype) {
-  return product_scatter_ws(dtype, B, Ci, Co, K, P, OH, OW);
+extern "C" size_t mcx_tconv_forward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t IH,
+                                              int64_t IW, int64_t OH, int64_t OW, int64_t K,
+                                              int64_t P, int dtype) {
+  return product_scatter_ws(dtype, B, Ci, Co, K, P, OH, OW, IH, IW);
 }
 
 extern "C" int mcx_tconv_forward(const void *x, const void *map, const void *iw, const void *w,

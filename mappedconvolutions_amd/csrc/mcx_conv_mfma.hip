@@ -1216,12 +1216,22 @@ namespace {
 // kernel instead (both kernels are always enqueued; the flag gates them on the device).
 constexpr int kTransSlots = 4;
 
+// A contribution that finds its cell full goes to the overflow list (destination pixel,
+// source pixel, tap, weight), applied afterwards with atomics by overflow_scatter_kernel;
+// only when that list is full too (or there is none) the flag sends the whole product to
+// the scatter kernel.
+struct OverflowEntry {
+  int p, n, k;
+  float wt;
+};
+
 template <int NCORN>
 __global__ void build_transposed_map_kernel(const float *__restrict__ map,
                                             const float *__restrict__ iw, int *__restrict__ cnt,
                                             float *__restrict__ tmap, float *__restrict__ tiw,
-                                            int *__restrict__ overflow, int np, int weighted,
-                                            int wrap, int DH, int DW, int MW, int K,
+                                            int *__restrict__ overflow,
+                                            OverflowEntry *__restrict__ ovf, int ovf_cap, int np,
+                                            int weighted, int wrap, int DH, int DW, int MW, int K,
                                             int64_t total) {
   const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (e >= total) return;
@@ -1243,8 +1253,45 @@ __global__ void build_transposed_map_kernel(const float *__restrict__ map,
         tmap[(cell * kTransSlots + slot) * 2 + 1] = ny;
         tiw[cell * kTransSlots + slot] = t.wt[c];
       } else {
-        *overflow = 1;  // benign race: every writer stores the same value
+        // overflow[0]: flag, overflow[1]: length of the overflow list
+        const int pos = ovf_cap > 0 ? atomicAdd(&overflow[1], 1) : 0;
+        if (pos < ovf_cap)
+          ovf[pos] = OverflowEntry{t.yy[c] * DW + t.xx[c], (int)n, k, t.wt[c]};
+        else
+          overflow[0] = 1;  // benign race: every writer stores the same value
       }
+    }
+  }
+}
+
+// dst[b, d, p] += wt * sum_s W[s, d, k] * src[b, s, n] for every overflow entry: one wave
+// per (entry, image), a lane per destination channel.  `wp` holds the weights packed as
+// Wp[k][s][d] (the gather-product layout); `src_cl`, when not null, is the channel-last copy
+// [B][MN][Spad] of the source, else src is [B][S][MN].  A fixed grid walks the list, so an
+// empty list costs one launch of idle workgroups.
+__global__ __launch_bounds__(64) void overflow_scatter_kernel(
+    const float *__restrict__ src, const float *__restrict__ src_cl,
+    const float *__restrict__ wp, float *__restrict__ dst,
+    const OverflowEntry *__restrict__ ovf, const int *__restrict__ overflow, int ovf_cap, int S,
+    int Spad, int D, int Dpad, int64_t MN, int64_t DN) {
+  if (overflow[0] != 0) return;  // the scatter kernel does the whole product
+  const int count = min(overflow[1], ovf_cap);
+  const int b = blockIdx.y, lane = threadIdx.x;
+  for (int e = blockIdx.x; e < count; e += gridDim.x) {
+    const OverflowEntry en = ovf[e];
+    const float *wk = wp + (int64_t)en.k * Spad * Dpad;
+    for (int d0 = 0; d0 < D; d0 += 64) {
+      const int d = d0 + lane;
+      float acc = 0.f;
+      if (src_cl) {
+        const float *row = src_cl + ((int64_t)b * MN + en.n) * Spad;
+        for (int sc = 0; sc < S; sc++) acc = __builtin_fmaf(row[sc], wk[(int64_t)sc * Dpad + min(d, Dpad - 1)], acc);
+      } else {
+        const float *col = src + (int64_t)b * S * MN + en.n;
+        for (int sc = 0; sc < S; sc++)
+          acc = __builtin_fmaf(col[(int64_t)sc * MN], wk[(int64_t)sc * Dpad + min(d, Dpad - 1)], acc);
+      }
+      if (d < D) atomic_add(dst + ((int64_t)b * D + d) * DN + en.p, en.wt * acc);
     }
   }
 }
@@ -1271,14 +1318,15 @@ __global__ void convert_planes_kernel(const float *__restrict__ src, TD *__restr
 }
 
 struct ScatterScratch {
-  size_t wq, wpt, cnt, tmap, tiw, acc32, total;  // byte offsets
+  size_t wq, wpt, cnt, tmap, tiw, acc32, ovf, stage, total;  // byte offsets
+  int64_t ovf_cap;  // entries of the overflow list (0: none)
   bool transposed_path;
 };
 
 // elem: bytes per data element; a non-fp32 destination needs an fp32 accumulation
-// image for the atomic path.
+// image for the atomic path.  MH x MW x K x P: the map (P = 0: unweighted).
 ScatterScratch scatter_scratch(int64_t B, int64_t S, int64_t D, int64_t K, int64_t DH, int64_t DW,
-                               size_t elem) {
+                               size_t elem, int64_t MH, int64_t MW, int64_t P) {
   ScatterScratch sc;
   size_t off = 0;
   sc.wq = off;
@@ -1291,13 +1339,23 @@ ScatterScratch scatter_scratch(int64_t B, int64_t S, int64_t D, int64_t K, int64
   if (sc.transposed_path) {
     sc.wpt = off;
     off += align256((size_t)(K * round_up(S, kGC) * round_up(D, kOT)) * 4);
-    sc.cnt = off;  // counters, then the overflow flag; cleared together with tmap and tiw
-    off += align256((size_t)(cells + 1) * 4);
+    sc.cnt = off;  // counters, the overflow flag and list length; cleared with tmap and tiw
+    off += align256((size_t)(cells + 2) * 4);
     sc.tmap = off;
     off += align256((size_t)cells * kTransSlots * 2 * 4);
     sc.tiw = off;
     off += align256((size_t)cells * kTransSlots * 4);
   }
+  // Overflow list (fp32 destinations: it is applied with float atomics): room for half of
+  // the contributions a bilinear map can make.
+  sc.ovf = sc.stage = off;
+  sc.ovf_cap = 0;
+  if (sc.transposed_path && elem == 4) {
+    sc.ovf_cap = std::min<int64_t>(MH * MW * K * (P ? P : 1) * 2, 0x3fffffffLL);
+    off += align256((size_t)sc.ovf_cap * sizeof(OverflowEntry));
+  }
+  sc.stage = off;  // channel-last copy of a single-row source (see launch_gather_product)
+  if (sc.transposed_path && MH == 1) off += align256((size_t)(B * MH * MW * round_up(S, kGC)) * 4);
   sc.total = off;
   return sc;
 }
@@ -1305,8 +1363,8 @@ ScatterScratch scatter_scratch(int64_t B, int64_t S, int64_t D, int64_t K, int64
 }  // namespace
 
 size_t mfma_product_scatter_bytes(int64_t B, int64_t S, int64_t D, int64_t K, int64_t DH,
-                                  int64_t DW, size_t elem) {
-  return scatter_scratch(B, S, D, K, DH, DW, elem).total;
+                                  int64_t DW, size_t elem, int64_t MH, int64_t MW, int64_t P) {
+  return scatter_scratch(B, S, D, K, DH, DW, elem, MH, MW, P).total;
 }
 
 // dst is fully overwritten: dst[b,d] = bias[d] (or 0) + scattered products.
@@ -1316,7 +1374,7 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
                          const TD *bias, TD *dst, void *scratch, int64_t B, int64_t S, int64_t D,
                          int64_t DH, int64_t DW, int64_t MH, int64_t MW, int64_t K, int64_t P,
                          int interp, hipStream_t s) {
-  const ScatterScratch sc = scatter_scratch(B, S, D, K, DH, DW, sizeof(TD));
+  const ScatterScratch sc = scatter_scratch(B, S, D, K, DH, DW, sizeof(TD), MH, MW, P);
   char *base = (char *)scratch;
   float *wq = (float *)(base + sc.wq);
   const int Spad = (int)round_up(S, kScSC), dchunks = (int)((D + kScDC - 1) / kScDC);
@@ -1331,23 +1389,34 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
     const int64_t cells = DH * DW * K;
     int *flag = cnt + cells;
     gate = flag;
-    if (int rc = fill_f32((float *)cnt, (int64_t)((sc.total - sc.cnt) / 4), 0.f, s)) return rc;
+    if (int rc = fill_f32((float *)cnt, (int64_t)((sc.ovf - sc.cnt) / 4), 0.f, s)) return rc;
+    OverflowEntry *ovf = (OverflowEntry *)(base + sc.ovf);
+    TD *stage = MH == 1 ? (TD *)(base + sc.stage) : nullptr;
     const int64_t entries = MH * MW * K;
     const unsigned blocks = (unsigned)((entries + 255) / 256);
     if (m.mode == kInterpNearest)
       hipLaunchKernelGGL(build_transposed_map_kernel<1>, dim3(blocks), dim3(256), 0, s, map, iw,
-                         cnt, tmap, tiw, flag, m.np, m.weighted, m.wrap, (int)DH, (int)DW,
-                         (int)MW, (int)K, entries);
+                         cnt, tmap, tiw, flag, ovf, (int)sc.ovf_cap, m.np, m.weighted, m.wrap,
+                         (int)DH, (int)DW, (int)MW, (int)K, entries);
     else
       hipLaunchKernelGGL(build_transposed_map_kernel<4>, dim3(blocks), dim3(256), 0, s, map, iw,
-                         cnt, tmap, tiw, flag, m.np, m.weighted, m.wrap, (int)DH, (int)DW,
-                         (int)MW, (int)K, entries);
+                         cnt, tmap, tiw, flag, ovf, (int)sc.ovf_cap, m.np, m.weighted, m.wrap,
+                         (int)DH, (int)DW, (int)MW, (int)K, entries);
     MCX_HIP_CHECK_LAUNCH();
     if (int rc = launch_pack_weights<TD>(w, wpt, D, S, K, 1, s)) return rc;
-    if (int rc = launch_gather_product<TD>(src, tmap, tiw, wpt, bias, dst, (TD *)nullptr, B, S, D,
-                                           MH, MW, DH,
-                                           DW, K, kTransSlots, kInterpNearest, gate, 1, s))
+    if (int rc = launch_gather_product<TD>(src, tmap, tiw, wpt, bias, dst, stage, B, S, D, MH, MW,
+                                           DH, DW, K, kTransSlots, kInterpNearest, gate, 1, s))
       return rc;
+    if constexpr (sizeof(TD) == 4) {
+      // what did not fit the four slots of its cell (fp32: the packed weights are Wp[k][s][d])
+      const bool cl = stage != nullptr &&
+                      MH * MW * round_up(S, kGC) * (int64_t)sizeof(TD) <= 0xffffffffLL;
+      hipLaunchKernelGGL(overflow_scatter_kernel, dim3(2048, (unsigned)B), dim3(64), 0, s,
+                         (const float *)src, cl ? (const float *)stage : (const float *)nullptr,
+                         wpt, (float *)dst, ovf, flag, (int)sc.ovf_cap, (int)S,
+                         (int)round_up(S, kGC), (int)D, (int)round_up(D, kOT), MH * MW, DH * DW);
+      MCX_HIP_CHECK_LAUNCH();
+    }
   }
 
   // atomic path (runs when there is no transposed map or it overflowed)
