@@ -55,8 +55,8 @@ size_t gather_product_ws(int dtype, int64_t G, int64_t O, int64_t K, int64_t P, 
   return use_mfma(dtype, P) ? mfma_gather_product_bytes(O, G, K, B, SH, SW) : 0;
 }
 size_t weight_grad_ws(int dtype, int64_t B, int64_t A, int64_t G, int64_t MH, int64_t MW,
-                      int64_t K, int64_t P) {
-  return use_mfma(dtype, P) ? mfma_weight_grad_bytes(B, A, G, MH, MW, K) : 0;
+                      int64_t K, int64_t P, int64_t GH, int64_t GW) {
+  return use_mfma(dtype, P) ? mfma_weight_grad_bytes(B, A, G, MH, MW, K, GH, GW) : 0;
 }
 size_t product_scatter_ws(int dtype, int64_t B, int64_t S, int64_t D, int64_t K, int64_t P,
                           int64_t DH, int64_t DW, int64_t MH, int64_t MW) {
@@ -184,7 +184,8 @@ int weight_grad<float>(bool mfma, const void *plain, const void *gath, const voi
     return generic_weight_grad<float>((const float *)plain, (const float *)gath,
                                       (const float *)map, (const float *)iw, (float *)gw, B, A, G,
                                       GH, GW, MH * MW, K, P, interp, s);
-  if (!ws || ws_bytes < mfma_weight_grad_bytes(B, A, G, MH, MW, K)) return MCX_E_WORKSPACE;
+  if (!ws || ws_bytes < mfma_weight_grad_bytes(B, A, G, MH, MW, K, GH, GW))
+    return MCX_E_WORKSPACE;
   return mfma_weight_grad<float>((const float *)plain, (const float *)gath, (const float *)map,
                                  (const float *)iw, (float *)gw, ws, B, A, G, GH, GW, MH, MW, K, P,
                                  interp, s);
@@ -230,7 +231,8 @@ int weight_grad<bf16_t>(bool mfma, const void *plain, const void *gath, const vo
                         int64_t G, int64_t GH, int64_t GW, int64_t MH, int64_t MW, int64_t K,
                         int64_t P, int interp, hipStream_t s) {
   if (!mfma) return MCX_E_DTYPE;
-  if (!ws || ws_bytes < mfma_weight_grad_bytes(B, A, G, MH, MW, K)) return MCX_E_WORKSPACE;
+  if (!ws || ws_bytes < mfma_weight_grad_bytes(B, A, G, MH, MW, K, GH, GW))
+    return MCX_E_WORKSPACE;
   return mfma_weight_grad<bf16_t>((const bf16_t *)plain, (const bf16_t *)gath, (const float *)map,
                                   (const float *)iw, (bf16_t *)gw, ws, B, A, G, GH, GW, MH, MW, K,
                                   P, interp, s);
@@ -326,7 +328,7 @@ extern "C" size_t mcx_conv_backward_workspace(int64_t B, int64_t Ci, int64_t Co,
                                               int64_t IW, int64_t OH, int64_t OW, int64_t K,
                                               int64_t P, int dtype) {
   // the gradients run one after the other on the stream and share the scratch
-  return std::max({weight_grad_ws(dtype, B, Co, Ci, OH, OW, K, P),
+  return std::max({weight_grad_ws(dtype, B, Co, Ci, OH, OW, K, P, IH, IW),
                    product_scatter_ws(dtype, B, Co, Ci, K, P, IH, IW, OH, OW),
                    bias_grad_ws(dtype, B, Co, OH * OW)});
 }
@@ -373,7 +375,7 @@ extern "C" size_t mcx_tconv_backward_workspace(int64_t B, int64_t Ci, int64_t Co
   // backward-input is a gather-product with the channel roles swapped; the
   // gradients run one after the other and share the scratch
   return std::max({gather_product_ws(dtype, Co, Ci, K, P, B, OH, OW),
-                   weight_grad_ws(dtype, B, Ci, Co, IH, IW, K, P),
+                   weight_grad_ws(dtype, B, Ci, Co, IH, IW, K, P, OH, OW),
                    bias_grad_ws(dtype, B, Co, OH * OW)});
 }
 

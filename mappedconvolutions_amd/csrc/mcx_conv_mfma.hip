@@ -379,7 +379,9 @@ constexpr int kWgCB = 2;            // 16-channel blocks of gathered channels pe
 constexpr int kWgKT = 9;            // taps per pass (accumulators in registers)
 constexpr int kLdPx = kTilePx + 4;  // LDS row stride (floats)
 
-template <typename TD, int NCORN, int NP>
+// CL: `gath` is a channel-last copy [B][GH*GW][Gpad] of the gathered operand (see the
+// gather-product kernel).
+template <typename TD, int NCORN, int NP, bool CL>
 __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad_mfma_kernel(
     const TD *__restrict__ plain, const TD *__restrict__ gath,
     const float *__restrict__ map, const float *__restrict__ iw, float *__restrict__ part, int A,
@@ -503,7 +505,8 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
     const int gi = i0 + (p >> tw_shift), gj = j0 + (p & tw_mask);
     const bool live = gi < MH && gj < MW;
     const int64_t n_g = live ? (int64_t)gi * MW + gj : 0;
-    const TD *gath_b = gath + (int64_t)b * G * gplane;
+    const int Gpad = (G + kGC - 1) / kGC * kGC;
+    const TD *gath_b = gath + (int64_t)b * (CL ? Gpad : G) * gplane;
 
     unsigned off[NE];
     float wt[NE];
@@ -517,7 +520,7 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
                                          live ? (weighted ? iw[e] : 1.f) : 0.f, t);
 #pragma unroll
         for (int i = 0; i < NCORN; i++) {
-          o[sp * NCORN + i] = t.off[i];
+          o[sp * NCORN + i] = CL ? t.off[i] * (unsigned)Gpad : t.off[i];
           w_[sp * NCORN + i] = t.wt[i];
         }
       }
@@ -535,11 +538,35 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
     };
     auto issue = [&](int cb) {
       const int g0 = g_first + cb * kGC + half * 8;
+      if constexpr (CL) {
+        // 8 contiguous channels of the pixel row; a workgroup whose channels lie past the
+        // padded count reads the last valid group (its products are not stored)
+        const char *base = reinterpret_cast<const char *>(gath_b + min(g0, Gpad - 8));
 #pragma unroll
-      for (int ch = 0; ch < 8; ch++) {
-        const TD *pl = gath_b + (int64_t)min(g0 + ch, G - 1) * gplane;
+        for (int i = 0; i < NE; i++) {
+          const char *row = base + off[i];
+          if constexpr (kBf16) {
+            const uint4 q = *reinterpret_cast<const uint4 *>(row);
+            const unsigned w4[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
-        for (int i = 0; i < NE; i++) v[ch][i] = load_at(pl, off[i]);
+            for (int j = 0; j < 4; j++) {
+              v[2 * j][i] = __builtin_bit_cast(float, w4[j] << 16);
+              v[2 * j + 1][i] = __builtin_bit_cast(float, w4[j] & 0xffff0000u);
+            }
+          } else {
+            const float4 q0 = reinterpret_cast<const float4 *>(row)[0];
+            const float4 q1 = reinterpret_cast<const float4 *>(row)[1];
+            v[0][i] = q0.x; v[1][i] = q0.y; v[2][i] = q0.z; v[3][i] = q0.w;
+            v[4][i] = q1.x; v[5][i] = q1.y; v[6][i] = q1.z; v[7][i] = q1.w;
+          }
+        }
+      } else {
+#pragma unroll
+        for (int ch = 0; ch < 8; ch++) {
+          const TD *pl = gath_b + (int64_t)min(g0 + ch, G - 1) * gplane;
+#pragma unroll
+          for (int i = 0; i < NE; i++) v[ch][i] = load_at(pl, off[i]);
+        }
       }
     };
     auto stage = [&](int buf) {
@@ -1167,11 +1194,14 @@ int mfma_gather_product(const TD *src, const float *map, const float *iw, const 
 }
 
 // ---- weight gradient ---------------------------------------------------------------
-size_t mfma_weight_grad_bytes(int64_t B, int64_t A, int64_t G, int64_t MH, int64_t MW,
-                              int64_t K) {
+// Per-range partial sums, then (single-row gathered operands) their channel-last copy.
+size_t mfma_weight_grad_bytes(int64_t B, int64_t A, int64_t G, int64_t MH, int64_t MW, int64_t K,
+                              int64_t GH, int64_t GW) {
   const PixelTiling t = make_tiling(B, MH, MW);
-  return align256((size_t)weight_grad_ranges(t.total, A, G, K) * (size_t)(A * G * K) *
-                  sizeof(float));
+  size_t n = align256((size_t)weight_grad_ranges(t.total, A, G, K) * (size_t)(A * G * K) *
+                      sizeof(float));
+  if (GH == 1) n += align256((size_t)(B * GH * GW * round_up(G, kGC)) * sizeof(float));
+  return n;
 }
 
 // scratch: mfma_weight_grad_bytes(...) bytes (per-range partial sums).
@@ -1184,16 +1214,39 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
   if (t.total > 0x7fffffffLL) return MCX_E_SHAPE;
   const int ranges = weight_grad_ranges(t.total, A, G, K);
   const int cgroups = (int)((G + kWgCB * kGC - 1) / (kWgCB * kGC));
+  const int64_t Gpad = round_up(G, kGC);
+  const bool cl = use_channel_last(GH, interp) &&
+                  GH * GW * Gpad * (int64_t)sizeof(TD) <= 0xffffffffLL;
+  if (cl) {
+    TD *stage = reinterpret_cast<TD *>((char *)scratch +
+                                       align256((size_t)ranges * (size_t)(A * G * K) * 4));
+    dim3 tg((unsigned)((GH * GW + 63) / 64), (unsigned)((Gpad + 63) / 64), (unsigned)B);
+    hipLaunchKernelGGL(to_channel_last_kernel<TD>, tg, dim3(256), 0, s, gath, stage, (int)G,
+                       (int)Gpad, GH * GW);
+    MCX_HIP_CHECK_LAUNCH();
+    gath = stage;
+  }
   dim3 grid((unsigned)(ranges * cgroups), (unsigned)((A + kWgA - 1) / kWgA),
             (unsigned)((K + kWgKT - 1) / kWgKT));
   const ModeArgs m = mode_args(interp, P);
-#define MCX_LAUNCH(NCORN, NP)                                                                    \
-  hipLaunchKernelGGL((weight_grad_mfma_kernel<TD, NCORN, NP>), grid, dim3(kThreads), 0, s, plain, \
-                     gath, map, iw, part, (int)A, (int)G, (int)GH, (int)GW, (int)MH, (int)MW,    \
-                     (int)K, m.weighted, m.wrap, t.tiles_x, t.tiles_per_img, t.tw_shift,         \
-                     (int)t.total, ranges, cgroups)
+#define MCX_LAUNCH_CL(NCORN, NP, CL)                                                             \
+  hipLaunchKernelGGL((weight_grad_mfma_kernel<TD, NCORN, NP, CL>), grid, dim3(kThreads), 0, s,   \
+                     plain, gath, map, iw, part, (int)A, (int)G, (int)GH, (int)GW, (int)MH,      \
+                     (int)MW, (int)K, m.weighted, m.wrap, t.tiles_x, t.tiles_per_img,            \
+                     t.tw_shift, (int)t.total, ranges, cgroups)
+#define MCX_LAUNCH(NCORN, NP)              \
+  if constexpr (NCORN == 1) {              \
+    if (cl) {                              \
+      MCX_LAUNCH_CL(NCORN, NP, true);      \
+    } else {                               \
+      MCX_LAUNCH_CL(NCORN, NP, false);     \
+    }                                      \
+  } else {                                 \
+    MCX_LAUNCH_CL(NCORN, NP, false);       \
+  }
   MCX_DISPATCH_TAPS(m, MCX_LAUNCH)
 #undef MCX_LAUNCH
+#undef MCX_LAUNCH_CL
   MCX_HIP_CHECK_LAUNCH();
   const int64_t n = A * G * K;
   hipLaunchKernelGGL(reduce_partials_kernel<TD>, dim3((unsigned)((n + 63) / 64)), dim3(64), 0, s,
