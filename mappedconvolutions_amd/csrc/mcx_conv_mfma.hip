@@ -126,7 +126,8 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
     const TD *__restrict__ src, const float *__restrict__ map, const float *__restrict__ iw,
     const float *__restrict__ wp, const TD *__restrict__ bias, TD *__restrict__ y, int G,
     int O, int Opad, int Gpad, int SH, int SW, int OH, int OW, int K, int weighted, int wrap,
-    int tiles_x, int tiles_per_img, int tw_shift, const int *__restrict__ gate, int run_if_zero) {
+    int tiles_x, int tiles_per_img, int tw_shift, const int *__restrict__ gate, int run_if_zero,
+    const float *__restrict__ addend) {
   constexpr int NE = NP * NCORN;         // (offset, weight) pairs per pixel and tap
   constexpr int TG = kTapCache / NE > 0 ? kTapCache / NE : 1;  // taps cached in LDS at a time
   constexpr bool kBf16 = sizeof(TD) == 2;
@@ -351,12 +352,19 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
   const int ei = tile_y * th + (pe >> tw_shift), ej = (tile_x << tw_shift) + (pe & tw_mask);
   if (ei < OH && ej < OW) {
     TD *yb = y + (int64_t)b * O * N + (int64_t)ei * OW + ej;
+    // `addend`: an fp32 image [B][O][N] of contributions accumulated elsewhere (the overflow
+    // list of a transposed map, gate[1] entries long), added when there are any
+    const float *ab = (addend && gate && gate[1] > 0)
+                          ? addend + (int64_t)b * O * N + (int64_t)ei * OW + ej
+                          : nullptr;
 #pragma unroll
     for (int m = 0; m < 2 * OG; m++)
 #pragma unroll
       for (int i = 0; i < 16; i++) {
         const int o = o0 + 32 * m + (i >> 2) * 8 + lhi * 4 + (i & 3);
-        if (o < O) yb[(int64_t)o * N] = from_f32<TD>(acc[m][i] + (bias ? to_f32(bias[o]) : 0.f));
+        if (o < O)
+          yb[(int64_t)o * N] = from_f32<TD>(acc[m][i] + (bias ? to_f32(bias[o]) : 0.f) +
+                                            (ab ? ab[(int64_t)o * N] : 0.f));
       }
   }
 }
@@ -1098,7 +1106,8 @@ template <typename TD>
 int launch_gather_product(const TD *src, const float *map, const float *iw, const float *wp,
                           const TD *bias, TD *y, TD *stage, int64_t B, int64_t G, int64_t O,
                           int64_t SH, int64_t SW, int64_t OH, int64_t OW, int64_t K, int64_t P,
-                          int interp, const int *gate, int run_if_zero, hipStream_t s) {
+                          int interp, const int *gate, int run_if_zero, hipStream_t s,
+                          const float *addend = nullptr) {
   const int Opad = (int)round_up(O, kOT), Gpad = (int)round_up(G, kGC);
   const bool cl = stage != nullptr && use_channel_last(SH, interp) &&
                   SH * SW * Gpad * (int64_t)sizeof(TD) <= 0xffffffffLL;
@@ -1119,7 +1128,7 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
   hipLaunchKernelGGL((gather_product_mfma_kernel<TD, NCORN, NP, OG, CL>), grid, dim3(kThreads),  \
                      0, s, src, map, iw, wp, bias, y, (int)G, (int)O, Opad, Gpad, (int)SH,       \
                      (int)SW, (int)OH, (int)OW, (int)K, m.weighted, m.wrap, t.tiles_x,           \
-                     t.tiles_per_img, t.tw_shift, gate, run_if_zero)
+                     t.tiles_per_img, t.tw_shift, gate, run_if_zero, addend)
 #define MCX_LAUNCH_OG(NCORN, NP, OG)           \
   if constexpr (NCORN == 1) {                  \
     if (cl) {                                  \
@@ -1317,36 +1326,65 @@ __global__ void build_transposed_map_kernel(const float *__restrict__ map,
   }
 }
 
-// dst[b, d, p] += wt * sum_s W[s, d, k] * src[b, s, n] for every overflow entry: one wave
-// per (entry, image), a lane per destination channel.  `wp` holds the weights packed as
-// Wp[k][s][d] (the gather-product layout); `src_cl`, when not null, is the channel-last copy
-// [B][MN][Spad] of the source, else src is [B][S][MN].  A fixed grid walks the list, so an
-// empty list costs one launch of idle workgroups.
+// accum[b, d, p] += wt * sum_s W[s, d, k] * src[b, s, n] for every overflow entry: one wave
+// per (entry, image), a lane per destination channel.  `wp` holds the weights in the
+// gather-product's packed layout (fp32: Wp[k][s][d]; bf16: Wb[k][chunk][kg][d][8]); `src_cl`,
+// when not null, is the channel-last copy [B][MN][Spad] of the source, else src is
+// [B][S][MN].  `accum` is the fp32 destination itself or an fp32 image added by the gather's
+// epilogue.  A fixed grid walks the list, so an empty list costs one launch of idle workgroups.
+template <typename TD>
 __global__ __launch_bounds__(64) void overflow_scatter_kernel(
-    const float *__restrict__ src, const float *__restrict__ src_cl,
-    const float *__restrict__ wp, float *__restrict__ dst,
-    const OverflowEntry *__restrict__ ovf, const int *__restrict__ overflow, int ovf_cap, int S,
-    int Spad, int D, int Dpad, int64_t MN, int64_t DN) {
+    const TD *__restrict__ src, const TD *__restrict__ src_cl, const void *__restrict__ wp,
+    float *__restrict__ accum, const OverflowEntry *__restrict__ ovf,
+    const int *__restrict__ overflow, int ovf_cap, int S, int Spad, int D, int Dpad, int64_t MN,
+    int64_t DN) {
   if (overflow[0] != 0) return;  // the scatter kernel does the whole product
   const int count = min(overflow[1], ovf_cap);
   const int b = blockIdx.y, lane = threadIdx.x;
+  const int chunks = Spad / kGC;
   for (int e = blockIdx.x; e < count; e += gridDim.x) {
     const OverflowEntry en = ovf[e];
-    const float *wk = wp + (int64_t)en.k * Spad * Dpad;
     for (int d0 = 0; d0 < D; d0 += 64) {
-      const int d = d0 + lane;
+      const int d = min(d0 + lane, Dpad - 1);
       float acc = 0.f;
-      if (src_cl) {
-        const float *row = src_cl + ((int64_t)b * MN + en.n) * Spad;
-        for (int sc = 0; sc < S; sc++) acc = __builtin_fmaf(row[sc], wk[(int64_t)sc * Dpad + min(d, Dpad - 1)], acc);
-      } else {
-        const float *col = src + (int64_t)b * S * MN + en.n;
-        for (int sc = 0; sc < S; sc++)
-          acc = __builtin_fmaf(col[(int64_t)sc * MN], wk[(int64_t)sc * Dpad + min(d, Dpad - 1)], acc);
+      for (int s8 = 0; s8 < Spad / 8; s8++) {  // 8 source channels at a time (both are padded)
+        float x[8], wv[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+          const int sc = s8 * 8 + j;
+          x[j] = src_cl ? to_f32(src_cl[((int64_t)b * MN + en.n) * Spad + sc])
+                        : (sc < S ? to_f32(src[((int64_t)b * S + sc) * MN + en.n]) : 0.f);
+        }
+        if constexpr (sizeof(TD) == 2) {
+          const int64_t wi = ((((int64_t)en.k * chunks + (s8 >> 1)) * 2 + (s8 & 1)) * Dpad + d) << 3;
+          const uint4 q = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(wp) + wi);
+          const unsigned w4[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            wv[2 * j] = __builtin_bit_cast(float, w4[j] << 16);
+            wv[2 * j + 1] = __builtin_bit_cast(float, w4[j] & 0xffff0000u);
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; j++)
+            wv[j] = reinterpret_cast<const float *>(wp)[((int64_t)en.k * Spad + s8 * 8 + j) * Dpad + d];
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) acc = __builtin_fmaf(x[j], wv[j], acc);
       }
-      if (d < D) atomic_add(dst + ((int64_t)b * D + d) * DN + en.p, en.wt * acc);
+      if (d0 + lane < D) atomic_add(accum + ((int64_t)b * D + d) * DN + en.p, en.wt * acc);
     }
   }
+}
+
+// Clears the fp32 image the overflow list of a non-fp32 product is accumulated into; only
+// when the list is in use and not empty.
+__global__ void clear_overflow_image_kernel(float *__restrict__ img, int64_t total,
+                                            const int *__restrict__ overflow) {
+  if (overflow[0] != 0 || overflow[1] <= 0) return;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x)
+    img[i] = 0.f;
 }
 
 // dst[b,c,:] = bias[c] (or 0); runs only when the gate agrees (see above).
@@ -1399,11 +1437,10 @@ ScatterScratch scatter_scratch(int64_t B, int64_t S, int64_t D, int64_t K, int64
     sc.tiw = off;
     off += align256((size_t)cells * kTransSlots * 4);
   }
-  // Overflow list (fp32 destinations: it is applied with float atomics): room for half of
-  // the contributions a bilinear map can make.
+  // Overflow list: room for half of the contributions a bilinear map can make.
   sc.ovf = sc.stage = off;
   sc.ovf_cap = 0;
-  if (sc.transposed_path && elem == 4) {
+  if (sc.transposed_path) {
     sc.ovf_cap = std::min<int64_t>(MH * MW * K * (P ? P : 1) * 2, 0x3fffffffLL);
     off += align256((size_t)sc.ovf_cap * sizeof(OverflowEntry));
   }
@@ -1457,18 +1494,44 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
                          (int)DH, (int)DW, (int)MW, (int)K, entries);
     MCX_HIP_CHECK_LAUNCH();
     if (int rc = launch_pack_weights<TD>(w, wpt, D, S, K, 1, s)) return rc;
-    if (int rc = launch_gather_product<TD>(src, tmap, tiw, wpt, bias, dst, stage, B, S, D, MH, MW,
-                                           DH, DW, K, kTransSlots, kInterpNearest, gate, 1, s))
-      return rc;
-    if constexpr (sizeof(TD) == 4) {
-      // what did not fit the four slots of its cell (fp32: the packed weights are Wp[k][s][d])
-      const bool cl = stage != nullptr &&
-                      MH * MW * round_up(S, kGC) * (int64_t)sizeof(TD) <= 0xffffffffLL;
-      hipLaunchKernelGGL(overflow_scatter_kernel, dim3(2048, (unsigned)B), dim3(64), 0, s,
-                         (const float *)src, cl ? (const float *)stage : (const float *)nullptr,
-                         wpt, (float *)dst, ovf, flag, (int)sc.ovf_cap, (int)S,
-                         (int)round_up(S, kGC), (int)D, (int)round_up(D, kOT), MH * MW, DH * DW);
+    // What did not fit the four slots of its cell is applied with float atomics: onto the
+    // fp32 destination after the gather has written it, or (other storage types) into the
+    // fp32 image first, which the gather's epilogue then adds.
+    const int64_t Spad16 = round_up(S, kGC);
+    const bool cl = stage != nullptr && use_channel_last(MH, kInterpNearest) &&
+                    MH * MW * Spad16 * (int64_t)sizeof(TD) <= 0xffffffffLL;
+    float *img = sizeof(TD) == 4 ? (float *)dst : (float *)(base + sc.acc32);
+    auto overflow_pass = [&]() -> int {
+      hipLaunchKernelGGL(overflow_scatter_kernel<TD>, dim3(2048, (unsigned)B), dim3(64), 0, s, src,
+                         cl ? (const TD *)stage : (const TD *)nullptr, (const void *)wpt, img, ovf,
+                         flag, (int)sc.ovf_cap, (int)S, (int)Spad16, (int)D,
+                         (int)round_up(D, kOT), MH * MW, DH * DW);
       MCX_HIP_CHECK_LAUNCH();
+      return 0;
+    };
+    if (sizeof(TD) == 4) {
+      if (int rc = launch_gather_product<TD>(src, tmap, tiw, wpt, bias, dst, stage, B, S, D, MH,
+                                             MW, DH, DW, K, kTransSlots, kInterpNearest, gate, 1,
+                                             s))
+        return rc;
+      if (int rc = overflow_pass()) return rc;
+    } else {
+      const int64_t total_img = B * D * DH * DW;
+      hipLaunchKernelGGL(clear_overflow_image_kernel,
+                         dim3((unsigned)std::min<int64_t>((total_img + 1023) / 1024, 65536)),
+                         dim3(256), 0, s, img, total_img, flag);
+      MCX_HIP_CHECK_LAUNCH();
+      if (cl) {  // the overflow pass reads the channel-last copy before the gather makes it
+        dim3 tg((unsigned)((MH * MW + 63) / 64), (unsigned)((Spad16 + 63) / 64), (unsigned)B);
+        hipLaunchKernelGGL(to_channel_last_kernel<TD>, tg, dim3(256), 0, s, src, stage, (int)S,
+                           (int)Spad16, MH * MW);
+        MCX_HIP_CHECK_LAUNCH();
+      }
+      if (int rc = overflow_pass()) return rc;
+      if (int rc = launch_gather_product<TD>(src, tmap, tiw, wpt, bias, dst, stage, B, S, D, MH,
+                                             MW, DH, DW, K, kTransSlots, kInterpNearest, gate, 1,
+                                             s, img))
+        return rc;
     }
   }
 
