@@ -352,10 +352,10 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
   const int ei = tile_y * th + (pe >> tw_shift), ej = (tile_x << tw_shift) + (pe & tw_mask);
   if (ei < OH && ej < OW) {
     TD *yb = y + (int64_t)b * O * N + (int64_t)ei * OW + ej;
-    // `addend`: an fp32 image [B][O][N] of contributions accumulated elsewhere (the overflow
-    // list of a transposed map, gate[1] entries long), added when there are any
+    // `addend`: a channel-last fp32 image [B][N][Opad] of contributions accumulated elsewhere
+    // (the overflow list of a transposed map, gate[1] entries long), added when there are any
     const float *ab = (addend && gate && gate[1] > 0)
-                          ? addend + (int64_t)b * O * N + (int64_t)ei * OW + ej
+                          ? addend + ((int64_t)b * N + (int64_t)ei * OW + ej) * Opad
                           : nullptr;
 #pragma unroll
     for (int m = 0; m < 2 * OG; m++)
@@ -364,7 +364,7 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
         const int o = o0 + 32 * m + (i >> 2) * 8 + lhi * 4 + (i & 3);
         if (o < O)
           yb[(int64_t)o * N] = from_f32<TD>(acc[m][i] + (bias ? to_f32(bias[o]) : 0.f) +
-                                            (ab ? ab[(int64_t)o * N] : 0.f));
+                                            (ab ? ab[o] : 0.f));
       }
   }
 }
@@ -1107,11 +1107,13 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
                           const TD *bias, TD *y, TD *stage, int64_t B, int64_t G, int64_t O,
                           int64_t SH, int64_t SW, int64_t OH, int64_t OW, int64_t K, int64_t P,
                           int interp, const int *gate, int run_if_zero, hipStream_t s,
-                          const float *addend = nullptr) {
+                          const float *addend = nullptr, bool staged = false) {
   const int Opad = (int)round_up(O, kOT), Gpad = (int)round_up(G, kGC);
   const bool cl = stage != nullptr && use_channel_last(SH, interp) &&
                   SH * SW * Gpad * (int64_t)sizeof(TD) <= 0xffffffffLL;
-  if (cl) {
+  if (cl && staged) {
+    src = stage;  // the caller has made the channel-last copy already
+  } else if (cl) {
     dim3 tg((unsigned)((SH * SW + 63) / 64), (unsigned)((Gpad + 63) / 64), (unsigned)B);
     hipLaunchKernelGGL(to_channel_last_kernel<TD>, tg, dim3(256), 0, s, src, stage, (int)G, Gpad,
                        SH * SW);
@@ -1330,8 +1332,9 @@ __global__ void build_transposed_map_kernel(const float *__restrict__ map,
 // per (entry, image), a lane per destination channel.  `wp` holds the weights in the
 // gather-product's packed layout (fp32: Wp[k][s][d]; bf16: Wb[k][chunk][kg][d][8]); `src_cl`,
 // when not null, is the channel-last copy [B][MN][Spad] of the source, else src is
-// [B][S][MN].  `accum` is the fp32 destination itself or an fp32 image added by the gather's
-// epilogue.  A fixed grid walks the list, so an empty list costs one launch of idle workgroups.
+// [B][S][MN].  `accum` is a channel-last fp32 image [B][DN][Dpad] (a wave's 64 atomics fall
+// into two cache lines instead of 64) that the gather's epilogue adds.  A fixed grid walks
+// the list, so an empty list costs one launch of idle workgroups.
 template <typename TD>
 __global__ __launch_bounds__(64) void overflow_scatter_kernel(
     const TD *__restrict__ src, const TD *__restrict__ src_cl, const void *__restrict__ wp,
@@ -1372,7 +1375,7 @@ __global__ __launch_bounds__(64) void overflow_scatter_kernel(
 #pragma unroll
         for (int j = 0; j < 8; j++) acc = __builtin_fmaf(x[j], wv[j], acc);
       }
-      if (d0 + lane < D) atomic_add(accum + ((int64_t)b * D + d) * DN + en.p, en.wt * acc);
+      if (d0 + lane < D) atomic_add(accum + ((int64_t)b * DN + en.p) * Dpad + d, en.wt * acc);
     }
   }
 }
@@ -1422,10 +1425,16 @@ ScatterScratch scatter_scratch(int64_t B, int64_t S, int64_t D, int64_t K, int64
   size_t off = 0;
   sc.wq = off;
   off += align256((size_t)(K * ((D + kScDC - 1) / kScDC) * round_up(S, kScSC) * kScDC) * 4);
-  sc.acc32 = off;
-  if (elem != 4) off += align256((size_t)(B * D * DH * DW) * 4);
   const int64_t cells = DH * DW * K;
   sc.transposed_path = cells * kTransSlots * 2 <= 0x7fffffffLL;
+  // One fp32 image: the scatter kernel's accumulation image of a non-fp32 destination
+  // ([B][D][DN]) or the channel-last overflow image ([B][DN][D padded to 64]); never both.
+  sc.acc32 = off;
+  {
+    const int64_t scatter_img = elem != 4 ? B * D * DH * DW : 0;
+    const int64_t overflow_img = sc.transposed_path ? B * DH * DW * round_up(D, kOT) : 0;
+    off += align256((size_t)std::max(scatter_img, overflow_img) * 4);
+  }
   sc.wpt = sc.cnt = sc.tmap = sc.tiw = off;
   if (sc.transposed_path) {
     sc.wpt = off;
@@ -1494,45 +1503,33 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
                          (int)DH, (int)DW, (int)MW, (int)K, entries);
     MCX_HIP_CHECK_LAUNCH();
     if (int rc = launch_pack_weights<TD>(w, wpt, D, S, K, 1, s)) return rc;
-    // What did not fit the four slots of its cell is applied with float atomics: onto the
-    // fp32 destination after the gather has written it, or (other storage types) into the
-    // fp32 image first, which the gather's epilogue then adds.
+    // What did not fit the four slots of its cell is accumulated with float atomics into a
+    // channel-last fp32 image (cleared only when there is anything to add), which the
+    // gather's epilogue adds.
     const int64_t Spad16 = round_up(S, kGC);
     const bool cl = stage != nullptr && use_channel_last(MH, kInterpNearest) &&
                     MH * MW * Spad16 * (int64_t)sizeof(TD) <= 0xffffffffLL;
-    float *img = sizeof(TD) == 4 ? (float *)dst : (float *)(base + sc.acc32);
-    auto overflow_pass = [&]() -> int {
-      hipLaunchKernelGGL(overflow_scatter_kernel<TD>, dim3(2048, (unsigned)B), dim3(64), 0, s, src,
-                         cl ? (const TD *)stage : (const TD *)nullptr, (const void *)wpt, img, ovf,
-                         flag, (int)sc.ovf_cap, (int)S, (int)Spad16, (int)D,
-                         (int)round_up(D, kOT), MH * MW, DH * DW);
+    float *img = (float *)(base + sc.acc32);
+    const int64_t total_img = B * DH * DW * round_up(D, kOT);
+    hipLaunchKernelGGL(clear_overflow_image_kernel,
+                       dim3((unsigned)std::min<int64_t>((total_img + 1023) / 1024, 4096)),
+                       dim3(256), 0, s, img, total_img, flag);
+    MCX_HIP_CHECK_LAUNCH();
+    if (cl) {  // the overflow pass reads the channel-last copy before the gather would make it
+      dim3 tg((unsigned)((MH * MW + 63) / 64), (unsigned)((Spad16 + 63) / 64), (unsigned)B);
+      hipLaunchKernelGGL(to_channel_last_kernel<TD>, tg, dim3(256), 0, s, src, stage, (int)S,
+                         (int)Spad16, MH * MW);
       MCX_HIP_CHECK_LAUNCH();
-      return 0;
-    };
-    if (sizeof(TD) == 4) {
-      if (int rc = launch_gather_product<TD>(src, tmap, tiw, wpt, bias, dst, stage, B, S, D, MH,
-                                             MW, DH, DW, K, kTransSlots, kInterpNearest, gate, 1,
-                                             s))
-        return rc;
-      if (int rc = overflow_pass()) return rc;
-    } else {
-      const int64_t total_img = B * D * DH * DW;
-      hipLaunchKernelGGL(clear_overflow_image_kernel,
-                         dim3((unsigned)std::min<int64_t>((total_img + 1023) / 1024, 65536)),
-                         dim3(256), 0, s, img, total_img, flag);
-      MCX_HIP_CHECK_LAUNCH();
-      if (cl) {  // the overflow pass reads the channel-last copy before the gather makes it
-        dim3 tg((unsigned)((MH * MW + 63) / 64), (unsigned)((Spad16 + 63) / 64), (unsigned)B);
-        hipLaunchKernelGGL(to_channel_last_kernel<TD>, tg, dim3(256), 0, s, src, stage, (int)S,
-                           (int)Spad16, MH * MW);
-        MCX_HIP_CHECK_LAUNCH();
-      }
-      if (int rc = overflow_pass()) return rc;
-      if (int rc = launch_gather_product<TD>(src, tmap, tiw, wpt, bias, dst, stage, B, S, D, MH,
-                                             MW, DH, DW, K, kTransSlots, kInterpNearest, gate, 1,
-                                             s, img))
-        return rc;
     }
+    hipLaunchKernelGGL(overflow_scatter_kernel<TD>, dim3(2048, (unsigned)B), dim3(64), 0, s, src,
+                       cl ? (const TD *)stage : (const TD *)nullptr, (const void *)wpt, img, ovf,
+                       flag, (int)sc.ovf_cap, (int)S, (int)Spad16, (int)D, (int)round_up(D, kOT),
+                       MH * MW, DH * DW);
+    MCX_HIP_CHECK_LAUNCH();
+    if (int rc = launch_gather_product<TD>(src, tmap, tiw, wpt, bias, dst, stage, B, S, D, MH, MW,
+                                           DH, DW, K, kTransSlots, kInterpNearest, gate, 1, s, img,
+                                           cl))
+      return rc;
   }
 
   // atomic path (runs when there is no transposed map or it overflowed)
