@@ -1122,6 +1122,8 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
   }
   const PixelTiling t = make_tiling(B, OH, OW);
   if (t.total > 0x7fffffffLL) return MCX_E_SHAPE;
+  // tap offsets are 32-bit byte offsets inside a source plane
+  if (SH * SW * (int64_t)sizeof(TD) > 0xffffffffLL) return MCX_E_SHAPE;
   // bf16 storage with at least 128 output channels: 128 outputs per workgroup
   const bool wide = sizeof(TD) == 2 && Opad % (2 * kOT) == 0;
   dim3 grid((unsigned)t.total, (unsigned)(Opad / (wide ? 2 * kOT : kOT)));
@@ -1223,6 +1225,7 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
   float *part = (float *)scratch;
   const PixelTiling t = make_tiling(B, MH, MW);
   if (t.total > 0x7fffffffLL) return MCX_E_SHAPE;
+  if (GH * GW * (int64_t)sizeof(TD) > 0xffffffffLL) return MCX_E_SHAPE;  // 32-bit tap offsets
   const int ranges = weight_grad_ranges(t.total, A, G, K);
   const int cgroups = (int)((G + kWgCB * kGC - 1) / (kWgCB * kGC));
   const int64_t Gpad = round_up(G, kGC);
