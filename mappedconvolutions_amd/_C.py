@@ -146,10 +146,11 @@ def _conv_backward(grad_output, sample_map, interp_weights, input, weight, bias,
     lib = _lib.load()
     ws_bytes = lib.mcx_conv_backward_workspace(B, Ci, Co, IH, IW, OH, OW, K, P, dt)
     ws = _workspace(ws_bytes, input.device)
-    # One C-ABI call per gradient (NULL skips the others) so each can be timed alone.
+    # Two C-ABI calls (NULL skips a gradient) so that the input gradient and the weight
+    # gradient can be timed alone; the bias gradient rides on the weight gradient's pass
+    # over grad_output.
     outs = {"conv_backward_input": (grad_input, None, None),
-            "conv_backward_weight": (None, grad_weight, None),
-            "conv_backward_bias": (None, None, grad_bias)}
+            "conv_backward_weight": (None, grad_weight, grad_bias)}
     with torch.cuda.device(input.device):
         for label, (gx, gw, gb) in outs.items():
             rc = _timed(label, input.device, lambda: lib.mcx_conv_backward(

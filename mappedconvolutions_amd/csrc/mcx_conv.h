@@ -46,7 +46,8 @@ size_t mfma_weight_grad_bytes(int64_t B, int64_t A, int64_t G, int64_t MH, int64
 template <typename TD>
 int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const float *iw, TD *gw,
                      void *scratch, int64_t B, int64_t A, int64_t G, int64_t GH, int64_t GW,
-                     int64_t MH, int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s);
+                     int64_t MH, int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s,
+                     TD *plain_sum);
 size_t mfma_product_scatter_bytes(int64_t B, int64_t S, int64_t D, int64_t K, int64_t DH,
                                   int64_t DW, size_t elem, int64_t MH, int64_t MW, int64_t P);
 template <typename TD>

@@ -89,7 +89,7 @@ template <typename T>
 int weight_grad(bool mfma, const void *plain, const void *gath, const void *map, const void *iw,
                 void *gw, void *ws, size_t ws_bytes, int64_t B, int64_t A, int64_t G, int64_t GH,
                 int64_t GW, int64_t MH, int64_t MW, int64_t K, int64_t P, int interp,
-                hipStream_t s);
+                hipStream_t s, void *plain_sum);  // plain_sum: matrix-core path only, may be NULL
 
 // gb[c] = sum over (b, n) of gy[b,c,n].
 template <typename T>
@@ -122,7 +122,7 @@ int bias_grad(const void *gy, void *gb, void *ws, size_t ws_bytes, int64_t B, in
   int weight_grad<T>(bool, const void *plain, const void *gath, const void *map, const void *iw,   \
                      void *gw, void *, size_t, int64_t B, int64_t A, int64_t G, int64_t GH,        \
                      int64_t GW, int64_t MH, int64_t MW, int64_t K, int64_t P, int interp,         \
-                     hipStream_t s) {                                                              \
+                     hipStream_t s, void *) {                                                      \
     return generic_weight_grad<T>((const T *)plain, (const T *)gath, (const T *)map,               \
                                   (const T *)iw, (T *)gw, B, A, G, GH, GW, MH * MW, K, P, interp,  \
                                   s);                                                              \
@@ -179,7 +179,7 @@ template <>
 int weight_grad<float>(bool mfma, const void *plain, const void *gath, const void *map,
                        const void *iw, void *gw, void *ws, size_t ws_bytes, int64_t B, int64_t A,
                        int64_t G, int64_t GH, int64_t GW, int64_t MH, int64_t MW, int64_t K,
-                       int64_t P, int interp, hipStream_t s) {
+                       int64_t P, int interp, hipStream_t s, void *plain_sum) {
   if (!mfma)
     return generic_weight_grad<float>((const float *)plain, (const float *)gath,
                                       (const float *)map, (const float *)iw, (float *)gw, B, A, G,
@@ -188,7 +188,7 @@ int weight_grad<float>(bool mfma, const void *plain, const void *gath, const voi
     return MCX_E_WORKSPACE;
   return mfma_weight_grad<float>((const float *)plain, (const float *)gath, (const float *)map,
                                  (const float *)iw, (float *)gw, ws, B, A, G, GH, GW, MH, MW, K, P,
-                                 interp, s);
+                                 interp, s, (float *)plain_sum);
 }
 
 template <>
@@ -229,13 +229,13 @@ template <>
 int weight_grad<bf16_t>(bool mfma, const void *plain, const void *gath, const void *map,
                         const void *iw, void *gw, void *ws, size_t ws_bytes, int64_t B, int64_t A,
                         int64_t G, int64_t GH, int64_t GW, int64_t MH, int64_t MW, int64_t K,
-                        int64_t P, int interp, hipStream_t s) {
+                        int64_t P, int interp, hipStream_t s, void *plain_sum) {
   if (!mfma) return MCX_E_DTYPE;
   if (!ws || ws_bytes < mfma_weight_grad_bytes(B, A, G, MH, MW, K, GH, GW))
     return MCX_E_WORKSPACE;
   return mfma_weight_grad<bf16_t>((const bf16_t *)plain, (const bf16_t *)gath, (const float *)map,
                                   (const float *)iw, (bf16_t *)gw, ws, B, A, G, GH, GW, MH, MW, K,
-                                  P, interp, s);
+                                  P, interp, s, (bf16_t *)plain_sum);
 }
 
 template <>
@@ -262,10 +262,13 @@ int conv_backward_t(bool mfma, const void *gy, const void *map, const void *iw, 
   if (gx && (rc = product_scatter<T>(mfma, gy, map, iw, w, nullptr, gx, ws, ws_bytes, d.B, d.Co,
                                      d.Ci, d.IH, d.IW, d.OH, d.OW, d.K, d.P, interp, s)))
     return rc;
+  // the matrix-core weight gradient stages every tile of gy: it sums them for the bias
+  // gradient on the way
+  const bool fused_bias = gw && gb && mfma;
   if (gw && (rc = weight_grad<T>(mfma, gy, x, map, iw, gw, ws, ws_bytes, d.B, d.Co, d.Ci, d.IH,
-                                 d.IW, d.OH, d.OW, d.K, d.P, interp, s)))
+                                 d.IW, d.OH, d.OW, d.K, d.P, interp, s, fused_bias ? gb : nullptr)))
     return rc;
-  if (gb) rc = bias_grad<T>(gy, gb, ws, ws_bytes, d.B, d.Co, d.OH * d.OW, s);
+  if (gb && !fused_bias) rc = bias_grad<T>(gy, gb, ws, ws_bytes, d.B, d.Co, d.OH * d.OW, s);
   return rc;
 }
 
@@ -287,7 +290,7 @@ int tconv_backward_t(bool mfma, const void *gy, const void *map, const void *iw,
                                     d.Ci, d.OH, d.OW, d.IH, d.IW, d.K, d.P, interp, s)))
     return rc;
   if (gw && (rc = weight_grad<T>(mfma, x, gy, map, iw, gw, ws, ws_bytes, d.B, d.Ci, d.Co, d.OH,
-                                 d.OW, d.IH, d.IW, d.K, d.P, interp, s)))
+                                 d.OW, d.IH, d.IW, d.K, d.P, interp, s, nullptr)))
     return rc;
   if (gb) rc = bias_grad<T>(gy, gb, ws, ws_bytes, d.B, d.Co, d.OH * d.OW, s);
   return rc;

@@ -394,7 +394,8 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
     const TD *__restrict__ plain, const TD *__restrict__ gath,
     const float *__restrict__ map, const float *__restrict__ iw, float *__restrict__ part, int A,
     int G, int GH, int GW, int MH, int MW, int K, int weighted, int wrap, int tiles_x,
-    int tiles_per_img, int tw_shift, int total_tiles, int ranges, int cgroups) {
+    int tiles_per_img, int tw_shift, int total_tiles, int ranges, int cgroups,
+    float *__restrict__ plain_sum_part) {
   constexpr int NE = NP * NCORN;  // (offset, weight) pairs per pixel and tap
   // The plain tile is only needed until each wave has copied its rows into registers;
   // the same LDS then holds the tile's resolved taps (offsets, then weights).
@@ -446,6 +447,11 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
   for (int k = 0; k < kWgKT; k++)
 #pragma unroll
     for (int cb = 0; cb < kWgCB; cb++) acc[k][cb] = floatx4{0.f, 0.f, 0.f, 0.f};
+  // Sum of the plain operand over pixels (the bias gradient of a convolution), taken from
+  // the staged tiles by the workgroups of the first channel group and tap pass: thread
+  // (row tid/4, quarter tid%4) adds 32 pixels of its row per tile.
+  const bool sum_plain = plain_sum_part != nullptr && cg == 0 && blockIdx.z == 0;
+  float plain_sum = 0.f;
 
   for (int tile = t_begin; tile < t_end; ++tile) {
     const int b = tile / tiles_per_img;
@@ -508,6 +514,30 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
         areg[4 * s4 + 2] = t.z;
         areg[4 * s4 + 3] = t.w;
       }
+    }
+
+    if (sum_plain) {
+      float t = 0.f;
+      if constexpr (kBf16) {
+        const uint4 *row = reinterpret_cast<const uint4 *>(&PtB[tid >> 2][(tid & 3) * 32]);
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const uint4 q = row[r];
+          const unsigned w4[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+          for (int j = 0; j < 4; j++)
+            t += __builtin_bit_cast(float, w4[j] << 16) +
+                 __builtin_bit_cast(float, w4[j] & 0xffff0000u);
+        }
+      } else {
+        const float4 *row = reinterpret_cast<const float4 *>(&Pt[tid >> 2][(tid & 3) * 32]);
+#pragma unroll
+        for (int r = 0; r < 8; r++) {
+          const float4 q = row[r];
+          t += (q.x + q.y) + (q.z + q.w);
+        }
+      }
+      plain_sum += t;
     }
 
     const int gi = i0 + (p >> tw_shift), gj = j0 + (p & tw_mask);
@@ -649,6 +679,12 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
     }
   }
 
+  if (sum_plain) {  // the four quarters of a row sit in neighbouring lanes
+    plain_sum += __shfl_xor(plain_sum, 1);
+    plain_sum += __shfl_xor(plain_sum, 2);
+    const int a = a0 + (tid >> 2);
+    if ((tid & 3) == 0 && a < A) plain_sum_part[(int64_t)range * A + a] = plain_sum;
+  }
   // partial gW of this workgroup: lane holds gathered channel l15 of each block and
   // plain channels a0 + 16*wave + 4*lq + i
   float *pr = part + (int64_t)range * A * G * K;
@@ -1207,21 +1243,25 @@ int mfma_gather_product(const TD *src, const float *map, const float *iw, const 
 }
 
 // ---- weight gradient ---------------------------------------------------------------
-// Per-range partial sums, then (single-row gathered operands) their channel-last copy.
+// Per-range partial sums of gW, per-range partial sums of the plain operand, then
+// (single-row gathered operands) their channel-last copy.
 size_t mfma_weight_grad_bytes(int64_t B, int64_t A, int64_t G, int64_t MH, int64_t MW, int64_t K,
                               int64_t GH, int64_t GW) {
   const PixelTiling t = make_tiling(B, MH, MW);
-  size_t n = align256((size_t)weight_grad_ranges(t.total, A, G, K) * (size_t)(A * G * K) *
-                      sizeof(float));
+  const size_t ranges = (size_t)weight_grad_ranges(t.total, A, G, K);
+  size_t n = align256(ranges * (size_t)(A * G * K) * sizeof(float));
+  n += align256(ranges * (size_t)A * sizeof(float));
   if (GH == 1) n += align256((size_t)(B * GH * GW * round_up(G, kGC)) * sizeof(float));
   return n;
 }
 
-// scratch: mfma_weight_grad_bytes(...) bytes (per-range partial sums).
+// scratch: mfma_weight_grad_bytes(...) bytes.  plain_sum (may be NULL): [A], receives the
+// sum of the plain operand over images and pixels (a convolution's bias gradient).
 template <typename TD>
 int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const float *iw, TD *gw,
                      void *scratch, int64_t B, int64_t A, int64_t G, int64_t GH, int64_t GW,
-                     int64_t MH, int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s) {
+                     int64_t MH, int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s,
+                     TD *plain_sum) {
   float *part = (float *)scratch;
   const PixelTiling t = make_tiling(B, MH, MW);
   if (t.total > 0x7fffffffLL) return MCX_E_SHAPE;
@@ -1231,9 +1271,10 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
   const int64_t Gpad = round_up(G, kGC);
   const bool cl = use_channel_last(GH, interp) &&
                   GH * GW * Gpad * (int64_t)sizeof(TD) <= 0xffffffffLL;
+  float *sum_part = reinterpret_cast<float *>((char *)scratch +
+                                              align256((size_t)ranges * (size_t)(A * G * K) * 4));
   if (cl) {
-    TD *stage = reinterpret_cast<TD *>((char *)scratch +
-                                       align256((size_t)ranges * (size_t)(A * G * K) * 4));
+    TD *stage = reinterpret_cast<TD *>((char *)sum_part + align256((size_t)ranges * A * 4));
     dim3 tg((unsigned)((GH * GW + 63) / 64), (unsigned)((Gpad + 63) / 64), (unsigned)B);
     hipLaunchKernelGGL(to_channel_last_kernel<TD>, tg, dim3(256), 0, s, gath, stage, (int)G,
                        (int)Gpad, GH * GW);
@@ -1247,7 +1288,8 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
   hipLaunchKernelGGL((weight_grad_mfma_kernel<TD, NCORN, NP, CL>), grid, dim3(kThreads), 0, s,   \
                      plain, gath, map, iw, part, (int)A, (int)G, (int)GH, (int)GW, (int)MH,      \
                      (int)MW, (int)K, m.weighted, m.wrap, t.tiles_x, t.tiles_per_img,            \
-                     t.tw_shift, (int)t.total, ranges, cgroups)
+                     t.tw_shift, (int)t.total, ranges, cgroups,                                  \
+                     plain_sum ? sum_part : (float *)nullptr)
 #define MCX_LAUNCH(NCORN, NP)              \
   if constexpr (NCORN == 1) {              \
     if (cl) {                              \
@@ -1266,6 +1308,11 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
   hipLaunchKernelGGL(reduce_partials_kernel<TD>, dim3((unsigned)((n + 63) / 64)), dim3(64), 0, s,
                      part, gw, ranges, n);
   MCX_HIP_CHECK_LAUNCH();
+  if (plain_sum) {
+    hipLaunchKernelGGL(reduce_partials_kernel<TD>, dim3((unsigned)((A + 63) / 64)), dim3(64), 0, s,
+                       sum_part, plain_sum, ranges, A);
+    MCX_HIP_CHECK_LAUNCH();
+  }
   return 0;
 }
 
@@ -1538,7 +1585,7 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
   // atomic path (runs when there is no transposed map or it overflowed)
   const int64_t total_dst = B * D * DH * DW;
   float *acc = sizeof(TD) == 4 ? (float *)dst : (float *)(base + sc.acc32);
-  const unsigned fill_blocks = (unsigned)std::min<int64_t>((total_dst + 1023) / 1024, 65536);
+  const unsigned fill_blocks = (unsigned)std::min<int64_t>((total_dst + 1023) / 1024, 8192);
   hipLaunchKernelGGL(init_planes_kernel<TD>, dim3(fill_blocks), dim3(256), 0, s, acc, bias, (int)D,
                      DH * DW, total_dst, gate, 0);
   MCX_HIP_CHECK_LAUNCH();
@@ -1630,7 +1677,7 @@ int mfma_bias_grad(const TD *g, TD *gb, void *scratch, int64_t B, int64_t C, int
                                        hipStream_t);                                              \
   template int mfma_weight_grad<TD>(const TD *, const TD *, const float *, const float *, TD *,   \
                                     void *, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, \
-                                    int64_t, int64_t, int64_t, int, hipStream_t);                 \
+                                    int64_t, int64_t, int64_t, int, hipStream_t, TD *);           \
   template int mfma_product_scatter<TD>(const TD *, const float *, const float *, const TD *,     \
                                         const TD *, TD *, void *, int64_t, int64_t, int64_t,      \
                                         int64_t, int64_t, int64_t, int64_t, int64_t, int64_t,     \
