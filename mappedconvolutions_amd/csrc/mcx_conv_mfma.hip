@@ -608,15 +608,25 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
       }
     };
     auto stage = [&](int buf) {
+      float sv[8];
 #pragma unroll
       for (int ch = 0; ch < 8; ch++) {
         float s = 0.f;
 #pragma unroll
         for (int i = 0; i < NE; i++) s = __builtin_fmaf(wt[i], v[ch][i], s);
-        if constexpr (kBf16)
-          SB[buf][half * 8 + ch][p] = from_f32<bf16_t>(s).v;
-        else
-          S[buf][half * 8 + ch][p] = s;
+        sv[ch] = s;
+      }
+      if constexpr (kBf16) {
+#pragma unroll
+        for (int c2 = 0; c2 < 4; c2++) {  // hardware round-to-nearest-even, two values at a time
+          const unsigned pk = __builtin_bit_cast(
+              unsigned, __builtin_convertvector(floatx2{sv[2 * c2], sv[2 * c2 + 1]}, bf16x2));
+          SB[buf][half * 8 + 2 * c2][p] = (uint16_t)(pk & 0xffffu);
+          SB[buf][half * 8 + 2 * c2 + 1][p] = (uint16_t)(pk >> 16);
+        }
+      } else {
+#pragma unroll
+        for (int ch = 0; ch < 8; ch++) S[buf][half * 8 + ch][p] = sv[ch];
       }
     };
 
