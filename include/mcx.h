@@ -52,6 +52,13 @@ int mcx_abi_version(void);
 /* Human-readable text for a return code of any function below. */
 const char *mcx_error_string(int code);
 
+/* Measurement aid, no counterpart in the reference.  The next convolution entry point this
+ * thread calls records the two caller-owned hipEvent_t handles on its stream right before
+ * and right after the launch of its dominant kernel (the gather-product or weight-gradient
+ * kernel), leaving out weight packing, map building and partial-sum reduction; the request
+ * is consumed by that launch.  NULL, NULL cancels a pending request. */
+int mcx_profile_dominant_kernel(void *start_event, void *stop_event);
+
 /* ---- Resample / Unresample ------------------------------------------------ */
 
 /* resample_from_map (+ weighted_resample_from_map):

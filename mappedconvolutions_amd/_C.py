@@ -19,21 +19,37 @@ _DTYPES = {torch.float32: MCX_F32, torch.float64: MCX_F64, torch.bfloat16: MCX_B
 # ops appends (label, start_event, end_event), recorded on the stream the kernels
 # are enqueued on.  Used by the benchmark to time individual kernels.
 profile_events = None
+profile_pool = []  # pre-made (start, end) event pairs, see make_event_pool
 
 # resample_to_map and the unpoolings run as gathers through a transposed map when
 # given a workspace; False selects the library's atomic-scatter form instead.
 scatter_as_gather = True
 
 
-def _timed(label, device, fn):
-    if profile_events is None:
-        return fn()
-    start = torch.cuda.Event(enable_timing=True)
-    end = torch.cuda.Event(enable_timing=True)
+def make_event_pool(n, device):
+    """n pairs of timing events whose underlying handles exist (an event gets its handle at
+    its first record), for `profile_pool`."""
     stream = torch.cuda.current_stream(device)
-    start.record(stream)
+    pool = []
+    for _ in range(n):
+        pair = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+        for e in pair:
+            e.record(stream)
+        pool.append(pair)
+    return pool
+
+
+def _timed(label, device, fn):
+    """Run one C-ABI call; with `profile_events` set and a pair left in `profile_pool`, ask
+    the library to record the pair around the call's dominant kernel (the only cost inside
+    a timed region: one extra C call and two event records)."""
+    if profile_events is None or not profile_pool:
+        return fn()
+    start, end = profile_pool.pop()
+    lib = _lib.load()
+    lib.mcx_profile_dominant_kernel(start.cuda_event, end.cuda_event)
     rc = fn()
-    end.record(stream)
+    lib.mcx_profile_dominant_kernel(None, None)
     profile_events.append((label, start, end))
     return rc
 

@@ -20,6 +20,7 @@ _sz = ctypes.c_size_t
 SIGNATURES = {
     "mcx_abi_version": (_i, []),
     "mcx_error_string": (ctypes.c_char_p, [_i]),
+    "mcx_profile_dominant_kernel": (_i, [_p, _p]),
     "mcx_resample_from_map": (_i, [_p] * 4 + [_i64] * 7 + [_i, _i, _p]),
     "mcx_resample_to_map_workspace": (_sz, [_i64] * 5 + [_i, _i]),
     "mcx_resample_to_map": (_i, [_p] * 5 + [_sz] + [_i64] * 7 + [_i, _i, _p]),

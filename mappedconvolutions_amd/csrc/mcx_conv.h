@@ -60,4 +60,7 @@ template <typename TD>
 int mfma_bias_grad(const TD *g, TD *gb, void *scratch, int64_t B, int64_t C, int64_t N,
                    hipStream_t s);
 
+// One-shot timing of the next gather-product / weight-gradient kernel launched by this thread.
+void set_profile_events(void *start, void *stop);
+
 }  // namespace mcx

@@ -16,6 +16,19 @@
 namespace mcx {
 namespace {
 
+// One-shot kernel timing (see mcx_profile_dominant_kernel): a pair of caller-owned events
+// recorded right before and after the next launch of a gather-product or weight-gradient
+// kernel made by the calling thread.
+thread_local hipEvent_t g_prof_start = nullptr, g_prof_stop = nullptr;
+inline void profile_begin(hipStream_t s) {
+  if (g_prof_start) (void)hipEventRecord(g_prof_start, s);
+}
+inline void profile_end(hipStream_t s) {
+  if (g_prof_stop) (void)hipEventRecord(g_prof_stop, s);
+  g_prof_start = g_prof_stop = nullptr;
+}
+
+
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int kThreads = 256;
@@ -1199,7 +1212,9 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
   } else {                                                  \
     MCX_LAUNCH_OG(NCORN, NP, 1);                            \
   }
+  profile_begin(s);
   MCX_DISPATCH_TAPS(m, MCX_LAUNCH)
+  profile_end(s);
 #undef MCX_LAUNCH
 #undef MCX_LAUNCH_OG
 #undef MCX_LAUNCH_CL
@@ -1310,7 +1325,9 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
   } else {                                 \
     MCX_LAUNCH_CL(NCORN, NP, false);       \
   }
+  profile_begin(s);
   MCX_DISPATCH_TAPS(m, MCX_LAUNCH)
+  profile_end(s);
 #undef MCX_LAUNCH
 #undef MCX_LAUNCH_CL
   MCX_HIP_CHECK_LAUNCH();
@@ -1697,4 +1714,11 @@ int mfma_bias_grad(const TD *g, TD *gb, void *scratch, int64_t B, int64_t C, int
 MCX_INSTANTIATE_TD(float)
 MCX_INSTANTIATE_TD(bf16_t)
 
+}  // namespace mcx
+
+namespace mcx {
+void set_profile_events(void *start, void *stop) {
+  g_prof_start = (hipEvent_t)start;
+  g_prof_stop = (hipEvent_t)stop;
+}
 }  // namespace mcx
