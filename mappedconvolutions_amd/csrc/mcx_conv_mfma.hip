@@ -400,16 +400,46 @@ constexpr int kWgCB = 2;            // 16-channel blocks of gathered channels pe
 constexpr int kWgKT = 9;            // taps per pass (accumulators in registers)
 constexpr int kLdPx = kTilePx + 4;  // LDS row stride (floats)
 
+// mask[0] |= bit (point * NCORN + corner) for every pair of the map with a nonzero weight.
+template <int NCORN>
+__global__ void map_pair_mask_kernel(const float *__restrict__ map, const float *__restrict__ iw,
+                                     int *__restrict__ mask, int np, int weighted, int wrap,
+                                     int GH, int GW, int64_t total) {
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  unsigned m = 0;
+  if (e < total) {
+    for (int sp = 0; sp < np; sp++) {
+      const int64_t q = e * np + sp;
+      PairTap<NCORN> t;
+      resolve_pairs<NCORN, 4>(map[q * 2], map[q * 2 + 1], GH, GW, wrap != 0,
+                              weighted ? iw[q] : 1.f, t);
+#pragma unroll
+      for (int i = 0; i < NCORN; i++)
+        if (t.wt[i] != 0.f) m |= 1u << (sp * NCORN + i);
+    }
+  }
+  for (int d = 32; d > 0; d >>= 1) m |= __shfl_xor(m, d);
+  if ((threadIdx.x & 63) == 0 && m) atomicOr(mask, (int)m);
+}
+
 // CL: `gath` is a channel-last copy [B][GH*GW][Gpad] of the gathered operand (see the
 // gather-product kernel).
-template <typename TD, int NCORN, int NP, bool CL>
+// NA: leading (offset, weight) pairs of a tap that are loaded and added.  NA < NP*NCORN is
+// valid when the remaining pairs are zero for every sample of the map (bilinear corners of
+// integral row coordinates, unused points); map_pair_mask_kernel finds that out on the
+// device and `pair_mask` / `run_if_leading` let exactly one of two launched variants run.
+template <typename TD, int NCORN, int NP, bool CL, int NA>
 __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad_mfma_kernel(
     const TD *__restrict__ plain, const TD *__restrict__ gath,
     const float *__restrict__ map, const float *__restrict__ iw, float *__restrict__ part, int A,
     int G, int GH, int GW, int MH, int MW, int K, int weighted, int wrap, int tiles_x,
     int tiles_per_img, int tw_shift, int total_tiles, int ranges, int cgroups,
-    float *__restrict__ plain_sum_part) {
+    float *__restrict__ plain_sum_part, const int *__restrict__ pair_mask, int run_if_leading) {
   constexpr int NE = NP * NCORN;  // (offset, weight) pairs per pixel and tap
+  static_assert(NA >= 1 && NA <= NE, "NA counts leading pairs");
+  // two variants are launched, with NA == 2 (run_if_leading) and NA == NE; the map's mask of
+  // pairs in use decides which of them does the work
+  if (pair_mask && (((unsigned)*pair_mask < (1u << 2)) != (run_if_leading != 0))) return;
   // The plain tile is only needed until each wave has copied its rows into registers;
   // the same LDS then holds the tile's resolved taps (offsets, then weights).
   constexpr int kPtFloats = kWgA * kLdPx;
@@ -579,7 +609,7 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
     auto load_tap = [&](int k) {  // k: tap within this pass
       if (kCacheTaps) {
 #pragma unroll
-        for (int i = 0; i < NE; i++) {
+        for (int i = 0; i < NA; i++) {
           off[i] = TapOff[k][p][i];
           wt[i] = TapWt[k][p][i];
         }
@@ -594,7 +624,7 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
         // padded count reads the last valid group (its products are not stored)
         const char *base = reinterpret_cast<const char *>(gath_b + min(g0, Gpad - 8));
 #pragma unroll
-        for (int i = 0; i < NE; i++) {
+        for (int i = 0; i < NA; i++) {
           const char *row = base + off[i];
           if constexpr (kBf16) {
             const uint4 q = *reinterpret_cast<const uint4 *>(row);
@@ -616,7 +646,7 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
         for (int ch = 0; ch < 8; ch++) {
           const TD *pl = gath_b + (int64_t)min(g0 + ch, G - 1) * gplane;
 #pragma unroll
-          for (int i = 0; i < NE; i++) v[ch][i] = load_at(pl, off[i]);
+          for (int i = 0; i < NA; i++) v[ch][i] = load_at(pl, off[i]);
         }
       }
     };
@@ -626,7 +656,7 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
       for (int ch = 0; ch < 8; ch++) {
         float s = 0.f;
 #pragma unroll
-        for (int i = 0; i < NE; i++) s = __builtin_fmaf(wt[i], v[ch][i], s);
+        for (int i = 0; i < NA; i++) s = __builtin_fmaf(wt[i], v[ch][i], s);
         sv[ch] = s;
       }
       if constexpr (kBf16) {
@@ -1276,6 +1306,7 @@ size_t mfma_weight_grad_bytes(int64_t B, int64_t A, int64_t G, int64_t MH, int64
   const size_t ranges = (size_t)weight_grad_ranges(t.total, A, G, K);
   size_t n = align256(ranges * (size_t)(A * G * K) * sizeof(float));
   n += align256(ranges * (size_t)A * sizeof(float));
+  n += 256;  // the map's pair mask
   if (GH == 1) n += align256((size_t)(B * GH * GW * round_up(G, kGC)) * sizeof(float));
   return n;
 }
@@ -1298,8 +1329,9 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
                   GH * GW * Gpad * (int64_t)sizeof(TD) <= 0xffffffffLL;
   float *sum_part = reinterpret_cast<float *>((char *)scratch +
                                               align256((size_t)ranges * (size_t)(A * G * K) * 4));
+  int *pair_mask = reinterpret_cast<int *>((char *)sum_part + align256((size_t)ranges * A * 4));
   if (cl) {
-    TD *stage = reinterpret_cast<TD *>((char *)sum_part + align256((size_t)ranges * A * 4));
+    TD *stage = reinterpret_cast<TD *>((char *)pair_mask + 256);
     dim3 tg((unsigned)((GH * GW + 63) / 64), (unsigned)((Gpad + 63) / 64), (unsigned)B);
     hipLaunchKernelGGL(to_channel_last_kernel<TD>, tg, dim3(256), 0, s, gath, stage, (int)G,
                        (int)Gpad, GH * GW);
@@ -1309,12 +1341,35 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
   dim3 grid((unsigned)(ranges * cgroups), (unsigned)((A + kWgA - 1) / kWgA),
             (unsigned)((K + kWgKT - 1) / kWgKT));
   const ModeArgs m = mode_args(interp, P);
-#define MCX_LAUNCH_CL(NCORN, NP, CL)                                                             \
-  hipLaunchKernelGGL((weight_grad_mfma_kernel<TD, NCORN, NP, CL>), grid, dim3(kThreads), 0, s,   \
-                     plain, gath, map, iw, part, (int)A, (int)G, (int)GH, (int)GW, (int)MH,      \
+  // bf16 storage with four pairs per tap: the kernel is bound by its gathers, so it pays to
+  // find out (on the device) whether only the first two pairs are ever in use and to launch
+  // both variants, of which one returns at once.
+  const bool two_variants = sizeof(TD) == 2 && m.np * (m.mode == kInterpNearest ? 1 : 4) == 4;
+  if (two_variants) {
+    if (int rc = fill_f32((float *)pair_mask, 1, 0.f, s)) return rc;
+    const int64_t samples = MH * MW * K;
+    const dim3 mg((unsigned)((samples + 255) / 256));
+    if (m.mode == kInterpNearest)
+      hipLaunchKernelGGL(map_pair_mask_kernel<1>, mg, dim3(256), 0, s, map, iw, pair_mask, m.np,
+                         m.weighted, m.wrap, (int)GH, (int)GW, samples);
+    else
+      hipLaunchKernelGGL(map_pair_mask_kernel<4>, mg, dim3(256), 0, s, map, iw, pair_mask, m.np,
+                         m.weighted, m.wrap, (int)GH, (int)GW, samples);
+    MCX_HIP_CHECK_LAUNCH();
+  }
+#define MCX_LAUNCH_NA(NCORN, NP, CL, NA, MASK, LEAD)                                             \
+  hipLaunchKernelGGL((weight_grad_mfma_kernel<TD, NCORN, NP, CL, NA>), grid, dim3(kThreads), 0,  \
+                     s, plain, gath, map, iw, part, (int)A, (int)G, (int)GH, (int)GW, (int)MH,   \
                      (int)MW, (int)K, m.weighted, m.wrap, t.tiles_x, t.tiles_per_img,            \
                      t.tw_shift, (int)t.total, ranges, cgroups,                                  \
-                     plain_sum ? sum_part : (float *)nullptr)
+                     plain_sum ? sum_part : (float *)nullptr, MASK, LEAD)
+#define MCX_LAUNCH_CL(NCORN, NP, CL)                                          \
+  if constexpr (sizeof(TD) == 2 && NCORN * NP == 4) {                         \
+    MCX_LAUNCH_NA(NCORN, NP, CL, 2, pair_mask, 1);                            \
+    MCX_LAUNCH_NA(NCORN, NP, CL, NCORN * NP, pair_mask, 0);                   \
+  } else {                                                                    \
+    MCX_LAUNCH_NA(NCORN, NP, CL, NCORN * NP, (const int *)nullptr, 0);        \
+  }
 #define MCX_LAUNCH(NCORN, NP)              \
   if constexpr (NCORN == 1) {              \
     if (cl) {                              \
@@ -1329,6 +1384,7 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
   MCX_DISPATCH_TAPS(m, MCX_LAUNCH)
   profile_end(s);
 #undef MCX_LAUNCH
+#undef MCX_LAUNCH_NA
 #undef MCX_LAUNCH_CL
   MCX_HIP_CHECK_LAUNCH();
   const int64_t n = A * G * K;

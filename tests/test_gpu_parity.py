@@ -260,6 +260,35 @@ def test_conv_bf16_vs_fp32_oracle(interp, p, device):
         assert rel_err(a.float(), r) < 2e-2, nm
 
 
+@pytest.mark.parametrize("interp", [0, 1])
+def test_conv_bf16_two_leading_pairs(interp, device):
+    """Maps that use only the first two (offset, weight) pairs of a tap take the weight
+    gradient's reduced variant: nearest with P=4 whose last two interp weights are zero, and
+    bilinear with integral rows (the lower corners weigh exactly zero)."""
+    g = torch.Generator().manual_seed(720 + interp)
+    B, Ci, Co, IH, IW, OH, OW, K = 2, 40, 24, 18, 44, 14, 38, 7
+    bf = lambda t: t.to(torch.bfloat16)
+    p = 4 if interp == 0 else 0
+    smap, wts = helpers.random_map(g, OH, OW, K, p, IH, IW, torch.float32)
+    if interp == 0:
+        wts[..., 2:] = 0
+    else:
+        smap[..., 1] = smap[..., 1].round()
+    x = bf(torch.randn(B, Ci, IH, IW, generator=g))
+    w = bf(torch.randn(Co, Ci, K, generator=g) / 8)
+    b = bf(torch.randn(Co, generator=g))
+    gy = bf(torch.randn(B, Co, OH, OW, generator=g))
+    if p:
+        g_o = O.weighted_mapped_conv_backward(gy.float(), smap, wts, x.float(), w.float(),
+                                              b.float(), K, interp)
+        gr = _C.weighted_mapped_conv_backward(*dev(gy, smap, wts, x, w, b), K, interp)
+    else:
+        g_o = O.mapped_conv_backward(gy.float(), smap, x.float(), w.float(), b.float(), K, interp)
+        gr = _C.mapped_conv_backward(*dev(gy, smap, x, w, b), K, interp)
+    for a, r, nm in zip(gr, g_o, ("grad_input", "grad_weight", "grad_bias")):
+        assert rel_err(a.float(), r) < 2e-2, nm
+
+
 def test_transposed_conv_bf16(device):
     g = torch.Generator().manual_seed(720)
     B, Ci, Co, IH, IW, OH, OW, K = 2, 16, 24, 10, 33, 14, 40, 4
