@@ -192,6 +192,40 @@ int mcx_tconv_backward(const void *gy, const void *map, const void *iw, const vo
 int mcx_knn(const void *ref, const void *query, int64_t *idx, void *dist, int64_t B, int64_t D,
             int64_t R, int64_t Q, int64_t k, int dtype, void *stream);
 
+/* ---- sample-map builders and cube-map resampling ----------------------------- */
+
+enum {
+  MCX_PROJ_GRID = 0,            /* lon/lat grid in radians: grid_projection_map */
+  MCX_PROJ_GNOMONIC = 1,        /* reverse_gnomonic_projection_map + convert_spherical_to_image */
+  MCX_PROJ_EQUIRECTANGULAR = 2, /* reverse_equirectangular_projection_map + conversion */
+  MCX_PROJ_PERSPECTIVE = 3      /* perspective_projection_map (the pixel grid) */
+};
+
+/* get_projection_map / get_perspective_projection_map:
+ * package/layers/util/spherical_projections.py:12-24, 33-35 (builders :39-193,
+ * conversion package/layers/util/conversions.py:6-17).  Writes the float sample map
+ * [ceil(H/stride), ceil(W/stride), kh*kw, 2] of an H x W equirectangular (or, for
+ * MCX_PROJ_PERSPECTIVE, plain) image, (x, y) last, on the device.  `dilation` is used
+ * by GRID and PERSPECTIVE only, like in the reference.  Entries are evaluated in double
+ * and rounded once.  H >= 2 for the three spherical projections; at most 65535 output
+ * rows. */
+int mcx_projection_map(float *out, int64_t H, int64_t W, int64_t kh, int64_t kw, int proj,
+                       int64_t stride, int64_t dilation, void *stream);
+
+/* get_reverse_cube_projection_map: spherical_projections.py:26-30 (:261-311,
+ * conversions.py:20-181, grids.py:23-37).  Float sample map
+ * [ceil(dim/stride), ceil(6*dim/stride), kh*kw, 2] into the dim x 6*dim cube-map image
+ * with faces [-z, -x, +z, +x, +y, -y]. */
+int mcx_cube_projection_map(float *out, int64_t cube_dim, int64_t kh, int64_t kw, int64_t stride,
+                            void *stream);
+
+/* cube2rect: include/util/layers/cube2rect_layer.h:29-43, kernel
+ * include/util/cuda/cube2rect.cuh:16-64, host src/util/cuda/cube2rect_layer.cu:11-29.
+ * cubemap [C, dim, 6*dim] -> rect [C, RH, RW]; interp 1 bilinear, anything else nearest;
+ * F32 and F64. */
+int mcx_cube2rect(const void *cubemap, void *rect, int64_t C, int64_t cube_dim, int64_t RH,
+                  int64_t RW, int interp, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -505,3 +505,61 @@ def knn_forward(ref, query, k):
                                  _stream(ref))
     _lib.check(rc, "knn_forward")
     return [idx, dist]
+
+
+# ------------------------------------------------------- map builders, cube2rect
+PROJECTIONS = {"grid": 0, "gnomonic": 1, "equirectangular": 2, "perspective": 3}
+
+
+def projection_map(shape, kernel_size, proj, stride, dilation, device):
+    """Sample map [ceil(H/stride), ceil(W/stride), kh*kw, 2] (float32, on `device`) of the
+    reference's host-side builders, package/layers/util/spherical_projections.py:12-24,33-35;
+    `proj` is a key of PROJECTIONS."""
+    H, W = (int(v) for v in shape)
+    kh, kw = (int(v) for v in kernel_size)
+    stride, dilation = int(stride), int(dilation)
+    device = torch.device(device)
+    if device.type != "cuda":
+        raise RuntimeError("maps are built on the GPU: this backend has no CPU implementation")
+    out = torch.empty((-(-H // stride), -(-W // stride), kh * kw, 2), dtype=torch.float32,
+                      device=device)
+    with torch.cuda.device(device):
+        rc = _lib.load().mcx_projection_map(_ptr(out), H, W, kh, kw, PROJECTIONS[proj], stride,
+                                            dilation, _stream(out))
+    _lib.check(rc, "projection_map")
+    return out
+
+
+def cube_projection_map(cube_dim, kernel_size, stride, device):
+    """spherical_projections.py:26-30 -> [ceil(dim/stride), ceil(6*dim/stride), kh*kw, 2]."""
+    dim, stride = int(cube_dim), int(stride)
+    kh, kw = (int(v) for v in kernel_size)
+    device = torch.device(device)
+    if device.type != "cuda":
+        raise RuntimeError("maps are built on the GPU: this backend has no CPU implementation")
+    out = torch.empty((-(-dim // stride), -(-6 * dim // stride), kh * kw, 2),
+                      dtype=torch.float32, device=device)
+    with torch.cuda.device(device):
+        rc = _lib.load().mcx_cube_projection_map(_ptr(out), dim, kh, kw, stride, _stream(out))
+    _lib.check(rc, "cube_projection_map")
+    return out
+
+
+def cube2rect(cubemap, rect_height, rect_width, interpolation):
+    """include/util/layers/cube2rect_layer.h:29-43: cubemap [C, dim, 6*dim] with faces
+    [-z, -x, +z, +x, +y, -y] -> equirectangular [C, rect_height, rect_width]."""
+    _contig(cubemap=cubemap)
+    _on_gpu("cubemap", cubemap)
+    if cubemap.dtype not in (torch.float32, torch.float64):
+        raise RuntimeError("unsupported dtype %s" % cubemap.dtype)
+    if cubemap.dim() != 3 or cubemap.shape[2] != 6 * cubemap.shape[1]:
+        raise RuntimeError("cubemap must be [C, dim, 6*dim], got %s" % (tuple(cubemap.shape),))
+    C, dim = cubemap.shape[0], cubemap.shape[1]
+    RH, RW = int(rect_height), int(rect_width)
+    rect = torch.empty((C, RH, RW), dtype=cubemap.dtype, device=cubemap.device)
+    with torch.cuda.device(cubemap.device):
+        rc = _lib.load().mcx_cube2rect(_ptr(cubemap), _ptr(rect), C, dim, RH, RW,
+                                       int(interpolation), _DTYPES[cubemap.dtype],
+                                       _stream(cubemap))
+    _lib.check(rc, "cube2rect")
+    return rect

@@ -32,6 +32,7 @@ _EXT_MODULES = {
     "_resample": ["resample_to_map", "resample_from_map"],
     "_weighted_resample": ["weighted_resample_to_map", "weighted_resample_from_map"],
     "_knn": ["knn_forward"],
+    "_cube2rect": ["cube2rect"],
 }
 
 

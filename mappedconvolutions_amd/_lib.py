@@ -38,6 +38,9 @@ SIGNATURES = {
     "mcx_tconv_backward_workspace": (_sz, [_i64] * 9 + [_i]),
     "mcx_tconv_backward": (_i, [_p] * 9 + [_sz] + [_i64] * 9 + [_i, _i, _p]),
     "mcx_knn": (_i, [_p] * 4 + [_i64] * 5 + [_i, _p]),
+    "mcx_projection_map": (_i, [_p] + [_i64] * 4 + [_i] + [_i64] * 2 + [_p]),
+    "mcx_cube_projection_map": (_i, [_p] + [_i64] * 4 + [_p]),
+    "mcx_cube2rect": (_i, [_p] * 2 + [_i64] * 4 + [_i, _i, _p]),
 }
 
 _lib = None

@@ -4,8 +4,8 @@
 
 Each workload is one of the reference configurations other than the headline one
 (which `bench.py` at the repository root measures): the weighted mesh convolution,
-the cube-to-equirectangular resampling with pooling, KNN, and the encoder-scale
-bf16 convolution.  For every op the script prints one JSON line with the time per
+the cube-to-equirectangular resampling with pooling, KNN, the encoder-scale
+bf16 convolution, and the sample-map builders.  For every op the script prints one JSON line with the time per
 call (events on the launch stream, inputs resident in HBM), the algorithmic bytes
 or flops of the call and the fraction of the MI355X roofline that bounds it.
 """
@@ -128,7 +128,26 @@ def config5(dev):
           flops=2 * flop, peak_tflops=BF16_MFMA_TFLOPS)
 
 
-WORKLOADS = {"config3": config3, "config4": config4, "knn": knn, "config5": config5}
+def maps(dev):
+    """Map builders at the encoder scale (512x1024, 5x5) and cube2rect of config 4's cube."""
+    from .util import (cube_to_rect, get_projection_map, get_reverse_cube_projection_map)
+    H, W, ks = 512, 1024, (5, 5)
+    out_bytes = H * W * 25 * 2 * 4
+    for proj in ("gnomonic", "equirectangular"):
+        _line("projection map %s 512x1024 5x5" % proj,
+              _time(lambda: get_projection_map((H, W), ks, proj, device=dev)), nbytes=out_bytes)
+    _line("cube projection map dim 256 3x3",
+          _time(lambda: get_reverse_cube_projection_map(256, (3, 3), device=dev)),
+          nbytes=256 * 1536 * 9 * 2 * 4)
+    cube = torch.rand(64, 256, 6 * 256, device=dev)
+    for interp in ("nearest", "bilinear"):
+        _line("cube2rect %s C=64 dim 256 -> 512x1024" % interp,
+              _time(lambda: cube_to_rect(cube, H, W, interp)),
+              nbytes=cube.numel() * 4 + 64 * H * W * 4)
+
+
+WORKLOADS = {"config3": config3, "config4": config4, "knn": knn, "config5": config5,
+             "maps": maps}
 
 
 def main(argv):

@@ -397,7 +397,7 @@ extern "C" int mcx_tconv_backward(const void *gy, const void *map, const void *i
                                                 workspace_bytes, d, interp, s));
 }
 
-extern "C" int mcx_abi_version(void) { return 5; }
+extern "C" int mcx_abi_version(void) { return 6; }
 
 extern "C" int mcx_profile_dominant_kernel(void *start_event, void *stop_event) {
   mcx::set_profile_events(start_event, stop_event);

@@ -1,4 +1,7 @@
 from .point_functions import knn
+from .spherical_projections import (get_projection_map, get_perspective_projection_map,
+                                    get_reverse_cube_projection_map, cube_to_rect)
 from .synthetic import (latitude_map, cube_to_equirect_map, mesh_weighted_map, sphere_points)
 
-__all__ = ['knn', 'latitude_map', 'cube_to_equirect_map', 'mesh_weighted_map', 'sphere_points']
+__all__ = ['knn', 'get_projection_map', 'get_perspective_projection_map',
+           'get_reverse_cube_projection_map', 'cube_to_rect', 'latitude_map', 'cube_to_equirect_map', 'mesh_weighted_map', 'sphere_points']
