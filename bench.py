@@ -41,7 +41,7 @@ MEASURED_TRAFFIC_BYTES = {
 KERNEL_OF = {
     "conv_forward": "gather_product_mfma_kernel<float,4,1,1,false>",
     "conv_backward_input": "gather_product_mfma_kernel<float,1,4,1,false>",
-    "conv_backward_weight": "weight_grad_mfma_kernel<float,4,1,false,4>",
+    "conv_backward_weight": "weight_grad_mfma_kernel<float,4,1,false,2>",
 }
 
 

@@ -401,13 +401,18 @@ constexpr int kWgKT = 9;            // taps per pass (accumulators in registers)
 constexpr int kLdPx = kTilePx + 4;  // LDS row stride (floats)
 
 // mask[0] |= bit (point * NCORN + corner) for every pair of the map with a nonzero weight.
+// Grid-stride over the samples and one global access per workgroup: every access goes to
+// the same address and is served one at a time.
 template <int NCORN>
 __global__ void map_pair_mask_kernel(const float *__restrict__ map, const float *__restrict__ iw,
                                      int *__restrict__ mask, int np, int weighted, int wrap,
                                      int GH, int GW, int64_t total) {
-  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  __shared__ unsigned block_mask;
+  if (threadIdx.x == 0) block_mask = 0;
+  __syncthreads();
   unsigned m = 0;
-  if (e < total) {
+  for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total;
+       e += (int64_t)gridDim.x * blockDim.x) {
     for (int sp = 0; sp < np; sp++) {
       const int64_t q = e * np + sp;
       PairTap<NCORN> t;
@@ -419,7 +424,9 @@ __global__ void map_pair_mask_kernel(const float *__restrict__ map, const float 
     }
   }
   for (int d = 32; d > 0; d >>= 1) m |= __shfl_xor(m, d);
-  if ((threadIdx.x & 63) == 0 && m) atomicOr(mask, (int)m);
+  if ((threadIdx.x & 63) == 0 && m) atomicOr(&block_mask, m);
+  __syncthreads();
+  if (threadIdx.x == 0 && block_mask) atomicOr(mask, (int)block_mask);
 }
 
 // CL: `gath` is a channel-last copy [B][GH*GW][Gpad] of the gathered operand (see the
@@ -1341,14 +1348,14 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
   dim3 grid((unsigned)(ranges * cgroups), (unsigned)((A + kWgA - 1) / kWgA),
             (unsigned)((K + kWgKT - 1) / kWgKT));
   const ModeArgs m = mode_args(interp, P);
-  // bf16 storage with four pairs per tap: the kernel is bound by its gathers, so it pays to
-  // find out (on the device) whether only the first two pairs are ever in use and to launch
-  // both variants, of which one returns at once.
-  const bool two_variants = sizeof(TD) == 2 && m.np * (m.mode == kInterpNearest ? 1 : 4) == 4;
+  // Four pairs per tap: it pays to find out (on the device) whether only the first two pairs
+  // are ever in use (bilinear maps with integral rows, two of four points weighted) and to
+  // launch both variants, of which one returns at once.
+  const bool two_variants = m.np * (m.mode == kInterpNearest ? 1 : 4) == 4;
   if (two_variants) {
     if (int rc = fill_f32((float *)pair_mask, 1, 0.f, s)) return rc;
     const int64_t samples = MH * MW * K;
-    const dim3 mg((unsigned)((samples + 255) / 256));
+    const dim3 mg((unsigned)std::min<int64_t>((samples + 255) / 256, 512));
     if (m.mode == kInterpNearest)
       hipLaunchKernelGGL(map_pair_mask_kernel<1>, mg, dim3(256), 0, s, map, iw, pair_mask, m.np,
                          m.weighted, m.wrap, (int)GH, (int)GW, samples);
@@ -1364,7 +1371,7 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
                      t.tw_shift, (int)t.total, ranges, cgroups,                                  \
                      plain_sum ? sum_part : (float *)nullptr, MASK, LEAD)
 #define MCX_LAUNCH_CL(NCORN, NP, CL)                                          \
-  if constexpr (sizeof(TD) == 2 && NCORN * NP == 4) {                         \
+  if constexpr (NCORN * NP == 4) {                                            \
     MCX_LAUNCH_NA(NCORN, NP, CL, 2, pair_mask, 1);                            \
     MCX_LAUNCH_NA(NCORN, NP, CL, NCORN * NP, pair_mask, 0);                   \
   } else {                                                                    \
