@@ -134,14 +134,22 @@ struct OperandTiles<bf16_t> {  // bf16: 16-byte groups of 8 channels, [kg][pixel
 // to_channel_last_kernel): a sample's 8 channels are then one or two 16-byte loads from
 // one cache line instead of 8 loads from 8 lines.  Used for single-row sources (mesh
 // signals), whose maps point anywhere.
-template <typename TD, int NCORN, int NP, int OG, bool CL>
+// NA: leading (offset, weight) pairs of a tap that are loaded and added.  NA == NP * NCORN is
+// the general form, which skips the pairs a tile's mask shows to be zero across the tile.
+// NA == 2 (four-pair taps) is the branch-free form for maps that use nothing but the first
+// two pairs anywhere (bilinear with integral rows, transposed maps with at most two
+// contributions per cell): both forms are launched and `pair_mask` (bit i: pair i in use
+// somewhere in the map) lets exactly one of them run.
+template <typename TD, int NCORN, int NP, int OG, bool CL, int NA>
 __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma_kernel(
     const TD *__restrict__ src, const float *__restrict__ map, const float *__restrict__ iw,
     const float *__restrict__ wp, const TD *__restrict__ bias, TD *__restrict__ y, int G,
     int O, int Opad, int Gpad, int SH, int SW, int OH, int OW, int K, int weighted, int wrap,
     int tiles_x, int tiles_per_img, int tw_shift, const int *__restrict__ gate, int run_if_zero,
-    const float *__restrict__ addend) {
+    const float *__restrict__ addend, const int *__restrict__ pair_mask, int run_if_leading) {
   constexpr int NE = NP * NCORN;         // (offset, weight) pairs per pixel and tap
+  static_assert(NA >= 1 && NA <= NE, "NA counts leading pairs");
+  constexpr bool kMasked = NA == NE;
   constexpr int TG = kTapCache / NE > 0 ? kTapCache / NE : 1;  // taps cached in LDS at a time
   constexpr bool kBf16 = sizeof(TD) == 2;
   __shared__ __attribute__((aligned(16))) OperandTiles<TD> T;
@@ -153,6 +161,7 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
   // accumulated.
   __shared__ unsigned TapMask[TG][2][2];
   if (gate && ((*gate == 0) != (run_if_zero != 0))) return;  // device-side path selection
+  if (pair_mask && (((unsigned)*pair_mask < (1u << 2)) != (run_if_leading != 0))) return;
 
   const int tid = threadIdx.x;
   const int tile = xcd_contiguous_tile(blockIdx.x, gridDim.x);
@@ -184,10 +193,11 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
   const int w_off = (tid >> 4) * Opad + (tid & 15) * 4;
 
   auto load_tap = [&](int kl) {  // cached pairs of tap kl of the group -> registers
-    tmask = __builtin_amdgcn_readfirstlane(TapMask[kl][0][0] | TapMask[kl][0][1] |
-                                           TapMask[kl][1][0] | TapMask[kl][1][1]);
+    if constexpr (kMasked)
+      tmask = __builtin_amdgcn_readfirstlane(TapMask[kl][0][0] | TapMask[kl][0][1] |
+                                             TapMask[kl][1][0] | TapMask[kl][1][1]);
 #pragma unroll
-    for (int i = 0; i < NE; i++) {
+    for (int i = 0; i < NA; i++) {
       off[i] = TapOff[kl][p][i];
       wt[i] = TapWt[kl][p][i];
     }
@@ -207,8 +217,8 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
   };
   auto issue = [&](int k, int c) {
 #pragma unroll
-    for (int i = 0; i < NE; i++) {
-      if (!((tmask >> i) & 1u)) continue;  // wave-uniform
+    for (int i = 0; i < NA; i++) {
+      if (kMasked && !((tmask >> i) & 1u)) continue;  // wave-uniform
       if constexpr (CL) {
         const char *row = reinterpret_cast<const char *>(pl[0]) + off[i];
         if constexpr (kBf16) {
@@ -252,8 +262,8 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
 #pragma unroll
     for (int ch = 0; ch < 8; ch++) sv[ch] = 0.f;
 #pragma unroll
-    for (int i = 0; i < NE; i++) {
-      if (!((tmask >> i) & 1u)) continue;
+    for (int i = 0; i < NA; i++) {
+      if (kMasked && !((tmask >> i) & 1u)) continue;
 #pragma unroll
       for (int ch = 0; ch < 8; ch++) sv[ch] = __builtin_fmaf(wt[i], v[ch][i], sv[ch]);
     }
@@ -1203,7 +1213,8 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
                           const TD *bias, TD *y, TD *stage, int64_t B, int64_t G, int64_t O,
                           int64_t SH, int64_t SW, int64_t OH, int64_t OW, int64_t K, int64_t P,
                           int interp, const int *gate, int run_if_zero, hipStream_t s,
-                          const float *addend = nullptr, bool staged = false) {
+                          const float *addend = nullptr, bool staged = false,
+                          const int *pair_mask = nullptr) {
   const int Opad = (int)round_up(O, kOT), Gpad = (int)round_up(G, kGC);
   const bool cl = stage != nullptr && use_channel_last(SH, interp) &&
                   SH * SW * Gpad * (int64_t)sizeof(TD) <= 0xffffffffLL;
@@ -1224,11 +1235,24 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
   const bool wide = sizeof(TD) == 2 && Opad % (2 * kOT) == 0;
   dim3 grid((unsigned)t.total, (unsigned)(Opad / (wide ? 2 * kOT : kOT)));
   const ModeArgs m = mode_args(interp, P);
-#define MCX_LAUNCH_CL(NCORN, NP, OG, CL)                                                         \
-  hipLaunchKernelGGL((gather_product_mfma_kernel<TD, NCORN, NP, OG, CL>), grid, dim3(kThreads),  \
-                     0, s, src, map, iw, wp, bias, y, (int)G, (int)O, Opad, Gpad, (int)SH,       \
-                     (int)SW, (int)OH, (int)OW, (int)K, m.weighted, m.wrap, t.tiles_x,           \
-                     t.tiles_per_img, t.tw_shift, gate, run_if_zero, addend)
+  // `pair_mask` (four-pair taps only): launch the two-pair form as well; the mask picks one
+#define MCX_LAUNCH_NA(NCORN, NP, OG, CL, NA, MASK, LEAD)                                         \
+  hipLaunchKernelGGL((gather_product_mfma_kernel<TD, NCORN, NP, OG, CL, NA>), grid,              \
+                     dim3(kThreads), 0, s, src, map, iw, wp, bias, y, (int)G, (int)O, Opad,      \
+                     Gpad, (int)SH, (int)SW, (int)OH, (int)OW, (int)K, m.weighted, m.wrap,       \
+                     t.tiles_x, t.tiles_per_img, t.tw_shift, gate, run_if_zero, addend, MASK,    \
+                     LEAD)
+#define MCX_LAUNCH_CL(NCORN, NP, OG, CL)                                      \
+  if constexpr (NCORN * NP == 4) {                                            \
+    if (pair_mask) {                                                          \
+      MCX_LAUNCH_NA(NCORN, NP, OG, CL, 2, pair_mask, 1);                      \
+      MCX_LAUNCH_NA(NCORN, NP, OG, CL, NCORN * NP, pair_mask, 0);             \
+    } else {                                                                  \
+      MCX_LAUNCH_NA(NCORN, NP, OG, CL, NCORN * NP, (const int *)nullptr, 0);  \
+    }                                                                         \
+  } else {                                                                    \
+    MCX_LAUNCH_NA(NCORN, NP, OG, CL, NCORN * NP, (const int *)nullptr, 0);    \
+  }
 #define MCX_LAUNCH_OG(NCORN, NP, OG)           \
   if constexpr (NCORN == 1) {                  \
     if (cl) {                                  \
@@ -1255,6 +1279,7 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
 #undef MCX_LAUNCH
 #undef MCX_LAUNCH_OG
 #undef MCX_LAUNCH_CL
+#undef MCX_LAUNCH_NA
   MCX_HIP_CHECK_LAUNCH();
   return 0;
 }
@@ -1276,6 +1301,21 @@ int launch_pack_weights(const TD *w, float *wp, int64_t O, int64_t G, int64_t K,
   return 0;
 }
 
+// mask[0] = OR over the map's samples of the bits of their nonzero pairs.
+int launch_pair_mask(const float *map, const float *iw, int *mask, const ModeArgs &m, int64_t GH,
+                     int64_t GW, int64_t samples, hipStream_t s) {
+  if (int rc = fill_f32((float *)mask, 1, 0.f, s)) return rc;
+  const dim3 mg((unsigned)std::min<int64_t>((samples + 255) / 256, 512));
+  if (m.mode == kInterpNearest)
+    hipLaunchKernelGGL(map_pair_mask_kernel<1>, mg, dim3(256), 0, s, map, iw, mask, m.np,
+                       m.weighted, m.wrap, (int)GH, (int)GW, samples);
+  else
+    hipLaunchKernelGGL(map_pair_mask_kernel<4>, mg, dim3(256), 0, s, map, iw, mask, m.np,
+                       m.weighted, m.wrap, (int)GH, (int)GW, samples);
+  MCX_HIP_CHECK_LAUNCH();
+  return 0;
+}
+
 }  // namespace
 
 // ---- gather-product --------------------------------------------------------------
@@ -1284,6 +1324,7 @@ int launch_pack_weights(const TD *w, float *wp, int64_t O, int64_t G, int64_t K,
 size_t mfma_gather_product_bytes(int64_t O, int64_t G, int64_t K, int64_t B, int64_t SH,
                                  int64_t SW) {
   size_t n = align256((size_t)(K * round_up(G, kGC) * round_up(O, kOT)) * sizeof(float));
+  n += 256;  // the map's pair mask
   if (SH == 1) n += align256((size_t)(B * SH * SW * round_up(G, kGC)) * sizeof(float));
   return n;
 }
@@ -1295,13 +1336,17 @@ int mfma_gather_product(const TD *src, const float *map, const float *iw, const 
                         int64_t SH, int64_t SW, int64_t OH, int64_t OW, int64_t K, int64_t P,
                         int interp, hipStream_t s) {
   float *wp = (float *)scratch;
-  TD *stage = SH == 1 ? reinterpret_cast<TD *>(
-                            (char *)scratch +
-                            align256((size_t)(K * round_up(G, kGC) * round_up(O, kOT)) * 4))
-                      : nullptr;
+  int *pair_mask = reinterpret_cast<int *>(
+      (char *)scratch + align256((size_t)(K * round_up(G, kGC) * round_up(O, kOT)) * 4));
+  TD *stage = SH == 1 ? reinterpret_cast<TD *>((char *)pair_mask + 256) : nullptr;
   if (int rc = launch_pack_weights<TD>(w, wp, O, G, K, 0, s)) return rc;
+  const ModeArgs m = mode_args(interp, P);
+  const bool four_pairs = m.np * (m.mode == kInterpNearest ? 1 : 4) == 4;
+  if (four_pairs)
+    if (int rc = launch_pair_mask(map, iw, pair_mask, m, SH, SW, OH * OW * K, s)) return rc;
   return launch_gather_product<TD>(src, map, iw, wp, bias, y, stage, B, G, O, SH, SW, OH, OW, K,
-                                   P, interp, nullptr, 0, s);
+                                   P, interp, nullptr, 0, s, nullptr, false,
+                                   four_pairs ? pair_mask : nullptr);
 }
 
 // ---- weight gradient ---------------------------------------------------------------
@@ -1352,18 +1397,8 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
   // are ever in use (bilinear maps with integral rows, two of four points weighted) and to
   // launch both variants, of which one returns at once.
   const bool two_variants = m.np * (m.mode == kInterpNearest ? 1 : 4) == 4;
-  if (two_variants) {
-    if (int rc = fill_f32((float *)pair_mask, 1, 0.f, s)) return rc;
-    const int64_t samples = MH * MW * K;
-    const dim3 mg((unsigned)std::min<int64_t>((samples + 255) / 256, 512));
-    if (m.mode == kInterpNearest)
-      hipLaunchKernelGGL(map_pair_mask_kernel<1>, mg, dim3(256), 0, s, map, iw, pair_mask, m.np,
-                         m.weighted, m.wrap, (int)GH, (int)GW, samples);
-    else
-      hipLaunchKernelGGL(map_pair_mask_kernel<4>, mg, dim3(256), 0, s, map, iw, pair_mask, m.np,
-                         m.weighted, m.wrap, (int)GH, (int)GW, samples);
-    MCX_HIP_CHECK_LAUNCH();
-  }
+  if (two_variants)
+    if (int rc = launch_pair_mask(map, iw, pair_mask, m, GH, GW, MH * MW * K, s)) return rc;
 #define MCX_LAUNCH_NA(NCORN, NP, CL, NA, MASK, LEAD)                                             \
   hipLaunchKernelGGL((weight_grad_mfma_kernel<TD, NCORN, NP, CL, NA>), grid, dim3(kThreads), 0,  \
                      s, plain, gath, map, iw, part, (int)A, (int)G, (int)GH, (int)GW, (int)MH,   \
@@ -1428,6 +1463,22 @@ struct OverflowEntry {
   int p, n, k;
   float wt;
 };
+
+// mask[0] |= bits [0, min(cnt, kTransSlots)) for every cell: the slots in use.
+__global__ void slot_mask_kernel(const int *__restrict__ cnt, int64_t cells,
+                                 int *__restrict__ mask) {
+  __shared__ unsigned block_mask;
+  if (threadIdx.x == 0) block_mask = 0;
+  __syncthreads();
+  unsigned m = 0;
+  for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < cells;
+       e += (int64_t)gridDim.x * blockDim.x)
+    m |= (1u << min(cnt[e], kTransSlots)) - 1u;
+  for (int d = 32; d > 0; d >>= 1) m |= __shfl_xor(m, d);
+  if ((threadIdx.x & 63) == 0 && m) atomicOr(&block_mask, m);
+  __syncthreads();
+  if (threadIdx.x == 0 && block_mask) atomicOr(mask, (int)block_mask);
+}
 
 template <int NCORN>
 __global__ void build_transposed_map_kernel(const float *__restrict__ map,
@@ -1580,7 +1631,7 @@ ScatterScratch scatter_scratch(int64_t B, int64_t S, int64_t D, int64_t K, int64
     sc.wpt = off;
     off += align256((size_t)(K * round_up(S, kGC) * round_up(D, kOT)) * 4);
     sc.cnt = off;  // counters, the overflow flag and list length; cleared with tmap and tiw
-    off += align256((size_t)(cells + 2) * 4);
+    off += align256((size_t)(cells + 4) * 4);
     sc.tmap = off;
     off += align256((size_t)cells * kTransSlots * 2 * 4);
     sc.tiw = off;
@@ -1642,6 +1693,10 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
                          cnt, tmap, tiw, flag, ovf, (int)sc.ovf_cap, m.np, m.weighted, m.wrap,
                          (int)DH, (int)DW, (int)MW, (int)K, entries);
     MCX_HIP_CHECK_LAUNCH();
+    // flag[2]: mask of the slots in use anywhere (bit i: some cell holds more than i entries)
+    hipLaunchKernelGGL(slot_mask_kernel, dim3((unsigned)std::min<int64_t>((cells + 255) / 256, 512)),
+                       dim3(256), 0, s, cnt, cells, flag + 2);
+    MCX_HIP_CHECK_LAUNCH();
     if (int rc = launch_pack_weights<TD>(w, wpt, D, S, K, 1, s)) return rc;
     // What did not fit the four slots of its cell is accumulated with float atomics into a
     // channel-last fp32 image (cleared only when there is anything to add), which the
@@ -1668,7 +1723,7 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
     MCX_HIP_CHECK_LAUNCH();
     if (int rc = launch_gather_product<TD>(src, tmap, tiw, wpt, bias, dst, stage, B, S, D, MH, MW,
                                            DH, DW, K, kTransSlots, kInterpNearest, gate, 1, s, img,
-                                           cl))
+                                           cl, flag + 2))
       return rc;
   }
 
