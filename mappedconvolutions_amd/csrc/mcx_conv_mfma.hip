@@ -305,20 +305,23 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
     __syncthreads();
     for (int kl = half; kl < kn; kl += 2) {
       unsigned m = 0;
+      // points whose pairs all lie beyond the leading NA are known to weigh nothing
+      constexpr int kPoints = (NA + NCORN - 1) / NCORN;
 #pragma unroll
-      for (int sp = 0; sp < NP; sp++) {
+      for (int sp = 0; sp < kPoints; sp++) {
         const int64_t e = (n_g * K + k0 + kl) * NP + sp;
         PairTap<NCORN> t;
         resolve_pairs<NCORN, sizeof(TD)>(map[e * 2], map[e * 2 + 1], SH, SW, wrap != 0,
                                          live ? (weighted ? iw[e] : 1.f) : 0.f, t);
 #pragma unroll
         for (int i = 0; i < NCORN; i++) {
+          if (sp * NCORN + i >= NA) continue;
           TapOff[kl][p][sp * NCORN + i] = CL ? t.off[i] * (unsigned)Gpad : t.off[i];
           TapWt[kl][p][sp * NCORN + i] = t.wt[i];
-          if (__builtin_amdgcn_ballot_w64(t.wt[i] != 0.f)) m |= 1u << (sp * NCORN + i);
+          if (kMasked && __builtin_amdgcn_ballot_w64(t.wt[i] != 0.f)) m |= 1u << (sp * NCORN + i);
         }
       }
-      if ((tid & 63) == 0) TapMask[kl][half][(tid >> 6) & 1] = m;
+      if (kMasked && (tid & 63) == 0) TapMask[kl][half][(tid >> 6) & 1] = m;
     }
     __syncthreads();
 
