@@ -146,7 +146,8 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
     const float *__restrict__ wp, const TD *__restrict__ bias, TD *__restrict__ y, int G,
     int O, int Opad, int Gpad, int SH, int SW, int OH, int OW, int K, int weighted, int wrap,
     int tiles_x, int tiles_per_img, int tw_shift, const int *__restrict__ gate, int run_if_zero,
-    const float *__restrict__ addend, const int *__restrict__ pair_mask, int run_if_leading) {
+    const float *__restrict__ addend, const int *__restrict__ pair_mask, int run_if_leading,
+    int packed_map) {
   constexpr int NE = NP * NCORN;         // (offset, weight) pairs per pixel and tap
   static_assert(NA >= 1 && NA <= NE, "NA counts leading pairs");
   constexpr bool kMasked = NA == NE;
@@ -311,8 +312,15 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
       for (int sp = 0; sp < kPoints; sp++) {
         const int64_t e = (n_g * K + k0 + kl) * NP + sp;
         PairTap<NCORN> t;
-        resolve_pairs<NCORN, sizeof(TD)>(map[e * 2], map[e * 2 + 1], SH, SW, wrap != 0,
-                                         live ? (weighted ? iw[e] : 1.f) : 0.f, t);
+        if (NCORN == 1 && packed_map) {
+          // pre-resolved entry (a transposed map): element index of the source, weight
+          const float2 q = reinterpret_cast<const float2 *>(map)[e];
+          t.off[0] = __builtin_bit_cast(unsigned, q.x) * (unsigned)sizeof(TD);
+          t.wt[0] = live ? q.y : 0.f;
+        } else {
+          resolve_pairs<NCORN, sizeof(TD)>(map[e * 2], map[e * 2 + 1], SH, SW, wrap != 0,
+                                           live ? (weighted ? iw[e] : 1.f) : 0.f, t);
+        }
 #pragma unroll
         for (int i = 0; i < NCORN; i++) {
           if (sp * NCORN + i >= NA) continue;
@@ -1217,7 +1225,7 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
                           int64_t SH, int64_t SW, int64_t OH, int64_t OW, int64_t K, int64_t P,
                           int interp, const int *gate, int run_if_zero, hipStream_t s,
                           const float *addend = nullptr, bool staged = false,
-                          const int *pair_mask = nullptr) {
+                          const int *pair_mask = nullptr, bool packed_map = false) {
   const int Opad = (int)round_up(O, kOT), Gpad = (int)round_up(G, kGC);
   const bool cl = stage != nullptr && use_channel_last(SH, interp) &&
                   SH * SW * Gpad * (int64_t)sizeof(TD) <= 0xffffffffLL;
@@ -1244,7 +1252,7 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
                      dim3(kThreads), 0, s, src, map, iw, wp, bias, y, (int)G, (int)O, Opad,      \
                      Gpad, (int)SH, (int)SW, (int)OH, (int)OW, (int)K, m.weighted, m.wrap,       \
                      t.tiles_x, t.tiles_per_img, t.tw_shift, gate, run_if_zero, addend, MASK,    \
-                     LEAD)
+                     LEAD, packed_map ? 1 : 0)
 #define MCX_LAUNCH_CL(NCORN, NP, OG, CL)                                      \
   if constexpr (NCORN * NP == 4) {                                            \
     if (pair_mask) {                                                          \
@@ -1453,7 +1461,7 @@ namespace {
 // resolution-preserving maps such as the latitude-distorted kernels), the product-
 // scatter equals a weighted, nearest-neighbour gather-product over the transposed
 // map, which needs no atomics at all and reuses the forward kernel.  This kernel
-// builds that map: tmap[p][k][slot] = (x, y) of source pixel n, tiw = corner weight;
+// builds that map: tmap[p][k][slot] = (index of source pixel n as bits, corner weight);
 // a slot counter per (p, k) hands out slots and an overflow flag selects the scatter
 // kernel instead (both kernels are always enqueued; the flag gates them on the device).
 constexpr int kTransSlots = 4;
@@ -1486,8 +1494,7 @@ __global__ void slot_mask_kernel(const int *__restrict__ cnt, int64_t cells,
 template <int NCORN>
 __global__ void build_transposed_map_kernel(const float *__restrict__ map,
                                             const float *__restrict__ iw, int *__restrict__ cnt,
-                                            float *__restrict__ tmap, float *__restrict__ tiw,
-                                            int *__restrict__ overflow,
+                                            float2 *__restrict__ tmap, int *__restrict__ overflow,
                                             OverflowEntry *__restrict__ ovf, int ovf_cap, int np,
                                             int weighted, int wrap, int DH, int DW, int MW, int K,
                                             int64_t total) {
@@ -1495,7 +1502,7 @@ __global__ void build_transposed_map_kernel(const float *__restrict__ map,
   if (e >= total) return;
   const int k = (int)(e % K);
   const int64_t n = e / K;
-  const float nx = (float)(n % MW), ny = (float)(n / MW);
+  const float nbits = __builtin_bit_cast(float, (int)n);
   for (int sp = 0; sp < np; sp++) {
     const int64_t m = e * np + sp;
     CoordTap<NCORN> t;
@@ -1507,9 +1514,7 @@ __global__ void build_transposed_map_kernel(const float *__restrict__ map,
       const int64_t cell = ((int64_t)t.yy[c] * DW + t.xx[c]) * K + k;
       const int slot = atomicAdd(&cnt[cell], 1);
       if (slot < kTransSlots) {
-        tmap[(cell * kTransSlots + slot) * 2] = nx;
-        tmap[(cell * kTransSlots + slot) * 2 + 1] = ny;
-        tiw[cell * kTransSlots + slot] = t.wt[c];
+        tmap[cell * kTransSlots + slot] = make_float2(nbits, t.wt[c]);
       } else {
         // overflow[0]: flag, overflow[1]: length of the overflow list
         const int pos = ovf_cap > 0 ? atomicAdd(&overflow[1], 1) : 0;
@@ -1606,7 +1611,7 @@ __global__ void convert_planes_kernel(const float *__restrict__ src, TD *__restr
 }
 
 struct ScatterScratch {
-  size_t wq, wpt, cnt, tmap, tiw, acc32, ovf, stage, total;  // byte offsets
+  size_t wq, wpt, cnt, tmap, acc32, ovf, stage, total;  // byte offsets
   int64_t ovf_cap;  // entries of the overflow list (0: none)
   bool transposed_path;
 };
@@ -1629,16 +1634,14 @@ ScatterScratch scatter_scratch(int64_t B, int64_t S, int64_t D, int64_t K, int64
     const int64_t overflow_img = sc.transposed_path ? B * DH * DW * round_up(D, kOT) : 0;
     off += align256((size_t)std::max(scatter_img, overflow_img) * 4);
   }
-  sc.wpt = sc.cnt = sc.tmap = sc.tiw = off;
+  sc.wpt = sc.cnt = sc.tmap = off;
   if (sc.transposed_path) {
     sc.wpt = off;
     off += align256((size_t)(K * round_up(S, kGC) * round_up(D, kOT)) * 4);
-    sc.cnt = off;  // counters, the overflow flag and list length; cleared with tmap and tiw
+    sc.cnt = off;  // counters, the overflow flag and list length; cleared with tmap
     off += align256((size_t)(cells + 4) * 4);
-    sc.tmap = off;
+    sc.tmap = off;  // [cell][slot] (source pixel index as bits, weight)
     off += align256((size_t)cells * kTransSlots * 2 * 4);
-    sc.tiw = off;
-    off += align256((size_t)cells * kTransSlots * 4);
   }
   // Overflow list: room for half of the contributions a bilinear map can make.
   sc.ovf = sc.stage = off;
@@ -1677,7 +1680,7 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
   if (sc.transposed_path) {
     // build the transposed map, then try the atomic-free gather form first
     int *cnt = (int *)(base + sc.cnt);
-    float *tmap = (float *)(base + sc.tmap), *tiw = (float *)(base + sc.tiw);
+    float2 *tmap = (float2 *)(base + sc.tmap);
     float *wpt = (float *)(base + sc.wpt);
     const int64_t cells = DH * DW * K;
     int *flag = cnt + cells;
@@ -1689,11 +1692,11 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
     const unsigned blocks = (unsigned)((entries + 255) / 256);
     if (m.mode == kInterpNearest)
       hipLaunchKernelGGL(build_transposed_map_kernel<1>, dim3(blocks), dim3(256), 0, s, map, iw,
-                         cnt, tmap, tiw, flag, ovf, (int)sc.ovf_cap, m.np, m.weighted, m.wrap,
+                         cnt, tmap, flag, ovf, (int)sc.ovf_cap, m.np, m.weighted, m.wrap,
                          (int)DH, (int)DW, (int)MW, (int)K, entries);
     else
       hipLaunchKernelGGL(build_transposed_map_kernel<4>, dim3(blocks), dim3(256), 0, s, map, iw,
-                         cnt, tmap, tiw, flag, ovf, (int)sc.ovf_cap, m.np, m.weighted, m.wrap,
+                         cnt, tmap, flag, ovf, (int)sc.ovf_cap, m.np, m.weighted, m.wrap,
                          (int)DH, (int)DW, (int)MW, (int)K, entries);
     MCX_HIP_CHECK_LAUNCH();
     // flag[2]: mask of the slots in use anywhere (bit i: some cell holds more than i entries)
@@ -1724,9 +1727,9 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
                        flag, (int)sc.ovf_cap, (int)S, (int)Spad16, (int)D, (int)round_up(D, kOT),
                        MH * MW, DH * DW);
     MCX_HIP_CHECK_LAUNCH();
-    if (int rc = launch_gather_product<TD>(src, tmap, tiw, wpt, bias, dst, stage, B, S, D, MH, MW,
-                                           DH, DW, K, kTransSlots, kInterpNearest, gate, 1, s, img,
-                                           cl, flag + 2))
+    if (int rc = launch_gather_product<TD>(src, (const float *)tmap, nullptr, wpt, bias, dst,
+                                           stage, B, S, D, MH, MW, DH, DW, K, kTransSlots,
+                                           kInterpNearest, gate, 1, s, img, cl, flag + 2, true))
       return rc;
   }
 
