@@ -138,8 +138,8 @@ struct OperandTiles<bf16_t> {  // bf16: 16-byte groups of 8 channels, [kg][pixel
 // the general form, which skips the pairs a tile's mask shows to be zero across the tile.
 // NA == 2 (four-pair taps) is the branch-free form for maps that use nothing but the first
 // two pairs anywhere (bilinear with integral rows, transposed maps with at most two
-// contributions per cell): both forms are launched and `pair_mask` (bit i: pair i in use
-// somewhere in the map) lets exactly one of them run.
+// contributions per cell): both forms are launched and `pair_mask` (at least 4 iff a pair
+// beyond the first two is in use somewhere in the map) lets exactly one of them run.
 template <typename TD, int NCORN, int NP, int OG, bool CL, int NA>
 __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma_kernel(
     const TD *__restrict__ src, const float *__restrict__ map, const float *__restrict__ iw,
@@ -421,9 +421,17 @@ constexpr int kWgCB = 2;            // 16-channel blocks of gathered channels pe
 constexpr int kWgKT = 9;            // taps per pass (accumulators in registers)
 constexpr int kLdPx = kTilePx + 4;  // LDS row stride (floats)
 
-// mask[0] |= bit (point * NCORN + corner) for every pair of the map with a nonzero weight.
-// Grid-stride over the samples and one global access per workgroup: every access goes to
-// the same address and is served one at a time.
+// The consumers of a pair mask only ask whether a pair beyond the first two is in use
+// (mask >= 4).  Accesses to the one address are served one at a time (about 12 ns each), so a
+// workgroup reports only when it has such a pair and nobody has reported one yet.
+__device__ inline void report_pairs_beyond_two(int *mask, unsigned block_mask) {
+  if (threadIdx.x == 0 && block_mask >= 4u &&
+      (unsigned)__hip_atomic_load(mask, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < 4u)
+    atomicOr(mask, (int)block_mask);
+}
+
+// mask[0] >= 4 iff some sample of the map has a nonzero weight in a pair (point * NCORN +
+// corner) beyond the first two.  Grid-stride over the samples.
 template <int NCORN>
 __global__ void map_pair_mask_kernel(const float *__restrict__ map, const float *__restrict__ iw,
                                      int *__restrict__ mask, int np, int weighted, int wrap,
@@ -447,7 +455,7 @@ __global__ void map_pair_mask_kernel(const float *__restrict__ map, const float 
   for (int d = 32; d > 0; d >>= 1) m |= __shfl_xor(m, d);
   if ((threadIdx.x & 63) == 0 && m) atomicOr(&block_mask, m);
   __syncthreads();
-  if (threadIdx.x == 0 && block_mask) atomicOr(mask, (int)block_mask);
+  report_pairs_beyond_two(mask, block_mask);
 }
 
 // CL: `gath` is a channel-last copy [B][GH*GW][Gpad] of the gathered operand (see the
@@ -785,23 +793,34 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
   }
 }
 
+// out[e] = sum over ranges of part[r][e].  64 x 4 threads: four quarters of the ranges are
+// summed side by side (eight loads in flight each) and combined in a fixed order, so the
+// result does not depend on scheduling.
 template <typename TD>
-__global__ void reduce_partials_kernel(const float *__restrict__ part, TD *__restrict__ out,
-                                       int ranges, int64_t n) {
-  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (e >= n) return;
-  // eight loads in flight per thread; the order of the additions is fixed
+__global__ __launch_bounds__(256) void reduce_partials_kernel(const float *__restrict__ part,
+                                                              TD *__restrict__ out, int ranges,
+                                                              int64_t n) {
+  __shared__ float quarter[4][64];
+  const int64_t e = (int64_t)blockIdx.x * 64 + threadIdx.x;
+  const int per = (ranges + 3) / 4;
+  const int r0 = min((int)threadIdx.y * per, ranges), r1 = min(r0 + per, ranges);
   float s = 0.f;
-  int r = 0;
-  for (; r + 8 <= ranges; r += 8) {
-    float t[8];
+  if (e < n) {
+    int r = r0;
+    for (; r + 8 <= r1; r += 8) {
+      float t[8];
 #pragma unroll
-    for (int u = 0; u < 8; u++) t[u] = part[(int64_t)(r + u) * n + e];
+      for (int u = 0; u < 8; u++) t[u] = part[(int64_t)(r + u) * n + e];
 #pragma unroll
-    for (int u = 0; u < 8; u++) s += t[u];
+      for (int u = 0; u < 8; u++) s += t[u];
+    }
+    for (; r < r1; r++) s += part[(int64_t)r * n + e];
   }
-  for (; r < ranges; r++) s += part[(int64_t)r * n + e];
-  out[e] = from_f32<TD>(s);
+  quarter[threadIdx.y][threadIdx.x] = s;
+  __syncthreads();
+  if (threadIdx.y == 0 && e < n)
+    out[e] = from_f32<TD>(((quarter[0][threadIdx.x] + quarter[1][threadIdx.x]) +
+                           quarter[2][threadIdx.x]) + quarter[3][threadIdx.x]);
 }
 
 // ---------------------------------------------------------------------------------
@@ -1312,11 +1331,11 @@ int launch_pack_weights(const TD *w, float *wp, int64_t O, int64_t G, int64_t K,
   return 0;
 }
 
-// mask[0] = OR over the map's samples of the bits of their nonzero pairs.
+// mask[0] >= 4 iff the map uses a pair beyond the first two of a tap.
 int launch_pair_mask(const float *map, const float *iw, int *mask, const ModeArgs &m, int64_t GH,
                      int64_t GW, int64_t samples, hipStream_t s) {
   if (int rc = fill_f32((float *)mask, 1, 0.f, s)) return rc;
-  const dim3 mg((unsigned)std::min<int64_t>((samples + 255) / 256, 512));
+  const dim3 mg((unsigned)std::min<int64_t>((samples + 255) / 256, 2048));
   if (m.mode == kInterpNearest)
     hipLaunchKernelGGL(map_pair_mask_kernel<1>, mg, dim3(256), 0, s, map, iw, mask, m.np,
                        m.weighted, m.wrap, (int)GH, (int)GW, samples);
@@ -1441,12 +1460,12 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
 #undef MCX_LAUNCH_CL
   MCX_HIP_CHECK_LAUNCH();
   const int64_t n = A * G * K;
-  hipLaunchKernelGGL(reduce_partials_kernel<TD>, dim3((unsigned)((n + 63) / 64)), dim3(64), 0, s,
-                     part, gw, ranges, n);
+  hipLaunchKernelGGL(reduce_partials_kernel<TD>, dim3((unsigned)((n + 63) / 64)), dim3(64, 4), 0,
+                     s, part, gw, ranges, n);
   MCX_HIP_CHECK_LAUNCH();
   if (plain_sum) {
-    hipLaunchKernelGGL(reduce_partials_kernel<TD>, dim3((unsigned)((A + 63) / 64)), dim3(64), 0, s,
-                       sum_part, plain_sum, ranges, A);
+    hipLaunchKernelGGL(reduce_partials_kernel<TD>, dim3((unsigned)((A + 63) / 64)), dim3(64, 4), 0,
+                       s, sum_part, plain_sum, ranges, A);
     MCX_HIP_CHECK_LAUNCH();
   }
   return 0;
@@ -1475,7 +1494,7 @@ struct OverflowEntry {
   float wt;
 };
 
-// mask[0] |= bits [0, min(cnt, kTransSlots)) for every cell: the slots in use.
+// mask[0] >= 4 iff some cell holds more than two entries (bits [0, min(cnt, kTransSlots))).
 __global__ void slot_mask_kernel(const int *__restrict__ cnt, int64_t cells,
                                  int *__restrict__ mask) {
   __shared__ unsigned block_mask;
@@ -1488,7 +1507,7 @@ __global__ void slot_mask_kernel(const int *__restrict__ cnt, int64_t cells,
   for (int d = 32; d > 0; d >>= 1) m |= __shfl_xor(m, d);
   if ((threadIdx.x & 63) == 0 && m) atomicOr(&block_mask, m);
   __syncthreads();
-  if (threadIdx.x == 0 && block_mask) atomicOr(mask, (int)block_mask);
+  report_pairs_beyond_two(mask, block_mask);
 }
 
 template <int NCORN>
@@ -1700,7 +1719,7 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
                          (int)DH, (int)DW, (int)MW, (int)K, entries);
     MCX_HIP_CHECK_LAUNCH();
     // flag[2]: mask of the slots in use anywhere (bit i: some cell holds more than i entries)
-    hipLaunchKernelGGL(slot_mask_kernel, dim3((unsigned)std::min<int64_t>((cells + 255) / 256, 512)),
+    hipLaunchKernelGGL(slot_mask_kernel, dim3((unsigned)std::min<int64_t>((cells + 255) / 256, 2048)),
                        dim3(256), 0, s, cnt, cells, flag + 2);
     MCX_HIP_CHECK_LAUNCH();
     if (int rc = launch_pack_weights<TD>(w, wpt, D, S, K, 1, s)) return rc;
