@@ -51,7 +51,9 @@ __device__ inline int xcd_contiguous_tile(int wg, int total) {
 // `transposed` reads W[g][o][k] instead (weights stored source-channel major).
 template <typename TD>
 __global__ void pack_weights_kernel(const TD *__restrict__ w, float *__restrict__ wp, int O,
-                                    int G, int K, int Opad, int Gpad, int transposed) {
+                                    int G, int K, int Opad, int Gpad, int transposed,
+                                    int *__restrict__ clear) {
+  if (clear && blockIdx.x == 0 && threadIdx.x == 0) *clear = 0;  // a flag word of the caller
   const int64_t total = (int64_t)K * Gpad * Opad;
   for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total;
        e += (int64_t)gridDim.x * blockDim.x) {
@@ -75,7 +77,8 @@ typedef float floatx2 __attribute__((ext_vector_type(2)));
 template <typename TD>
 __global__ void pack_weights_bf16_kernel(const TD *__restrict__ w, uint16_t *__restrict__ wb,
                                          int O, int G, int K, int Opad, int Gpad,
-                                         int transposed) {
+                                         int transposed, int *__restrict__ clear) {
+  if (clear && blockIdx.x == 0 && threadIdx.x == 0) *clear = 0;  // a flag word of the caller
   const int chunks = Gpad / kGC;
   const int64_t total = (int64_t)K * Gpad * Opad;
   for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total;
@@ -793,15 +796,23 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
   }
 }
 
-// out[e] = sum over ranges of part[r][e].  64 x 4 threads: four quarters of the ranges are
-// summed side by side (eight loads in flight each) and combined in a fixed order, so the
-// result does not depend on scheduling.
+// out[e] = sum over ranges of part[r][e], for two independent jobs in one launch (the second
+// may be empty).  64 x 4 threads: four quarters of the ranges are summed side by side (eight
+// loads in flight each) and combined in a fixed order, so the result does not depend on
+// scheduling.
 template <typename TD>
-__global__ __launch_bounds__(256) void reduce_partials_kernel(const float *__restrict__ part,
-                                                              TD *__restrict__ out, int ranges,
-                                                              int64_t n) {
+__global__ __launch_bounds__(256) void reduce_partials_kernel(
+    const float *__restrict__ part, TD *__restrict__ out, int64_t n,
+    const float *__restrict__ part2, TD *__restrict__ out2, int64_t n2, int ranges) {
   __shared__ float quarter[4][64];
-  const int64_t e = (int64_t)blockIdx.x * 64 + threadIdx.x;
+  const int blocks1 = (int)((n + 63) / 64);
+  int64_t e = (int64_t)blockIdx.x * 64 + threadIdx.x;
+  if ((int)blockIdx.x >= blocks1) {  // second job
+    e -= (int64_t)blocks1 * 64;
+    part = part2;
+    out = out2;
+    n = n2;
+  }
   const int per = (ranges + 3) / 4;
   const int r0 = min((int)threadIdx.y * per, ranges), r1 = min(r0 + per, ranges);
   float s = 0.f;
@@ -1316,25 +1327,27 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
 
 template <typename TD>
 int launch_pack_weights(const TD *w, float *wp, int64_t O, int64_t G, int64_t K, int transposed,
-                        hipStream_t s) {
+                        hipStream_t s, int *clear = nullptr) {
   const int Opad = (int)round_up(O, kOT), Gpad = (int)round_up(G, kGC);
   const int64_t packed = (int64_t)K * Gpad * Opad;
   const dim3 grid((unsigned)std::min<int64_t>((packed + 255) / 256, 4096));
   if (sizeof(TD) == 2)  // bf16 storage: bf16 MFMA operand layout (same scratch, half the bytes)
     hipLaunchKernelGGL(pack_weights_bf16_kernel<TD>, grid, dim3(256), 0, s, w,
                        reinterpret_cast<uint16_t *>(wp), (int)O, (int)G, (int)K, Opad, Gpad,
-                       transposed);
+                       transposed, clear);
   else
     hipLaunchKernelGGL(pack_weights_kernel<TD>, grid, dim3(256), 0, s, w, wp, (int)O, (int)G,
-                       (int)K, Opad, Gpad, transposed);
+                       (int)K, Opad, Gpad, transposed, clear);
   MCX_HIP_CHECK_LAUNCH();
   return 0;
 }
 
 // mask[0] >= 4 iff the map uses a pair beyond the first two of a tap.
+// `cleared`: an earlier kernel on the stream has zeroed the mask.
 int launch_pair_mask(const float *map, const float *iw, int *mask, const ModeArgs &m, int64_t GH,
-                     int64_t GW, int64_t samples, hipStream_t s) {
-  if (int rc = fill_f32((float *)mask, 1, 0.f, s)) return rc;
+                     int64_t GW, int64_t samples, hipStream_t s, bool cleared = false) {
+  if (!cleared)
+    if (int rc = fill_f32((float *)mask, 1, 0.f, s)) return rc;
   const dim3 mg((unsigned)std::min<int64_t>((samples + 255) / 256, 2048));
   if (m.mode == kInterpNearest)
     hipLaunchKernelGGL(map_pair_mask_kernel<1>, mg, dim3(256), 0, s, map, iw, mask, m.np,
@@ -1369,11 +1382,11 @@ int mfma_gather_product(const TD *src, const float *map, const float *iw, const 
   int *pair_mask = reinterpret_cast<int *>(
       (char *)scratch + align256((size_t)(K * round_up(G, kGC) * round_up(O, kOT)) * 4));
   TD *stage = SH == 1 ? reinterpret_cast<TD *>((char *)pair_mask + 256) : nullptr;
-  if (int rc = launch_pack_weights<TD>(w, wp, O, G, K, 0, s)) return rc;
+  if (int rc = launch_pack_weights<TD>(w, wp, O, G, K, 0, s, pair_mask)) return rc;
   const ModeArgs m = mode_args(interp, P);
   const bool four_pairs = m.np * (m.mode == kInterpNearest ? 1 : 4) == 4;
   if (four_pairs)
-    if (int rc = launch_pair_mask(map, iw, pair_mask, m, SH, SW, OH * OW * K, s)) return rc;
+    if (int rc = launch_pair_mask(map, iw, pair_mask, m, SH, SW, OH * OW * K, s, true)) return rc;
   return launch_gather_product<TD>(src, map, iw, wp, bias, y, stage, B, G, O, SH, SW, OH, OW, K,
                                    P, interp, nullptr, 0, s, nullptr, false,
                                    four_pairs ? pair_mask : nullptr);
@@ -1460,14 +1473,10 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
 #undef MCX_LAUNCH_CL
   MCX_HIP_CHECK_LAUNCH();
   const int64_t n = A * G * K;
-  hipLaunchKernelGGL(reduce_partials_kernel<TD>, dim3((unsigned)((n + 63) / 64)), dim3(64, 4), 0,
-                     s, part, gw, ranges, n);
+  const int64_t n2 = plain_sum ? A : 0;
+  hipLaunchKernelGGL(reduce_partials_kernel<TD>, dim3((unsigned)((n + 63) / 64 + (n2 + 63) / 64)),
+                     dim3(64, 4), 0, s, part, gw, n, sum_part, plain_sum, n2, ranges);
   MCX_HIP_CHECK_LAUNCH();
-  if (plain_sum) {
-    hipLaunchKernelGGL(reduce_partials_kernel<TD>, dim3((unsigned)((A + 63) / 64)), dim3(64, 4), 0,
-                       s, sum_part, plain_sum, ranges, A);
-    MCX_HIP_CHECK_LAUNCH();
-  }
   return 0;
 }
 
@@ -1493,22 +1502,6 @@ struct OverflowEntry {
   int p, n, k;
   float wt;
 };
-
-// mask[0] >= 4 iff some cell holds more than two entries (bits [0, min(cnt, kTransSlots))).
-__global__ void slot_mask_kernel(const int *__restrict__ cnt, int64_t cells,
-                                 int *__restrict__ mask) {
-  __shared__ unsigned block_mask;
-  if (threadIdx.x == 0) block_mask = 0;
-  __syncthreads();
-  unsigned m = 0;
-  for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < cells;
-       e += (int64_t)gridDim.x * blockDim.x)
-    m |= (1u << min(cnt[e], kTransSlots)) - 1u;
-  for (int d = 32; d > 0; d >>= 1) m |= __shfl_xor(m, d);
-  if ((threadIdx.x & 63) == 0 && m) atomicOr(&block_mask, m);
-  __syncthreads();
-  report_pairs_beyond_two(mask, block_mask);
-}
 
 template <int NCORN>
 __global__ void build_transposed_map_kernel(const float *__restrict__ map,
@@ -1598,10 +1591,24 @@ __global__ __launch_bounds__(64) void overflow_scatter_kernel(
   }
 }
 
-// Clears the fp32 image the overflow list of a non-fp32 product is accumulated into; only
-// when the list is in use and not empty.
-__global__ void clear_overflow_image_kernel(float *__restrict__ img, int64_t total,
-                                            const int *__restrict__ overflow) {
+// Two jobs that follow the building of a transposed map, in one launch.  (1) mask[0] >= 4
+// iff some cell holds more than two entries (bits [0, min(cnt, kTransSlots))).  (2) Clear
+// the fp32 image the overflow list is accumulated into, only when the list is in use and
+// not empty.
+__global__ void after_transposed_map_kernel(const int *__restrict__ cnt, int64_t cells,
+                                            int *__restrict__ mask, float *__restrict__ img,
+                                            int64_t total, const int *__restrict__ overflow) {
+  __shared__ unsigned block_mask;
+  if (threadIdx.x == 0) block_mask = 0;
+  __syncthreads();
+  unsigned m = 0;
+  for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < cells;
+       e += (int64_t)gridDim.x * blockDim.x)
+    m |= (1u << min(cnt[e], kTransSlots)) - 1u;
+  for (int d = 32; d > 0; d >>= 1) m |= __shfl_xor(m, d);
+  if ((threadIdx.x & 63) == 0 && m) atomicOr(&block_mask, m);
+  __syncthreads();
+  report_pairs_beyond_two(mask, block_mask);
   if (overflow[0] != 0 || overflow[1] <= 0) return;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
        i += (int64_t)gridDim.x * blockDim.x)
@@ -1718,10 +1725,6 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
                          cnt, tmap, flag, ovf, (int)sc.ovf_cap, m.np, m.weighted, m.wrap,
                          (int)DH, (int)DW, (int)MW, (int)K, entries);
     MCX_HIP_CHECK_LAUNCH();
-    // flag[2]: mask of the slots in use anywhere (bit i: some cell holds more than i entries)
-    hipLaunchKernelGGL(slot_mask_kernel, dim3((unsigned)std::min<int64_t>((cells + 255) / 256, 2048)),
-                       dim3(256), 0, s, cnt, cells, flag + 2);
-    MCX_HIP_CHECK_LAUNCH();
     if (int rc = launch_pack_weights<TD>(w, wpt, D, S, K, 1, s)) return rc;
     // What did not fit the four slots of its cell is accumulated with float atomics into a
     // channel-last fp32 image (cleared only when there is anything to add), which the
@@ -1731,9 +1734,11 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
                     MH * MW * Spad16 * (int64_t)sizeof(TD) <= 0xffffffffLL;
     float *img = (float *)(base + sc.acc32);
     const int64_t total_img = B * DH * DW * round_up(D, kOT);
-    hipLaunchKernelGGL(clear_overflow_image_kernel,
-                       dim3((unsigned)std::min<int64_t>((total_img + 1023) / 1024, 4096)),
-                       dim3(256), 0, s, img, total_img, flag);
+    // flag[2]: at least 4 iff some cell holds more than two entries
+    hipLaunchKernelGGL(after_transposed_map_kernel,
+                       dim3((unsigned)std::min<int64_t>(
+                           std::max((total_img + 1023) / 1024, (cells + 255) / 256), 4096)),
+                       dim3(256), 0, s, cnt, cells, flag + 2, img, total_img, flag);
     MCX_HIP_CHECK_LAUNCH();
     if (cl) {  // the overflow pass reads the channel-last copy before the gather would make it
       dim3 tg((unsigned)((MH * MW + 63) / 64), (unsigned)((Spad16 + 63) / 64), (unsigned)B);
