@@ -177,6 +177,7 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
   const int o0 = blockIdx.y * (kOT * OG);
   const int N = OH * OW;
   const int64_t plane = (int64_t)SH * SW;
+  const int64_t plane_bytes = plane * (int64_t)sizeof(TD);
 
   // gather role: pixel p of the tile, channels [half*8, half*8+8) of each chunk
   const int p = tid & (kTilePx - 1);
@@ -213,6 +214,13 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
     const int g0 = c * kGC + half * 8;
     if constexpr (CL) {
       pl[0] = src_b + g0;  // the 8 channels are contiguous; offsets select the pixel row
+    } else if (g0 + 8 <= G) {  // all eight planes exist: one product, then additions
+      const char *q = reinterpret_cast<const char *>(src_b) + (int64_t)g0 * plane_bytes;
+#pragma unroll
+      for (int ch = 0; ch < 8; ch++) {
+        pl[ch] = reinterpret_cast<const TD *>(q);
+        q += plane_bytes;
+      }
     } else {
 #pragma unroll
       for (int ch = 0; ch < 8; ch++)  // padded channels read a valid plane, weights are 0
