@@ -34,13 +34,13 @@ GEMM_FLOP = 2.0 * B * H * W * CO * CI * K  # one of the three products
 # count); profiles/conv_fwd_bwd_headline_hbm_traffic.txt holds the runs.  Counters cannot be read
 # from inside the process, so the figures are the recorded ones; other workloads report null.
 MEASURED_TRAFFIC_BYTES = {
-    "conv_forward": 855.3e6 + 268.4e6,
-    "conv_backward_input": 2048.5e6 + 268.4e6,
-    "conv_backward_weight": 2026.3e6 + 91.3e6,
+    "conv_forward": 783.9e6 + 268.4e6,
+    "conv_backward_input": 1411.8e6 + 268.4e6,
+    "conv_backward_weight": 1531.4e6 + 92.5e6,
 }
 KERNEL_OF = {
-    "conv_forward": "gather_product_mfma_kernel<float,4,1,1,false>",
-    "conv_backward_input": "gather_product_mfma_kernel<float,1,4,1,false>",
+    "conv_forward": "gather_product_mfma_kernel<float,4,1,1,false,2>",
+    "conv_backward_input": "gather_product_mfma_kernel<float,1,4,1,false,2>",
     "conv_backward_weight": "weight_grad_mfma_kernel<float,4,1,false,2>",
 }
 
