@@ -150,7 +150,7 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
     int O, int Opad, int Gpad, int SH, int SW, int OH, int OW, int K, int weighted, int wrap,
     int tiles_x, int tiles_per_img, int tw_shift, const int *__restrict__ gate, int run_if_zero,
     const float *__restrict__ addend, const int *__restrict__ pair_mask, int run_if_leading,
-    int packed_map) {
+    int packed_map, int accumulate) {
   constexpr int NE = NP * NCORN;         // (offset, weight) pairs per pixel and tap
   static_assert(NA >= 1 && NA <= NE, "NA counts leading pairs");
   constexpr bool kMasked = NA == NE;
@@ -166,6 +166,9 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
   __shared__ unsigned TapMask[TG][2][2];
   if (gate && ((*gate == 0) != (run_if_zero != 0))) return;  // device-side path selection
   if (pair_mask && (((unsigned)*pair_mask < (1u << 2)) != (run_if_leading != 0))) return;
+  // a pass that adds onto y (the second level of a transposed map) has nothing to do when
+  // no pair of its map is in use
+  if (accumulate && pair_mask && *pair_mask == 0) return;
 
   const int tid = threadIdx.x;
   const int tile = xcd_contiguous_tile(blockIdx.x, gridDim.x);
@@ -407,9 +410,10 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
 #pragma unroll
       for (int i = 0; i < 16; i++) {
         const int o = o0 + 32 * m + (i >> 2) * 8 + lhi * 4 + (i & 3);
-        if (o < O)
-          yb[(int64_t)o * N] = from_f32<TD>(acc[m][i] + (bias ? to_f32(bias[o]) : 0.f) +
-                                            (ab ? ab[o] : 0.f));
+        if (o < O) {
+          const float start = accumulate ? to_f32(yb[(int64_t)o * N]) : (bias ? to_f32(bias[o]) : 0.f);
+          yb[(int64_t)o * N] = from_f32<TD>(acc[m][i] + start + (ab ? ab[o] : 0.f));
+        }
       }
   }
 }
@@ -1263,7 +1267,8 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
                           int64_t SH, int64_t SW, int64_t OH, int64_t OW, int64_t K, int64_t P,
                           int interp, const int *gate, int run_if_zero, hipStream_t s,
                           const float *addend = nullptr, bool staged = false,
-                          const int *pair_mask = nullptr, bool packed_map = false) {
+                          const int *pair_mask = nullptr, bool packed_map = false,
+                          bool accumulate = false) {
   const int Opad = (int)round_up(O, kOT), Gpad = (int)round_up(G, kGC);
   const bool cl = stage != nullptr && use_channel_last(SH, interp) &&
                   SH * SW * Gpad * (int64_t)sizeof(TD) <= 0xffffffffLL;
@@ -1290,7 +1295,7 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
                      dim3(kThreads), 0, s, src, map, iw, wp, bias, y, (int)G, (int)O, Opad,      \
                      Gpad, (int)SH, (int)SW, (int)OH, (int)OW, (int)K, m.weighted, m.wrap,       \
                      t.tiles_x, t.tiles_per_img, t.tw_shift, gate, run_if_zero, addend, MASK,    \
-                     LEAD, packed_map ? 1 : 0)
+                     LEAD, packed_map ? 1 : 0, accumulate ? 1 : 0)
 #define MCX_LAUNCH_CL(NCORN, NP, OG, CL)                                      \
   if constexpr (NCORN * NP == 4) {                                            \
     if (pair_mask) {                                                          \
@@ -1514,7 +1519,8 @@ struct OverflowEntry {
 template <int NCORN>
 __global__ void build_transposed_map_kernel(const float *__restrict__ map,
                                             const float *__restrict__ iw, int *__restrict__ cnt,
-                                            float2 *__restrict__ tmap, int *__restrict__ overflow,
+                                            float2 *__restrict__ tmap, float2 *__restrict__ tmap2,
+                                            int *__restrict__ overflow,
                                             OverflowEntry *__restrict__ ovf, int ovf_cap, int np,
                                             int weighted, int wrap, int DH, int DW, int MW, int K,
                                             int64_t total) {
@@ -1535,6 +1541,8 @@ __global__ void build_transposed_map_kernel(const float *__restrict__ map,
       const int slot = atomicAdd(&cnt[cell], 1);
       if (slot < kTransSlots) {
         tmap[cell * kTransSlots + slot] = make_float2(nbits, t.wt[c]);
+      } else if (tmap2 && slot < 2 * kTransSlots) {  // second level (a second gather pass)
+        tmap2[cell * kTransSlots + slot - kTransSlots] = make_float2(nbits, t.wt[c]);
       } else {
         // overflow[0]: flag, overflow[1]: length of the overflow list
         const int pos = ovf_cap > 0 ? atomicAdd(&overflow[1], 1) : 0;
@@ -1600,23 +1608,31 @@ __global__ __launch_bounds__(64) void overflow_scatter_kernel(
 }
 
 // Two jobs that follow the building of a transposed map, in one launch.  (1) mask[0] >= 4
-// iff some cell holds more than two entries (bits [0, min(cnt, kTransSlots))).  (2) Clear
+// iff some cell holds more than two entries (bits [0, min(cnt, kTransSlots))); with a
+// second level, mask[1] holds the bits of the second-level slots in use (0: none).  (2) Clear
 // the fp32 image the overflow list is accumulated into, only when the list is in use and
 // not empty.
 __global__ void after_transposed_map_kernel(const int *__restrict__ cnt, int64_t cells,
-                                            int *__restrict__ mask, float *__restrict__ img,
-                                            int64_t total, const int *__restrict__ overflow) {
+                                            int *__restrict__ mask, int two_level,
+                                            float *__restrict__ img, int64_t total,
+                                            const int *__restrict__ overflow) {
   __shared__ unsigned block_mask;
   if (threadIdx.x == 0) block_mask = 0;
   __syncthreads();
   unsigned m = 0;
   for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < cells;
        e += (int64_t)gridDim.x * blockDim.x)
-    m |= (1u << min(cnt[e], kTransSlots)) - 1u;
+    m |= (1u << min(cnt[e], 2 * kTransSlots)) - 1u;
   for (int d = 32; d > 0; d >>= 1) m |= __shfl_xor(m, d);
   if ((threadIdx.x & 63) == 0 && m) atomicOr(&block_mask, m);
   __syncthreads();
-  report_pairs_beyond_two(mask, block_mask);
+  report_pairs_beyond_two(mask, block_mask & ((1u << kTransSlots) - 1u));
+  if (two_level && threadIdx.x == 0) {
+    const unsigned m2 = block_mask >> kTransSlots;
+    if (m2 && (m2 & ~(unsigned)__hip_atomic_load(mask + 1, __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT)))
+      atomicOr(mask + 1, (int)m2);
+  }
   if (overflow[0] != 0 || overflow[1] <= 0) return;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
        i += (int64_t)gridDim.x * blockDim.x)
@@ -1645,7 +1661,8 @@ __global__ void convert_planes_kernel(const float *__restrict__ src, TD *__restr
 }
 
 struct ScatterScratch {
-  size_t wq, wpt, cnt, tmap, acc32, ovf, stage, total;  // byte offsets
+  size_t wq, wpt, cnt, tmap, tmap2, acc32, ovf, stage, total;  // byte offsets
+  bool two_level;  // a second four-slot level, applied by a second gather pass
   int64_t ovf_cap;  // entries of the overflow list (0: none)
   bool transposed_path;
 };
@@ -1660,6 +1677,11 @@ ScatterScratch scatter_scratch(int64_t B, int64_t S, int64_t D, int64_t K, int64
   off += align256((size_t)(K * ((D + kScDC - 1) / kScDC) * round_up(S, kScSC) * kScDC) * 4);
   const int64_t cells = DH * DW * K;
   sc.transposed_path = cells * kTransSlots * 2 <= 0x7fffffffLL;
+  // Single-row maps (mesh signals) point anywhere, and their cells fill unevenly: with K * P
+  // contributions per vertex on average a four-slot cell overflows often, an eight-slot
+  // one rarely.
+  sc.two_level = sc.transposed_path && MH == 1;
+  sc.tmap2 = 0;
   // One fp32 image: the scatter kernel's accumulation image of a non-fp32 destination
   // ([B][D][DN]) or the channel-last overflow image ([B][DN][D padded to 64]); never both.
   sc.acc32 = off;
@@ -1676,6 +1698,8 @@ ScatterScratch scatter_scratch(int64_t B, int64_t S, int64_t D, int64_t K, int64
     off += align256((size_t)(cells + 4) * 4);
     sc.tmap = off;  // [cell][slot] (source pixel index as bits, weight)
     off += align256((size_t)cells * kTransSlots * 2 * 4);
+    sc.tmap2 = off;
+    if (sc.two_level) off += align256((size_t)cells * kTransSlots * 2 * 4);
   }
   // Overflow list: room for half of the contributions a bilinear map can make.
   sc.ovf = sc.stage = off;
@@ -1715,6 +1739,7 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
     // build the transposed map, then try the atomic-free gather form first
     int *cnt = (int *)(base + sc.cnt);
     float2 *tmap = (float2 *)(base + sc.tmap);
+    float2 *tmap2 = sc.two_level ? (float2 *)(base + sc.tmap2) : nullptr;
     float *wpt = (float *)(base + sc.wpt);
     const int64_t cells = DH * DW * K;
     int *flag = cnt + cells;
@@ -1726,11 +1751,11 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
     const unsigned blocks = (unsigned)((entries + 255) / 256);
     if (m.mode == kInterpNearest)
       hipLaunchKernelGGL(build_transposed_map_kernel<1>, dim3(blocks), dim3(256), 0, s, map, iw,
-                         cnt, tmap, flag, ovf, (int)sc.ovf_cap, m.np, m.weighted, m.wrap,
+                         cnt, tmap, tmap2, flag, ovf, (int)sc.ovf_cap, m.np, m.weighted, m.wrap,
                          (int)DH, (int)DW, (int)MW, (int)K, entries);
     else
       hipLaunchKernelGGL(build_transposed_map_kernel<4>, dim3(blocks), dim3(256), 0, s, map, iw,
-                         cnt, tmap, flag, ovf, (int)sc.ovf_cap, m.np, m.weighted, m.wrap,
+                         cnt, tmap, tmap2, flag, ovf, (int)sc.ovf_cap, m.np, m.weighted, m.wrap,
                          (int)DH, (int)DW, (int)MW, (int)K, entries);
     MCX_HIP_CHECK_LAUNCH();
     if (int rc = launch_pack_weights<TD>(w, wpt, D, S, K, 1, s)) return rc;
@@ -1746,7 +1771,8 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
     hipLaunchKernelGGL(after_transposed_map_kernel,
                        dim3((unsigned)std::min<int64_t>(
                            std::max((total_img + 1023) / 1024, (cells + 255) / 256), 4096)),
-                       dim3(256), 0, s, cnt, cells, flag + 2, img, total_img, flag);
+                       dim3(256), 0, s, cnt, cells, flag + 2, sc.two_level ? 1 : 0, img, total_img,
+                       flag);
     MCX_HIP_CHECK_LAUNCH();
     if (cl) {  // the overflow pass reads the channel-last copy before the gather would make it
       dim3 tg((unsigned)((MH * MW + 63) / 64), (unsigned)((Spad16 + 63) / 64), (unsigned)B);
@@ -1763,6 +1789,12 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
                                            stage, B, S, D, MH, MW, DH, DW, K, kTransSlots,
                                            kInterpNearest, gate, 1, s, img, cl, flag + 2, true))
       return rc;
+    if (sc.two_level)  // entries five to eight of every cell, added onto dst
+      if (int rc = launch_gather_product<TD>(src, (const float *)tmap2, nullptr, wpt,
+                                             (const TD *)nullptr, dst, stage, B, S, D, MH, MW, DH,
+                                             DW, K, kTransSlots, kInterpNearest, gate, 1, s,
+                                             nullptr, cl, flag + 3, true, true))
+        return rc;
   }
 
   // atomic path (runs when there is no transposed map or it overflowed)
