@@ -45,27 +45,58 @@ __global__ void fill_kernel(T *p, int64_t n, T v) {
 // OP_MAX: strict-greater running maximum from -FLT_MAX and the winning tap's
 // map offset (include/nn/common/mapped_max_pool.h:14-58).
 // grid: x over map locations, y over channel chunks, z over images.
+// The work of one thread: map location n, channels [c0, c0 + kCH) of image b.
 template <typename T, int MODE, int OP>
-__global__ __launch_bounds__(kThreads) void gather_kernel(
-    const T *__restrict__ in, const T *__restrict__ map, const T *__restrict__ iw,
-    T *__restrict__ out, int64_t *__restrict__ idx, int C, int IH, int IW, int N, int MW, int K,
-    int P) {
-  constexpr int kTileW = Patch<OP>::kW, kTileH = Patch<OP>::kH;
-  const int tiles_x = (MW + kTileW - 1) / kTileW;
-  // (pooling only: a resampling map's rows need not read neighbouring source rows, and the
-  // round-robin order measured faster there)
-  const int tile = OP == OP_RESAMPLE ? (int)blockIdx.x : xcd_contiguous(blockIdx.x, gridDim.x);
-  const int tx = (tile % tiles_x) * kTileW + threadIdx.x % kTileW;
-  const int ty = (tile / tiles_x) * kTileH + threadIdx.x / kTileW;
-  const int n = ty * MW + tx;
-  if (tx >= MW || n >= N) return;
-  const int c0 = blockIdx.y * kCH;
-  const int b = blockIdx.z;
+__device__ inline void direct_gather(const T *__restrict__ in, const T *__restrict__ map,
+                                     const T *__restrict__ iw, T *__restrict__ out,
+                                     int64_t *__restrict__ idx, int C, int IH, int IW, int N,
+                                     int K, int P, int n, int c0, int b) {
   const int64_t plane = (int64_t)IH * IW;
   const T *src = in + ((int64_t)b * C + c0) * plane;
   const int pm = P == 0 ? 1 : P;
   const int nc = min(kCH, C - c0);
 
+  if constexpr (OP != OP_RESAMPLE) {
+    // Pooling with few unweighted taps: resolve them all first and walk the channels in the
+    // outer loop, so that the K x 2..4 reads of one channel's few source rows follow each
+    // other closely and hit in cache (with the taps outside, a line was gone before the
+    // next tap came back to it: every sampled byte came from memory).
+    constexpr int kTaps = 9;
+    if (P == 0 && K <= kTaps) {
+      Tap<T, MODE> taps[kTaps];
+#pragma unroll
+      for (int k = 0; k < kTaps; k++) {
+        const int64_t e = (int64_t)n * K + min(k, K - 1);
+        taps[k].set(map[e * 2], map[e * 2 + 1], IH, IW);
+      }
+      const int64_t o = ((int64_t)b * C + c0) * N + n;
+      for (int c = 0; c < nc; c++) {
+        const T *pl = src + c * plane;
+        T val[kTaps];
+#pragma unroll
+        for (int k = 0; k < kTaps; k++) val[k] = taps[k].gather(pl);
+        T a = OP == OP_MAX ? T(-3.402823466e+38F) : T(0);
+        int bk = -1;
+#pragma unroll
+        for (int k = 0; k < kTaps; k++) {
+          if (k < K) {
+            if (OP == OP_MAX) {
+              if (val[k] > a) {
+                a = val[k];
+                bk = k;
+              }
+            } else {
+              a += val[k];
+            }
+          }
+        }
+        out[o + (int64_t)c * N] = OP == OP_AVG ? a / (T)K : a;
+        if (OP == OP_MAX)
+          idx[o + (int64_t)c * N] = bk < 0 ? (int64_t)-1 : ((int64_t)n * K + bk) * 2;
+      }
+      return;
+    }
+  }
   T acc[kCH];
   int64_t best[kCH];
 #pragma unroll
@@ -126,6 +157,24 @@ __global__ __launch_bounds__(kThreads) void gather_kernel(
     out[o + (int64_t)c * N] = OP == OP_AVG ? acc[c] / (T)K : acc[c];
     if (OP == OP_MAX) idx[o + (int64_t)c * N] = best[c];
   }
+}
+
+template <typename T, int MODE, int OP>
+__global__ __launch_bounds__(kThreads) void gather_kernel(
+    const T *__restrict__ in, const T *__restrict__ map, const T *__restrict__ iw,
+    T *__restrict__ out, int64_t *__restrict__ idx, int C, int IH, int IW, int N, int MW, int K,
+    int P) {
+  constexpr int kTileW = Patch<OP>::kW, kTileH = Patch<OP>::kH;
+  const int tiles_x = (MW + kTileW - 1) / kTileW;
+  // (pooling only: a resampling map's rows need not read neighbouring source rows, and the
+  // round-robin order measured faster there)
+  const int tile = OP == OP_RESAMPLE ? (int)blockIdx.x : xcd_contiguous(blockIdx.x, gridDim.x);
+  const int tx = (tile % tiles_x) * kTileW + threadIdx.x % kTileW;
+  const int ty = (tile / tiles_x) * kTileH + threadIdx.x / kTileW;
+  const int n = ty * MW + tx;
+  if (tx >= MW || n >= N) return;
+  direct_gather<T, MODE, OP>(in, map, iw, out, idx, C, IH, IW, N, K, P, n, blockIdx.y * kCH,
+                             blockIdx.z);
 }
 
 // Scatter form (adjoint of the gather).  OP_RESAMPLE: K == 1, pushes the value;
