@@ -394,6 +394,50 @@ __global__ __launch_bounds__(kThreads) void transposed_gather_kernel(
   const uint32_t end = local[p + 1] + bsum[(p + 1) / kScanBlock];
   const T *s0 = src + plane0 * nsrc;
   const int64_t *i0 = OP == UN_MAX ? idx + plane0 * nsrc : nullptr;
+  // Short lists (every lane of the wave has at most kListRegs entries: pooling maps): the
+  // list is read once into registers and the planes are walked in the outer loop, so that a
+  // plane's few source rows are read in one go and hit in cache; with the planes inside,
+  // every sampled byte came from memory.  The additions keep the order of the list.
+  constexpr int kListRegs = 24, kGroup = 6;
+  const uint32_t len = end - start;
+  if (OP != UN_RESAMPLE && __builtin_amdgcn_ballot_w64(len > (uint32_t)kListRegs) == 0) {
+    uint32_t code[kListRegs];
+    T w[kListRegs];
+    uint32_t longest = len;
+    for (int d = 32; d > 0; d >>= 1) longest = max(longest, (uint32_t)__shfl_xor((int)longest, d));
+    longest = __builtin_amdgcn_readfirstlane(longest);
+#pragma unroll
+    for (int u = 0; u < kListRegs; u++) {
+      const bool in = (uint32_t)u < len;
+      code[u] = e_src[in ? start + u : (len ? start : 0u)];
+      w[u] = in ? e_wt[start + u] : T(0);
+    }
+    T *d0 = dst + plane0 * ndst + p;
+    for (int c = 0; c < nc; c++) {
+      const T *sc = s0 + (int64_t)c * nsrc;
+      const int64_t *ic = OP == UN_MAX ? i0 + (int64_t)c * nsrc : nullptr;
+      T a = T(0);
+#pragma unroll
+      for (int g = 0; g < kListRegs / kGroup; g++) {
+        if ((uint32_t)(g * kGroup) < longest) {  // wave-uniform, once per six entries
+          T v[kGroup];
+          bool keep[kGroup];
+#pragma unroll
+          for (int j = 0; j < kGroup; j++) {
+            const uint32_t cd = code[g * kGroup + j];
+            const uint32_t n = OP == UN_MAX ? cd / (uint32_t)K : cd;
+            v[j] = sc[n];
+            keep[j] = OP == UN_MAX ? ic[n] == (int64_t)cd * idx_scale : true;
+          }
+#pragma unroll
+          for (int j = 0; j < kGroup; j++)
+            if (keep[j]) a = mcx_fma(w[g * kGroup + j], v[j], a);
+        }
+      }
+      d0[(int64_t)c * ndst] = OP == UN_AVG ? a / (T)K : a;
+    }
+    return;
+  }
   T acc[kTCH];
 #pragma unroll
   for (int c = 0; c < kTCH; c++) acc[c] = T(0);
