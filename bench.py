@@ -95,6 +95,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--interp", default="bilinear", choices=["bilinear", "nearest"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--map-plan-cache", action="store_true",
+                    help="not the headline configuration: keep the backward's plan of the sample "
+                         "map (transposed map, pair masks) across steps instead of rebuilding "
+                         "it in every call as the reference's kernels decode the map every call")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="before the warm-up, run three plain copy kernels over the input "
                          "(reads and writes B*Ci*H*W*4 bytes each) so that a counter run of this "
@@ -105,6 +109,7 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
     interp = 1 if args.interp == "bilinear" else 0
+    _C.enable_map_plan_cache(args.map_plan_cache)
     dev = torch.device("cuda:0")
     inputs = make_inputs(dev)
 
@@ -147,7 +152,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "MappedConvolution fwd+bwd B8 Ci64 Co64 256x512 K9 latitude map, "
-                               + args.interp, "interpolation": args.interp},
+                               + args.interp, "interpolation": args.interp,
+                   "map_plan_cache": bool(args.map_plan_cache)},
         "roofline": {"bound": "mfma", "kernel": KERNEL_OF.get(dominant, dominant) if interp == 1
                      else dominant,
                      "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS,

@@ -181,6 +181,27 @@ int mcx_tconv_backward(const void *gy, const void *map, const void *iw, const vo
                        int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
                        int dtype, void *stream);
 
+/* Map plan: no counterpart in the reference, which decodes sample_map inside its kernels at
+ * every call.  A training loop applies the same sample_map at every step, so what the
+ * backward derives from the map alone - the transposed map of its input gradient and the
+ * "which pairs are in use" masks - can be built once and reused.  A plan belongs to one
+ * (sample_map, interp_weights, interp, IH x IW, OH x OW, K, P); the caller rebuilds it when
+ * the map's contents change.  mcx_conv_plan_bytes is 0 where no plan exists (F64, P > 4):
+ * pass NULL, 0 then.  mcx_conv_backward_planned is mcx_conv_backward with the plan in place
+ * of the per-call build (plan NULL: identical to mcx_conv_backward); it only reads the plan,
+ * so one plan may serve concurrent calls. */
+size_t mcx_conv_plan_bytes(int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P,
+                           int dtype);
+int mcx_conv_plan_build(const void *map, const void *iw, void *plan, size_t plan_bytes,
+                        int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P,
+                        int interp, int dtype, void *stream);
+int mcx_conv_backward_planned(const void *gy, const void *map, const void *iw, const void *x,
+                              const void *w, void *gx, void *gw, void *gb, void *workspace,
+                              size_t workspace_bytes, const void *plan, size_t plan_bytes,
+                              int64_t B, int64_t Ci, int64_t Co, int64_t IH, int64_t IW,
+                              int64_t OH, int64_t OW, int64_t K, int64_t P, int interp, int dtype,
+                              void *stream);
+
 /* ---- KNN -------------------------------------------------------------------- */
 
 /* knn_forward: include/util/layers/knn_layer.h:25-35,41; kernels

@@ -142,8 +142,70 @@ def _conv_forward(input, sample_map, interp_weights, weight, bias, kernel_size, 
     return out
 
 
+# ---- map plans (no counterpart in the reference) ------------------------------------
+# What the convolution backward derives from sample_map alone (the transposed map of the
+# input gradient and the masks of pairs in use) can be built once and reused while the map
+# does not change.  `conv_map_plan` builds such a plan explicitly; with `map_plan_cache` set
+# to a dict (see enable_map_plan_cache) the backward ops keep the plans of the maps they
+# have seen, keyed by the tensors' storage and in-place version counters.  Off by default:
+# every call then rebuilds what it needs, like the reference.
+map_plan_cache = None
+_MAP_PLAN_CACHE_ENTRIES = 16
+
+
+def enable_map_plan_cache(enabled=True):
+    """Keep (or stop keeping) the plans of the sample maps seen by the convolution backward."""
+    global map_plan_cache
+    map_plan_cache = {} if enabled else None
+
+
+def conv_map_plan(sample_map, interp_weights, input_height, input_width, interpolation,
+                  data_dtype=torch.float32):
+    """Plan of a MappedConvolution's backward for one sample_map [OH, OW, K, (P,) 2] over an
+    input of input_height x input_width; None where the library has no plan for the case
+    (float64 data, P > 4).  Pass it as `plan=` to mapped_conv_backward /
+    weighted_mapped_conv_backward for as long as the map's contents stay the same."""
+    _contig(sample_map=sample_map, interp_weights=interp_weights)
+    _on_gpu("sample_map", sample_map, interp_weights=interp_weights)
+    P = _weighted_dims(sample_map, interp_weights, True)
+    OH, OW, K = sample_map.shape[:3]
+    dt = _DTYPES[data_dtype]
+    want = torch.float32 if data_dtype == torch.bfloat16 else data_dtype
+    if sample_map.dtype != want:
+        raise RuntimeError("sample_map must be %s for %s data" % (want, data_dtype))
+    lib = _lib.load()
+    IH, IW = int(input_height), int(input_width)
+    nbytes = lib.mcx_conv_plan_bytes(IH, IW, OH, OW, K, P, dt)
+    if nbytes == 0:
+        return None
+    plan = torch.empty((nbytes,), dtype=torch.uint8, device=sample_map.device)
+    with torch.cuda.device(sample_map.device):
+        rc = lib.mcx_conv_plan_build(_ptr(sample_map), _ptr(interp_weights), _ptr(plan), nbytes,
+                                     IH, IW, OH, OW, K, P, int(interpolation), dt,
+                                     _stream(sample_map))
+    _lib.check(rc, "conv_map_plan")
+    return plan
+
+
+def _cached_plan(sample_map, interp_weights, IH, IW, interpolation, data_dtype):
+    """Plan from the cache, rebuilt when a tensor was modified in place or replaced."""
+    def ident(t):
+        return None if t is None else (t.data_ptr(), t._version, tuple(t.shape))
+    key = (ident(sample_map), ident(interp_weights), IH, IW, int(interpolation), data_dtype,
+           sample_map.device.index)
+    hit = map_plan_cache.get(key)
+    if hit is not None:
+        return hit[0]
+    plan = conv_map_plan(sample_map, interp_weights, IH, IW, interpolation, data_dtype)
+    if len(map_plan_cache) >= _MAP_PLAN_CACHE_ENTRIES:
+        map_plan_cache.pop(next(iter(map_plan_cache)))
+    # the entry keeps the tensors alive, so their addresses cannot be handed to other maps
+    map_plan_cache[key] = (plan, sample_map, interp_weights)
+    return plan
+
+
 def _conv_backward(grad_output, sample_map, interp_weights, input, weight, bias, kernel_size,
-                   interpolation):
+                   interpolation, plan=None):
     _contig(input=input, sample_map=sample_map, interp_weights=interp_weights, weight=weight,
             bias=bias)
     grad_output = grad_output.contiguous()  # the reference reads it raw without a check
@@ -162,6 +224,9 @@ def _conv_backward(grad_output, sample_map, interp_weights, input, weight, bias,
     lib = _lib.load()
     ws_bytes = lib.mcx_conv_backward_workspace(B, Ci, Co, IH, IW, OH, OW, K, P, dt)
     ws = _workspace(ws_bytes, input.device)
+    if plan is None and map_plan_cache is not None:
+        plan = _cached_plan(sample_map, interp_weights, IH, IW, interpolation, input.dtype)
+    plan_bytes = 0 if plan is None else plan.numel()
     # Two C-ABI calls (NULL skips a gradient) so that the input gradient and the weight
     # gradient can be timed alone; the bias gradient rides on the weight gradient's pass
     # over grad_output.
@@ -169,10 +234,11 @@ def _conv_backward(grad_output, sample_map, interp_weights, input, weight, bias,
             "conv_backward_weight": (None, grad_weight, grad_bias)}
     with torch.cuda.device(input.device):
         for label, (gx, gw, gb) in outs.items():
-            rc = _timed(label, input.device, lambda: lib.mcx_conv_backward(
+            rc = _timed(label, input.device, lambda: lib.mcx_conv_backward_planned(
                 _ptr(grad_output), _ptr(sample_map), _ptr(interp_weights), _ptr(input),
-                _ptr(weight), _ptr(gx), _ptr(gw), _ptr(gb), _ptr(ws), ws_bytes, B, Ci, Co, IH, IW,
-                OH, OW, K, P, int(interpolation), dt, _stream(input)))
+                _ptr(weight), _ptr(gx), _ptr(gw), _ptr(gb), _ptr(ws), ws_bytes, _ptr(plan),
+                plan_bytes, B, Ci, Co, IH, IW, OH, OW, K, P, int(interpolation), dt,
+                _stream(input)))
             _lib.check(rc, "mapped_conv_backward")
     return [grad_input, grad_weight, grad_bias]
 
@@ -182,10 +248,12 @@ def mapped_conv_forward(input, sample_map, weight, bias, kernel_size, interpolat
     return _conv_forward(input, sample_map, None, weight, bias, kernel_size, interpolation)
 
 
-def mapped_conv_backward(grad_output, sample_map, input, weight, bias, kernel_size, interpolation):
-    """include/nn/layers/mapped_convolution_layer.h:90-93 -> [grad_input, grad_weight, grad_bias]."""
+def mapped_conv_backward(grad_output, sample_map, input, weight, bias, kernel_size, interpolation,
+                         plan=None):
+    """include/nn/layers/mapped_convolution_layer.h:90-93 -> [grad_input, grad_weight, grad_bias].
+    `plan` (optional, not in the reference): see conv_map_plan."""
     return _conv_backward(grad_output, sample_map, None, input, weight, bias, kernel_size,
-                          interpolation)
+                          interpolation, plan)
 
 
 def weighted_mapped_conv_forward(input, sample_map, interp_weights, weight, bias, kernel_size,
@@ -196,10 +264,10 @@ def weighted_mapped_conv_forward(input, sample_map, interp_weights, weight, bias
 
 
 def weighted_mapped_conv_backward(grad_output, sample_map, interp_weights, input, weight, bias,
-                                  kernel_size, interpolation):
-    """include/nn/layers/weighted_mapped_convolution_layer.h:97-100."""
+                                  kernel_size, interpolation, plan=None):
+    """include/nn/layers/weighted_mapped_convolution_layer.h:97-100.  `plan`: see conv_map_plan."""
     return _conv_backward(grad_output, sample_map, interp_weights, input, weight, bias,
-                          kernel_size, interpolation)
+                          kernel_size, interpolation, plan)
 
 
 # ---------------------------------------------------------------- transposed conv

@@ -33,6 +33,9 @@ SIGNATURES = {
     "mcx_conv_forward_workspace": (_sz, [_i64] * 9 + [_i]),
     "mcx_conv_backward_workspace": (_sz, [_i64] * 9 + [_i]),
     "mcx_conv_backward": (_i, [_p] * 9 + [_sz] + [_i64] * 9 + [_i, _i, _p]),
+    "mcx_conv_plan_bytes": (_sz, [_i64] * 6 + [_i]),
+    "mcx_conv_plan_build": (_i, [_p] * 3 + [_sz] + [_i64] * 6 + [_i, _i, _p]),
+    "mcx_conv_backward_planned": (_i, [_p] * 9 + [_sz, _p, _sz] + [_i64] * 9 + [_i, _i, _p]),
     "mcx_tconv_forward": (_i, [_p] * 7 + [_sz] + [_i64] * 9 + [_i, _i, _p]),
     "mcx_tconv_forward_workspace": (_sz, [_i64] * 9 + [_i]),
     "mcx_tconv_backward_workspace": (_sz, [_i64] * 9 + [_i]),

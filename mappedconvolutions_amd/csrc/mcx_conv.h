@@ -47,14 +47,22 @@ template <typename TD>
 int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const float *iw, TD *gw,
                      void *scratch, int64_t B, int64_t A, int64_t G, int64_t GH, int64_t GW,
                      int64_t MH, int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s,
-                     TD *plain_sum);
+                     TD *plain_sum, const void *plan = nullptr);
 size_t mfma_product_scatter_bytes(int64_t B, int64_t S, int64_t D, int64_t K, int64_t DH,
                                   int64_t DW, size_t elem, int64_t MH, int64_t MW, int64_t P);
 template <typename TD>
 int mfma_product_scatter(const TD *src, const float *map, const float *iw, const TD *w,
                          const TD *bias, TD *dst, void *scratch, int64_t B, int64_t S, int64_t D,
                          int64_t DH, int64_t DW, int64_t MH, int64_t MW, int64_t K, int64_t P,
-                         int interp, hipStream_t s);
+                         int interp, hipStream_t s, const void *plan = nullptr);
+// A plan is the transposed map of one sample map (DH x DW: the image the map samples; MH x MW:
+// the map), built once and passed to mfma_product_scatter / mfma_weight_grad in place of the
+// per-call build.  0 bytes: this shape has no transposed-map path.
+size_t mfma_scatter_plan_bytes(int64_t DH, int64_t DW, int64_t MH, int64_t MW, int64_t K,
+                               int64_t P);
+int mfma_scatter_plan_build(const float *map, const float *iw, void *plan, int64_t DH, int64_t DW,
+                            int64_t MH, int64_t MW, int64_t K, int64_t P, int interp,
+                            hipStream_t s);
 size_t mfma_bias_grad_bytes(int64_t B, int64_t C, int64_t N);
 template <typename TD>
 int mfma_bias_grad(const TD *g, TD *gb, void *scratch, int64_t B, int64_t C, int64_t N,

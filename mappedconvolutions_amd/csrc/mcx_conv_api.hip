@@ -82,14 +82,15 @@ template <typename T>
 int product_scatter(bool mfma, const void *src, const void *map, const void *iw, const void *w,
                     const void *bias, void *dst, void *ws, size_t ws_bytes, int64_t B, int64_t S,
                     int64_t D, int64_t DH, int64_t DW, int64_t MH, int64_t MW, int64_t K, int64_t P,
-                    int interp, hipStream_t s);
+                    int interp, hipStream_t s, const void *plan = nullptr);  // plan: see mcx.h
 
 // gW[a,g,k] = sum_{b,n} plain[b,a,n] * sample(gath[b,g], map[n,k]); n over MH x MW.
 template <typename T>
 int weight_grad(bool mfma, const void *plain, const void *gath, const void *map, const void *iw,
                 void *gw, void *ws, size_t ws_bytes, int64_t B, int64_t A, int64_t G, int64_t GH,
                 int64_t GW, int64_t MH, int64_t MW, int64_t K, int64_t P, int interp,
-                hipStream_t s, void *plain_sum);  // plain_sum: matrix-core path only, may be NULL
+                hipStream_t s, void *plain_sum,  // plain_sum: matrix-core path only, may be NULL
+                const void *plan = nullptr);
 
 // gb[c] = sum over (b, n) of gy[b,c,n].
 template <typename T>
@@ -110,7 +111,7 @@ int bias_grad(const void *gy, void *gb, void *ws, size_t ws_bytes, int64_t B, in
   int product_scatter<T>(bool, const void *src, const void *map, const void *iw, const void *w,    \
                          const void *bias, void *dst, void *, size_t, int64_t B, int64_t S,        \
                          int64_t D, int64_t DH, int64_t DW, int64_t MH, int64_t MW, int64_t K,     \
-                         int64_t P, int interp, hipStream_t s) {                                   \
+                         int64_t P, int interp, hipStream_t s, const void *) {                     \
     int rc = bias ? fill_bias<T>((T *)dst, (const T *)bias, B, D, DH * DW, s)                      \
                   : fill_zero<T>((T *)dst, B * D * DH * DW, s);                                    \
     if (rc) return rc;                                                                             \
@@ -122,7 +123,7 @@ int bias_grad(const void *gy, void *gb, void *ws, size_t ws_bytes, int64_t B, in
   int weight_grad<T>(bool, const void *plain, const void *gath, const void *map, const void *iw,   \
                      void *gw, void *, size_t, int64_t B, int64_t A, int64_t G, int64_t GH,        \
                      int64_t GW, int64_t MH, int64_t MW, int64_t K, int64_t P, int interp,         \
-                     hipStream_t s, void *) {                                                      \
+                     hipStream_t s, void *, const void *) {                                        \
     return generic_weight_grad<T>((const T *)plain, (const T *)gath, (const T *)map,               \
                                   (const T *)iw, (T *)gw, B, A, G, GH, GW, MH * MW, K, P, interp,  \
                                   s);                                                              \
@@ -159,7 +160,8 @@ template <>
 int product_scatter<float>(bool mfma, const void *src, const void *map, const void *iw,
                            const void *w, const void *bias, void *dst, void *ws, size_t ws_bytes,
                            int64_t B, int64_t S, int64_t D, int64_t DH, int64_t DW, int64_t MH,
-                           int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s) {
+                           int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s,
+                           const void *plan) {
   if (!mfma) {
     int rc = bias ? fill_bias<float>((float *)dst, (const float *)bias, B, D, DH * DW, s)
                   : fill_zero<float>((float *)dst, B * D * DH * DW, s);
@@ -172,14 +174,14 @@ int product_scatter<float>(bool mfma, const void *src, const void *map, const vo
     return MCX_E_WORKSPACE;
   return mfma_product_scatter<float>((const float *)src, (const float *)map, (const float *)iw,
                                      (const float *)w, (const float *)bias, (float *)dst, ws, B, S,
-                                     D, DH, DW, MH, MW, K, P, interp, s);
+                                     D, DH, DW, MH, MW, K, P, interp, s, plan);
 }
 
 template <>
 int weight_grad<float>(bool mfma, const void *plain, const void *gath, const void *map,
                        const void *iw, void *gw, void *ws, size_t ws_bytes, int64_t B, int64_t A,
                        int64_t G, int64_t GH, int64_t GW, int64_t MH, int64_t MW, int64_t K,
-                       int64_t P, int interp, hipStream_t s, void *plain_sum) {
+                       int64_t P, int interp, hipStream_t s, void *plain_sum, const void *plan) {
   if (!mfma)
     return generic_weight_grad<float>((const float *)plain, (const float *)gath,
                                       (const float *)map, (const float *)iw, (float *)gw, B, A, G,
@@ -188,7 +190,7 @@ int weight_grad<float>(bool mfma, const void *plain, const void *gath, const voi
     return MCX_E_WORKSPACE;
   return mfma_weight_grad<float>((const float *)plain, (const float *)gath, (const float *)map,
                                  (const float *)iw, (float *)gw, ws, B, A, G, GH, GW, MH, MW, K, P,
-                                 interp, s, (float *)plain_sum);
+                                 interp, s, (float *)plain_sum, plan);
 }
 
 template <>
@@ -216,26 +218,28 @@ template <>
 int product_scatter<bf16_t>(bool mfma, const void *src, const void *map, const void *iw,
                             const void *w, const void *bias, void *dst, void *ws, size_t ws_bytes,
                             int64_t B, int64_t S, int64_t D, int64_t DH, int64_t DW, int64_t MH,
-                            int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s) {
+                            int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s,
+                            const void *plan) {
   if (!mfma) return MCX_E_DTYPE;
   if (!ws || ws_bytes < mfma_product_scatter_bytes(B, S, D, K, DH, DW, 2, MH, MW, P))
     return MCX_E_WORKSPACE;
   return mfma_product_scatter<bf16_t>((const bf16_t *)src, (const float *)map, (const float *)iw,
                                       (const bf16_t *)w, (const bf16_t *)bias, (bf16_t *)dst, ws,
-                                      B, S, D, DH, DW, MH, MW, K, P, interp, s);
+                                      B, S, D, DH, DW, MH, MW, K, P, interp, s, plan);
 }
 
 template <>
 int weight_grad<bf16_t>(bool mfma, const void *plain, const void *gath, const void *map,
                         const void *iw, void *gw, void *ws, size_t ws_bytes, int64_t B, int64_t A,
                         int64_t G, int64_t GH, int64_t GW, int64_t MH, int64_t MW, int64_t K,
-                        int64_t P, int interp, hipStream_t s, void *plain_sum) {
+                        int64_t P, int interp, hipStream_t s, void *plain_sum,
+                        const void *plan) {
   if (!mfma) return MCX_E_DTYPE;
   if (!ws || ws_bytes < mfma_weight_grad_bytes(B, A, G, MH, MW, K, GH, GW))
     return MCX_E_WORKSPACE;
   return mfma_weight_grad<bf16_t>((const bf16_t *)plain, (const bf16_t *)gath, (const float *)map,
                                   (const float *)iw, (bf16_t *)gw, ws, B, A, G, GH, GW, MH, MW, K,
-                                  P, interp, s, (bf16_t *)plain_sum);
+                                  P, interp, s, (bf16_t *)plain_sum, plan);
 }
 
 template <>
@@ -257,16 +261,17 @@ int conv_forward_t(bool mfma, const void *x, const void *map, const void *iw, co
 template <typename T>
 int conv_backward_t(bool mfma, const void *gy, const void *map, const void *iw, const void *x,
                     const void *w, void *gx, void *gw, void *gb, void *ws, size_t ws_bytes,
-                    const ConvDims &d, int interp, hipStream_t s) {
+                    const ConvDims &d, int interp, hipStream_t s, const void *plan = nullptr) {
   int rc = 0;
   if (gx && (rc = product_scatter<T>(mfma, gy, map, iw, w, nullptr, gx, ws, ws_bytes, d.B, d.Co,
-                                     d.Ci, d.IH, d.IW, d.OH, d.OW, d.K, d.P, interp, s)))
+                                     d.Ci, d.IH, d.IW, d.OH, d.OW, d.K, d.P, interp, s, plan)))
     return rc;
   // the matrix-core weight gradient stages every tile of gy: it sums them for the bias
   // gradient on the way
   const bool fused_bias = gw && gb && mfma;
   if (gw && (rc = weight_grad<T>(mfma, gy, x, map, iw, gw, ws, ws_bytes, d.B, d.Co, d.Ci, d.IH,
-                                 d.IW, d.OH, d.OW, d.K, d.P, interp, s, fused_bias ? gb : nullptr)))
+                                 d.IW, d.OH, d.OW, d.K, d.P, interp, s, fused_bias ? gb : nullptr,
+                                 plan)))
     return rc;
   if (gb && !fused_bias) rc = bias_grad<T>(gy, gb, ws, ws_bytes, d.B, d.Co, d.OH * d.OW, s);
   return rc;
@@ -351,6 +356,47 @@ extern "C" int mcx_conv_backward(const void *gy, const void *map, const void *iw
                                                workspace_bytes, d, interp, s));
 }
 
+extern "C" size_t mcx_conv_plan_bytes(int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
+                                      int64_t P, int dtype) {
+  if (IH <= 0 || IW <= 0 || OH <= 0 || OW <= 0 || K <= 0 || P < 0) return 0;
+  return use_mfma(dtype, P) ? mfma_scatter_plan_bytes(IH, IW, OH, OW, K, P) : 0;
+}
+
+extern "C" int mcx_conv_plan_build(const void *map, const void *iw, void *plan, size_t plan_bytes,
+                                   int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
+                                   int64_t P, int interp, int dtype, void *stream) {
+  if (IH <= 0 || IW <= 0 || OH <= 0 || OW <= 0 || K <= 0 || P < 0) return MCX_E_SHAPE;
+  if (!map || !plan || (P > 0) != (iw != nullptr)) return MCX_E_NULL;
+  if (!use_mfma(dtype, P)) return MCX_E_DTYPE;
+  const size_t need = mfma_scatter_plan_bytes(IH, IW, OH, OW, K, P);
+  if (need == 0) return MCX_E_SHAPE;
+  if (plan_bytes < need) return MCX_E_WORKSPACE;
+  return mfma_scatter_plan_build((const float *)map, (const float *)iw, plan, IH, IW, OH, OW, K,
+                                 P, interp, (hipStream_t)stream);
+}
+
+extern "C" int mcx_conv_backward_planned(const void *gy, const void *map, const void *iw,
+                                         const void *x, const void *w, void *gx, void *gw,
+                                         void *gb, void *workspace, size_t workspace_bytes,
+                                         const void *plan, size_t plan_bytes, int64_t B,
+                                         int64_t Ci, int64_t Co, int64_t IH, int64_t IW,
+                                         int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
+                                         int dtype, void *stream) {
+  const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
+  if (int rc = check_dims(d, OH, OW)) return rc;
+  if (int rc = check_ptrs(gy, map, iw, w, P)) return rc;
+  if (gw && !x) return MCX_E_NULL;
+  hipStream_t s = (hipStream_t)stream;
+  const bool mfma = use_mfma(dtype, P);
+  if (plan) {
+    if (!mfma) return MCX_E_DTYPE;
+    const size_t need = mfma_scatter_plan_bytes(IH, IW, OH, OW, K, P);
+    if (need == 0 || plan_bytes < need) return MCX_E_WORKSPACE;
+  }
+  MCX_DISPATCH_DTYPE(dtype, conv_backward_t<T>(mfma, gy, map, iw, x, w, gx, gw, gb, workspace,
+                                               workspace_bytes, d, interp, s, plan));
+}
+
 extern "C" size_t mcx_tconv_forward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t IH,
                                               int64_t IW, int64_t OH, int64_t OW, int64_t K,
                                               int64_t P, int dtype) {
@@ -397,7 +443,7 @@ extern "C" int mcx_tconv_backward(const void *gy, const void *map, const void *i
                                                 workspace_bytes, d, interp, s));
 }
 
-extern "C" int mcx_abi_version(void) { return 6; }
+extern "C" int mcx_abi_version(void) { return 7; }
 
 extern "C" int mcx_profile_dominant_kernel(void *start_event, void *stop_event) {
   mcx::set_profile_events(start_event, stop_event);

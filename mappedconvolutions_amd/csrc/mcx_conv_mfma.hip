@@ -1425,7 +1425,7 @@ template <typename TD>
 int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const float *iw, TD *gw,
                      void *scratch, int64_t B, int64_t A, int64_t G, int64_t GH, int64_t GW,
                      int64_t MH, int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s,
-                     TD *plain_sum) {
+                     TD *plain_sum, const void *plan) {
   float *part = (float *)scratch;
   const PixelTiling t = make_tiling(B, MH, MW);
   if (t.total > 0x7fffffffLL) return MCX_E_SHAPE;
@@ -1453,8 +1453,12 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
   // are ever in use (bilinear maps with integral rows, two of four points weighted) and to
   // launch both variants, of which one returns at once.
   const bool two_variants = m.np * (m.mode == kInterpNearest ? 1 : 4) == 4;
-  if (two_variants)
-    if (int rc = launch_pair_mask(map, iw, pair_mask, m, GH, GW, MH * MW * K, s)) return rc;
+  if (two_variants) {
+    if (plan)  // flag word 4 of a plan built for this map (see mfma_scatter_plan_build)
+      pair_mask = (int *)const_cast<void *>(plan) + GH * GW * K + 4;
+    else if (int rc = launch_pair_mask(map, iw, pair_mask, m, GH, GW, MH * MW * K, s))
+      return rc;
+  }
 #define MCX_LAUNCH_NA(NCORN, NP, CL, NA, MASK, LEAD)                                             \
   hipLaunchKernelGGL((weight_grad_mfma_kernel<TD, NCORN, NP, CL, NA>), grid, dim3(kThreads), 0,  \
                      s, plain, gath, map, iw, part, (int)A, (int)G, (int)GH, (int)GW, (int)MH,   \
@@ -1695,7 +1699,7 @@ ScatterScratch scatter_scratch(int64_t B, int64_t S, int64_t D, int64_t K, int64
     sc.wpt = off;
     off += align256((size_t)(K * round_up(S, kGC) * round_up(D, kOT)) * 4);
     sc.cnt = off;  // counters, the overflow flag and list length; cleared with tmap
-    off += align256((size_t)(cells + 4) * 4);
+    off += align256((size_t)(cells + 8) * 4);
     sc.tmap = off;  // [cell][slot] (source pixel index as bits, weight)
     off += align256((size_t)cells * kTransSlots * 2 * 4);
     sc.tmap2 = off;
@@ -1714,7 +1718,62 @@ ScatterScratch scatter_scratch(int64_t B, int64_t S, int64_t D, int64_t K, int64
   return sc;
 }
 
+// Counters, flags, slots and overflow list of the transposed map of `map`, into the scratch
+// (or plan) region that starts at `cnt`.
+int build_transposed_map(const ScatterScratch &sc, const float *map, const float *iw, int *cnt,
+                         const ModeArgs &m, int64_t DH, int64_t DW, int64_t MH, int64_t MW,
+                         int64_t K, hipStream_t s) {
+  char *region = (char *)cnt - sc.cnt;
+  float2 *tmap = (float2 *)(region + sc.tmap);
+  float2 *tmap2 = sc.two_level ? (float2 *)(region + sc.tmap2) : nullptr;
+  OverflowEntry *ovf = (OverflowEntry *)(region + sc.ovf);
+  int *flag = cnt + DH * DW * K;
+  if (int rc = fill_f32((float *)cnt, (int64_t)((sc.ovf - sc.cnt) / 4), 0.f, s)) return rc;
+  const int64_t entries = MH * MW * K;
+  const unsigned blocks = (unsigned)((entries + 255) / 256);
+  if (m.mode == kInterpNearest)
+    hipLaunchKernelGGL(build_transposed_map_kernel<1>, dim3(blocks), dim3(256), 0, s, map, iw, cnt,
+                       tmap, tmap2, flag, ovf, (int)sc.ovf_cap, m.np, m.weighted, m.wrap, (int)DH,
+                       (int)DW, (int)MW, (int)K, entries);
+  else
+    hipLaunchKernelGGL(build_transposed_map_kernel<4>, dim3(blocks), dim3(256), 0, s, map, iw, cnt,
+                       tmap, tmap2, flag, ovf, (int)sc.ovf_cap, m.np, m.weighted, m.wrap, (int)DH,
+                       (int)DW, (int)MW, (int)K, entries);
+  MCX_HIP_CHECK_LAUNCH();
+  return 0;
+}
+
 }  // namespace
+
+// ---- plan: the transposed map of one sample map, kept by the caller across calls ----------
+// Layout: the scratch region [cnt, stage) of mfma_product_scatter (counters, eight flag words,
+// slots, second-level slots, overflow list); flag word 4 holds the pair mask of the map itself,
+// for the weight gradient.  Depends on the map, its interpolation and the two image sizes only.
+size_t mfma_scatter_plan_bytes(int64_t DH, int64_t DW, int64_t MH, int64_t MW, int64_t K,
+                               int64_t P) {
+  const ScatterScratch sc = scatter_scratch(1, 1, 1, K, DH, DW, 4, MH, MW, P);
+  return sc.transposed_path ? sc.stage - sc.cnt : 0;
+}
+
+int mfma_scatter_plan_build(const float *map, const float *iw, void *plan, int64_t DH, int64_t DW,
+                            int64_t MH, int64_t MW, int64_t K, int64_t P, int interp,
+                            hipStream_t s) {
+  const ScatterScratch sc = scatter_scratch(1, 1, 1, K, DH, DW, 4, MH, MW, P);
+  if (!sc.transposed_path) return MCX_E_SHAPE;
+  const ModeArgs m = mode_args(interp, P);
+  int *cnt = (int *)plan;
+  const int64_t cells = DH * DW * K;
+  int *flag = cnt + cells;
+  if (int rc = build_transposed_map(sc, map, iw, cnt, m, DH, DW, MH, MW, K, s)) return rc;
+  hipLaunchKernelGGL(after_transposed_map_kernel,
+                     dim3((unsigned)std::min<int64_t>((cells + 255) / 256, 4096)), dim3(256), 0, s,
+                     cnt, cells, flag + 2, sc.two_level ? 1 : 0, (float *)nullptr, (int64_t)0,
+                     flag);
+  MCX_HIP_CHECK_LAUNCH();
+  if (m.np * (m.mode == kInterpNearest ? 1 : 4) == 4)
+    return launch_pair_mask(map, iw, flag + 4, m, DH, DW, MH * MW * K, s, true);
+  return 0;
+}
 
 size_t mfma_product_scatter_bytes(int64_t B, int64_t S, int64_t D, int64_t K, int64_t DH,
                                   int64_t DW, size_t elem, int64_t MH, int64_t MW, int64_t P) {
@@ -1727,9 +1786,12 @@ template <typename TD>
 int mfma_product_scatter(const TD *src, const float *map, const float *iw, const TD *w,
                          const TD *bias, TD *dst, void *scratch, int64_t B, int64_t S, int64_t D,
                          int64_t DH, int64_t DW, int64_t MH, int64_t MW, int64_t K, int64_t P,
-                         int interp, hipStream_t s) {
+                         int interp, hipStream_t s, const void *plan) {
   const ScatterScratch sc = scatter_scratch(B, S, D, K, DH, DW, sizeof(TD), MH, MW, P);
   char *base = (char *)scratch;
+  // a plan is the transposed map of this very map, built earlier by mfma_scatter_plan_build:
+  // the part of the scratch from the counters up to the staging area, ready to use
+  char *pbase = plan ? (char *)const_cast<void *>(plan) - sc.cnt : base;
   float *wq = (float *)(base + sc.wq);
   const int Spad = (int)round_up(S, kScSC), dchunks = (int)((D + kScDC - 1) / kScDC);
   const ModeArgs m = mode_args(interp, P);
@@ -1737,27 +1799,17 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
 
   if (sc.transposed_path) {
     // build the transposed map, then try the atomic-free gather form first
-    int *cnt = (int *)(base + sc.cnt);
-    float2 *tmap = (float2 *)(base + sc.tmap);
-    float2 *tmap2 = sc.two_level ? (float2 *)(base + sc.tmap2) : nullptr;
+    int *cnt = (int *)(pbase + sc.cnt);
+    float2 *tmap = (float2 *)(pbase + sc.tmap);
+    float2 *tmap2 = sc.two_level ? (float2 *)(pbase + sc.tmap2) : nullptr;
     float *wpt = (float *)(base + sc.wpt);
     const int64_t cells = DH * DW * K;
     int *flag = cnt + cells;
     gate = flag;
-    if (int rc = fill_f32((float *)cnt, (int64_t)((sc.ovf - sc.cnt) / 4), 0.f, s)) return rc;
-    OverflowEntry *ovf = (OverflowEntry *)(base + sc.ovf);
+    OverflowEntry *ovf = (OverflowEntry *)(pbase + sc.ovf);
     TD *stage = MH == 1 ? (TD *)(base + sc.stage) : nullptr;
-    const int64_t entries = MH * MW * K;
-    const unsigned blocks = (unsigned)((entries + 255) / 256);
-    if (m.mode == kInterpNearest)
-      hipLaunchKernelGGL(build_transposed_map_kernel<1>, dim3(blocks), dim3(256), 0, s, map, iw,
-                         cnt, tmap, tmap2, flag, ovf, (int)sc.ovf_cap, m.np, m.weighted, m.wrap,
-                         (int)DH, (int)DW, (int)MW, (int)K, entries);
-    else
-      hipLaunchKernelGGL(build_transposed_map_kernel<4>, dim3(blocks), dim3(256), 0, s, map, iw,
-                         cnt, tmap, tmap2, flag, ovf, (int)sc.ovf_cap, m.np, m.weighted, m.wrap,
-                         (int)DH, (int)DW, (int)MW, (int)K, entries);
-    MCX_HIP_CHECK_LAUNCH();
+    if (!plan)
+      if (int rc = build_transposed_map(sc, map, iw, cnt, m, DH, DW, MH, MW, K, s)) return rc;
     if (int rc = launch_pack_weights<TD>(w, wpt, D, S, K, 1, s)) return rc;
     // What did not fit the four slots of its cell is accumulated with float atomics into a
     // channel-last fp32 image (cleared only when there is anything to add), which the
@@ -1767,12 +1819,12 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
                     MH * MW * Spad16 * (int64_t)sizeof(TD) <= 0xffffffffLL;
     float *img = (float *)(base + sc.acc32);
     const int64_t total_img = B * DH * DW * round_up(D, kOT);
-    // flag[2]: at least 4 iff some cell holds more than two entries
+    // flag[2]: at least 4 iff some cell holds more than two entries (a plan has it already)
     hipLaunchKernelGGL(after_transposed_map_kernel,
                        dim3((unsigned)std::min<int64_t>(
                            std::max((total_img + 1023) / 1024, (cells + 255) / 256), 4096)),
-                       dim3(256), 0, s, cnt, cells, flag + 2, sc.two_level ? 1 : 0, img, total_img,
-                       flag);
+                       dim3(256), 0, s, cnt, plan ? (int64_t)0 : cells, flag + 2,
+                       sc.two_level ? 1 : 0, img, total_img, flag);
     MCX_HIP_CHECK_LAUNCH();
     if (cl) {  // the overflow pass reads the channel-last copy before the gather would make it
       dim3 tg((unsigned)((MH * MW + 63) / 64), (unsigned)((Spad16 + 63) / 64), (unsigned)B);
@@ -1892,11 +1944,12 @@ int mfma_bias_grad(const TD *g, TD *gb, void *scratch, int64_t B, int64_t C, int
                                        hipStream_t);                                              \
   template int mfma_weight_grad<TD>(const TD *, const TD *, const float *, const float *, TD *,   \
                                     void *, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, \
-                                    int64_t, int64_t, int64_t, int, hipStream_t, TD *);           \
+                                    int64_t, int64_t, int64_t, int, hipStream_t, TD *,            \
+                                    const void *);                                                \
   template int mfma_product_scatter<TD>(const TD *, const float *, const float *, const TD *,     \
                                         const TD *, TD *, void *, int64_t, int64_t, int64_t,      \
                                         int64_t, int64_t, int64_t, int64_t, int64_t, int64_t,     \
-                                        int, hipStream_t);                                        \
+                                        int, hipStream_t, const void *);                          \
   template int mfma_bias_grad<TD>(const TD *, TD *, void *, int64_t, int64_t, int64_t,            \
                                   hipStream_t);
 MCX_INSTANTIATE_TD(float)

@@ -326,6 +326,77 @@ def test_conv_bf16_latitude_map_uses_both_backward_paths(device):
         assert rel_err(a.float(), r) < 2e-2, nm
 
 
+# ------------------------------------------------------------------ map plans
+@pytest.mark.parametrize("case", ["latitude_fp32", "random_fp32", "mesh_bf16"])
+def test_conv_backward_with_map_plan(case, device):
+    """A plan built once from the map (conv_map_plan) replaces the per-call build of the
+    transposed map and of the pair masks: same gradients as without it, and as the oracle."""
+    g = torch.Generator().manual_seed(900)
+    if case == "mesh_bf16":
+        B, Ci, Co, V, K, P = 2, 32, 48, 1500, 7, 4
+        smap, iw = synthetic.mesh_weighted_map(V, K, P, seed=9)
+        shape_in, shape_out, interp, dtype, tol = (B, Ci, 1, V), (B, Co, 1, V), 0, torch.bfloat16, 2e-2
+    else:
+        B, Ci, Co, H, W, K = 2, 24, 40, 24, 48, 9
+        iw = None
+        if case == "latitude_fp32":
+            smap = synthetic.latitude_map(H, W, 1)
+        else:
+            smap, _ = helpers.random_map(g, H, W, K, 0, H, W, torch.float32)
+        shape_in, shape_out, interp, dtype, tol = (B, Ci, H, W), (B, Co, H, W), 1, torch.float32, 1e-5
+    x = torch.randn(shape_in, generator=g).to(dtype)
+    gy = torch.randn(shape_out, generator=g).to(dtype)
+    w = (torch.randn(Co, Ci, K, generator=g) / 8).to(dtype)
+    b = torch.randn(Co, generator=g).to(dtype)
+    xd, sd, iwd, wd_, bd, gyd = dev(x, smap, iw, w, b, gy)
+    plan = _C.conv_map_plan(sd, iwd, shape_in[2], shape_in[3], interp, dtype)
+    assert plan is not None and plan.is_cuda
+    if iw is None:
+        g_o = O.mapped_conv_backward(gy.float(), smap, x.float(), w.float(), b.float(), K, interp)
+        plain = _C.mapped_conv_backward(gyd, sd, xd, wd_, bd, K, interp)
+        for _ in range(2):  # a plan is only read: it serves any number of calls
+            planned = _C.mapped_conv_backward(gyd, sd, xd, wd_, bd, K, interp, plan=plan)
+    else:
+        g_o = O.weighted_mapped_conv_backward(gy.float(), smap, iw, x.float(), w.float(),
+                                              b.float(), K, interp)
+        plain = _C.weighted_mapped_conv_backward(gyd, sd, iwd, xd, wd_, bd, K, interp)
+        for _ in range(2):
+            planned = _C.weighted_mapped_conv_backward(gyd, sd, iwd, xd, wd_, bd, K, interp,
+                                                       plan=plan)
+    for a, p_, r, nm in zip(planned, plain, g_o, ("grad_input", "grad_weight", "grad_bias")):
+        assert rel_err(a.float(), r) < tol, nm
+        assert rel_err(a.float(), p_.float()) < tol, nm
+
+
+def test_map_plan_cache_follows_in_place_changes(device):
+    """With the cache on, the second backward reuses the plan of the first; changing the map
+    in place bumps its version counter and the plan is rebuilt."""
+    g = torch.Generator().manual_seed(901)
+    B, C, H, W, K = 1, 16, 16, 32, 9
+    x, gy = torch.randn(B, C, H, W, generator=g), torch.randn(B, C, H, W, generator=g)
+    w, b = torch.randn(C, C, K, generator=g) / 8, torch.randn(C, generator=g)
+    smap = synthetic.latitude_map(H, W, 1)
+    xd, sd, wd_, bd, gyd = dev(x, smap, w, b, gy)
+    _C.enable_map_plan_cache(True)
+    try:
+        for _ in range(2):
+            got = _C.mapped_conv_backward(gyd, sd, xd, wd_, bd, K, 1)
+        assert len(_C.map_plan_cache) == 1
+        ref = O.mapped_conv_backward(gy, smap, x, w, b, K, 1)
+        for a, r in zip(got, ref):
+            assert rel_err(a, r) < 1e-5
+        sd[..., 0] += 0.25  # in place: same storage, new version
+        smap2 = sd.cpu()
+        got = _C.mapped_conv_backward(gyd, sd, xd, wd_, bd, K, 1)
+        assert len(_C.map_plan_cache) == 2
+        ref = O.mapped_conv_backward(gy, smap2, x, w, b, K, 1)
+        for a, r in zip(got, ref):
+            assert rel_err(a, r) < 1e-5
+    finally:
+        _C.enable_map_plan_cache(False)
+    assert _C.map_plan_cache is None
+
+
 # ------------------------------------------------- BASELINE configs 3, 4, 5 (scaled)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_config3_weighted_mesh_conv(dtype, device):
