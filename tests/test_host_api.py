@@ -45,6 +45,19 @@ def test_rejected_arguments_return_codes_without_a_gpu():
     assert lib.mcx_resample_from_map(1, 1, None, 1, 0, 1, 4, 4, 4, 4, 0, 1, 0, None) == -2
     assert lib.mcx_resample_from_map(1, 1, None, 1, 1, 1, 4, 4, 4, 4, 0, 1, 7, None) == -1
     assert lib.mcx_knn(1, 1, 1, 1, 1, 3, 10, 10, 65, 0, None) == -2
+    # map builders: NULL output, a spherical grid of one row (divides by H - 1), unknown projection
+    assert lib.mcx_projection_map(None, 8, 16, 3, 3, 1, 1, 1, None) == -3
+    assert lib.mcx_projection_map(1, 1, 16, 3, 3, 1, 1, 1, None) == -2
+    assert lib.mcx_projection_map(1, 8, 16, 3, 3, 9, 1, 1, None) == -2
+    assert lib.mcx_cube2rect(1, 1, 3, 8, 16, 32, 1, 2, None) == -1  # no bf16 cube2rect
+    # map plans: sized for the matrix-core paths only; too small a buffer is refused
+    need = lib.mcx_conv_plan_bytes(8, 8, 8, 8, 9, 0, 0)
+    assert need > 0 and lib.mcx_conv_plan_bytes(8, 8, 8, 8, 9, 0, 1) == 0
+    assert lib.mcx_conv_plan_build(1, None, 1, need - 1, 8, 8, 8, 8, 9, 0, 1, 0, None) == -4
+    assert lib.mcx_conv_plan_build(1, None, None, need, 8, 8, 8, 8, 9, 0, 1, 0, None) == -3
+    assert lib.mcx_conv_plan_build(1, None, 1, need, 8, 8, 8, 8, 9, 0, 1, 1, None) == -1
+    assert lib.mcx_conv_backward_planned(1, 1, None, 1, 1, 1, 1, 1, 1, 1 << 30, 1, need - 1, 1, 4,
+                                         4, 8, 8, 8, 8, 9, 0, 1, 0, None) == -4
 
 
 def test_layer_api_and_parameter_shapes():
