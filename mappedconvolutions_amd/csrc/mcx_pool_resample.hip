@@ -348,14 +348,69 @@ __global__ __launch_bounds__(kThreads) void scan_sums_kernel(uint32_t *__restric
 // at the same step.  Lists longer than kSortMax stay as filled.
 constexpr uint32_t kSortMax = 512;
 
+// Batcher's odd-even merge sort for kNetN keys as a list of compare-exchange pairs, made at
+// compile time so that the unrolled network indexes registers statically.
+constexpr int kNetN = 32;
+struct SortNetwork {
+  int n;
+  unsigned char a[256], b[256];
+};
+constexpr SortNetwork make_network() {
+  SortNetwork net{};
+  for (int p = 1; p < kNetN; p *= 2)
+    for (int k = p; k >= 1; k /= 2)
+      for (int j = k % p; j + k < kNetN; j += 2 * k)
+        for (int i = 0; i < k && i + j + k < kNetN; i++)
+          if ((i + j) / (2 * p) == (i + j + k) / (2 * p)) {
+            net.a[net.n] = (unsigned char)(i + j);
+            net.b[net.n] = (unsigned char)(i + j + k);
+            net.n++;
+          }
+  return net;
+}
+constexpr SortNetwork kNet = make_network();
+
 template <typename T>
 __global__ __launch_bounds__(kThreads) void sort_entries_kernel(
     const uint32_t *__restrict__ local, const uint32_t *__restrict__ bsum,
     uint32_t *__restrict__ e_src, T *__restrict__ e_wt, int ndst) {
   const int p = blockIdx.x * kThreads + threadIdx.x;
-  if (p >= ndst) return;
-  const uint32_t start = local[p] + bsum[p / kScanBlock];
-  const uint32_t end = local[p + 1] + bsum[(p + 1) / kScanBlock];
+  const bool live = p < ndst;
+  const uint32_t start = live ? local[p] + bsum[p / kScanBlock] : 0u;
+  const uint32_t end = live ? local[p + 1] + bsum[(p + 1) / kScanBlock] : 0u;
+  // Lists of up to kNetN entries in every lane of the wave (pooling and resampling maps):
+  // read once into registers, sorted by the network, written back.  Same order as the
+  // insertion sort below: by source, ties by weight.
+  // (a wave most of whose lists are very short is quicker with the insertion sort)
+  if (__builtin_amdgcn_ballot_w64(end - start > (uint32_t)kNetN) == 0 &&
+      __builtin_popcountll(__builtin_amdgcn_ballot_w64(end - start > 8u)) >= 32) {
+    uint32_t code[kNetN];
+    T w[kNetN];
+#pragma unroll
+    for (int u = 0; u < kNetN; u++) {
+      const bool in = start + u < end;
+      code[u] = in ? e_src[start + u] : 0xffffffffu;  // padding sorts to the end
+      w[u] = in ? e_wt[start + u] : T(0);
+    }
+#pragma unroll
+    for (int c = 0; c < kNet.n; c++) {
+      const int ia = kNet.a[c], ib = kNet.b[c];
+      const bool swap = code[ia] > code[ib] || (code[ia] == code[ib] && w[ia] > w[ib]);
+      const uint32_t ca = swap ? code[ib] : code[ia], cb = swap ? code[ia] : code[ib];
+      const T wa = swap ? w[ib] : w[ia], wb = swap ? w[ia] : w[ib];
+      code[ia] = ca; code[ib] = cb;
+      w[ia] = wa; w[ib] = wb;
+    }
+#pragma unroll
+    for (int u = 0; u < kNetN; u++) {
+      if (start + u < end) {
+        e_src[start + u] = code[u];
+        e_wt[start + u] = w[u];
+      }
+    }
+    return;
+  }
+  if (!live) return;
   if (end - start > kSortMax) return;
   for (uint32_t i = start + 1; i < end; i++) {
     const uint32_t code = e_src[i];
