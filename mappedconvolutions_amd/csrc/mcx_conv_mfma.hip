@@ -157,8 +157,8 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
   constexpr int TG = kTapCache / NE > 0 ? kTapCache / NE : 1;  // taps cached in LDS at a time
   constexpr bool kBf16 = sizeof(TD) == 2;
   __shared__ __attribute__((aligned(16))) OperandTiles<TD> T;
-  __shared__ __attribute__((aligned(16))) unsigned TapOff[TG][kTilePx][NE];
-  __shared__ __attribute__((aligned(16))) float TapWt[TG][kTilePx][NE];
+  __shared__ __attribute__((aligned(16))) unsigned TapOff[TG][kTilePx][NA];
+  __shared__ __attribute__((aligned(16))) float TapWt[TG][kTilePx][NA];
   // Bit e of TapMask[kl][h]: some pixel of the half-tile resolved by wave pair h has a
   // nonzero weight in pair e of tap kl.  Pairs that are zero across the whole tile
   // (bilinear corners of integral coordinates, unused slots) are neither loaded nor
