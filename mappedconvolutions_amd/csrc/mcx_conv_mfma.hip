@@ -154,7 +154,10 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
   constexpr int NE = NP * NCORN;         // (offset, weight) pairs per pixel and tap
   static_assert(NA >= 1 && NA <= NE, "NA counts leading pairs");
   constexpr bool kMasked = NA == NE;
-  constexpr int TG = kTapCache / NE > 0 ? kTapCache / NE : 1;  // taps cached in LDS at a time
+  // taps cached in LDS at a time: 12 pairs per pixel, or 6 where that leaves room for a
+  // fifth workgroup on the CU
+  constexpr int kPairs = NA <= 2 ? kTapCache / 2 : kTapCache;
+  constexpr int TG = NA <= 2 ? kPairs / NA : (kTapCache / NE > 0 ? kTapCache / NE : 1);
   constexpr bool kBf16 = sizeof(TD) == 2;
   __shared__ __attribute__((aligned(16))) OperandTiles<TD> T;
   __shared__ __attribute__((aligned(16))) unsigned TapOff[TG][kTilePx][NA];
