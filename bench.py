@@ -34,9 +34,9 @@ GEMM_FLOP = 2.0 * B * H * W * CO * CI * K  # one of the three products
 # count); profiles/conv_fwd_bwd_headline_hbm_traffic.txt holds the runs.  Counters cannot be read
 # from inside the process, so the figures are the recorded ones; other workloads report null.
 MEASURED_TRAFFIC_BYTES = {
-    "conv_forward": 783.9e6 + 268.4e6,
-    "conv_backward_input": 1411.8e6 + 268.4e6,
-    "conv_backward_weight": 1531.4e6 + 92.5e6,
+    "conv_forward": 906.1e6 + 268.4e6,
+    "conv_backward_input": 1432.5e6 + 268.4e6,
+    "conv_backward_weight": 1530.3e6 + 92.0e6,
 }
 KERNEL_OF = {
     "conv_forward": "gather_product_mfma_kernel<float,4,1,1,false,2>",
