@@ -497,7 +497,7 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
   // The plain tile is only needed until each wave has copied its rows into registers;
   // the same LDS then holds the tile's resolved taps (offsets, then weights).
   constexpr int kPtFloats = kWgA * kLdPx;
-  constexpr int kTapFloats = 2 * kWgKT * kTilePx * NE;
+  constexpr int kTapFloats = 2 * kWgKT * kTilePx * NA;
   constexpr bool kCacheTaps = kTapFloats <= kPtFloats + 1024;
   __shared__ __attribute__((aligned(16))) float PtMem[kCacheTaps && kTapFloats > kPtFloats ? kTapFloats : kPtFloats];
   __shared__ __attribute__((aligned(16))) float S[2][kGC][kLdPx];
@@ -509,9 +509,11 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
   constexpr int kLdPxB = kTilePx + 8;
   uint16_t(*PtB)[kLdPxB] = reinterpret_cast<uint16_t(*)[kLdPxB]>(PtMem);
   uint16_t(*SB)[kGC][kLdPxB] = reinterpret_cast<uint16_t(*)[kGC][kLdPxB]>(&S[0][0][0]);
-  unsigned(*TapOff)[kTilePx][NE] = reinterpret_cast<unsigned(*)[kTilePx][NE]>(PtMem);
-  float(*TapWt)[kTilePx][NE] =
-      reinterpret_cast<float(*)[kTilePx][NE]>(PtMem + kWgKT * kTilePx * NE);
+  // (NA pairs per pixel: with two, a lane's offsets are one 8-byte word and the lanes of a
+  // wave read consecutive words)
+  unsigned(*TapOff)[kTilePx][NA] = reinterpret_cast<unsigned(*)[kTilePx][NA]>(PtMem);
+  float(*TapWt)[kTilePx][NA] =
+      reinterpret_cast<float(*)[kTilePx][NA]>(PtMem + kWgKT * kTilePx * NA);
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l15 = lane & 15, lq = lane >> 4;
@@ -736,7 +738,7 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
         float w_[NE];
         resolve_tap(k_base + k, o, w_);
 #pragma unroll
-        for (int i = 0; i < NE; i++) {
+        for (int i = 0; i < NA; i++) {
           TapOff[k][p][i] = o[i];
           TapWt[k][p][i] = w_[i];
         }
