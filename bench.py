@@ -36,7 +36,7 @@ GEMM_FLOP = 2.0 * B * H * W * CO * CI * K  # one of the three products
 MEASURED_TRAFFIC_BYTES = {
     "conv_forward": 906.1e6 + 268.4e6,
     "conv_backward_input": 1432.5e6 + 268.4e6,
-    "conv_backward_weight": 1530.3e6 + 92.0e6,
+    "conv_backward_weight": 1535.9e6 + 89.1e6,
 }
 KERNEL_OF = {
     "conv_forward": "gather_product_mfma_kernel<float,4,1,1,false,2>",
