@@ -426,16 +426,22 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
 // (convolution: plain = grad_output, gath = input; transposed: plain = input,
 // gath = grad_output).  The reduction dimension is the pixel axis, so a workgroup
 // walks a range of pixel tiles and keeps its slice of gW in MFMA accumulators:
-// 64 plain channels x 32 gathered channels x up to 9 taps.  Per tile the plain
-// tile P[64][128] is staged in LDS once and each wave keeps its 16 rows as MFMA A
-// operands in registers; per (tap, 16-channel block) the gathered samples go to
+// 64 plain channels x 32 gathered channels x up to 9 taps (fp32; bf16 storage: 128 x 16 x 9).
+// Per tile the plain tile P[64][128] is staged in LDS once and each wave keeps its 16 rows
+// as MFMA A operands in registers; per (tap, 16-channel block) the gathered samples go to
 // LDS as S[16][128] (same gather as the forward kernel) and every wave issues 32
-// v_mfma_f32_16x16x4_f32.  Each workgroup writes its partial gW to scratch; a
+// v_mfma_f32_16x16x4_f32 (bf16: 8 v_mfma_f32_16x16x32_bf16).  Each workgroup writes its partial gW to scratch; a
 // second kernel sums the partials in a fixed order (deterministic result).
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-constexpr int kWgA = 64;            // plain channels per workgroup
-constexpr int kWgCB = 2;            // 16-channel blocks of gathered channels per workgroup
+// Plain channels and 16-channel blocks of gathered channels per workgroup.  With bf16 storage
+// the gather bounds the kernel, not the MFMAs: a workgroup then takes 128 plain channels (two
+// 16-row blocks per wave) against one block of gathered channels, so that a convolution of up
+// to 128 output channels gathers every sample once.
+template <typename TD>
+constexpr int wg_plain_channels() { return sizeof(TD) == 2 ? 128 : 64; }
+template <typename TD>
+constexpr int wg_gathered_blocks() { return sizeof(TD) == 2 ? 1 : 2; }
 constexpr int kWgKT = 9;            // taps per pass (accumulators in registers)
 constexpr int kLdPx = kTilePx + 4;  // LDS row stride (floats)
 
@@ -496,19 +502,22 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
   if (pair_mask && (((unsigned)*pair_mask < (1u << 2)) != (run_if_leading != 0))) return;
   // The plain tile is only needed until each wave has copied its rows into registers;
   // the same LDS then holds the tile's resolved taps (offsets, then weights).
-  constexpr int kPtFloats = kWgA * kLdPx;
-  constexpr int kTapFloats = 2 * kWgKT * kTilePx * NA;
-  constexpr bool kCacheTaps = kTapFloats <= kPtFloats + 1024;
-  __shared__ __attribute__((aligned(16))) float PtMem[kCacheTaps && kTapFloats > kPtFloats ? kTapFloats : kPtFloats];
-  __shared__ __attribute__((aligned(16))) float S[2][kGC][kLdPx];
-  float(*Pt)[kLdPx] = reinterpret_cast<float(*)[kLdPx]>(PtMem);
   // bf16 storage: both tiles hold bf16 (row stride kLdPxB keeps 16-byte row reads of 16
   // different rows on different banks) and feed v_mfma_f32_16x16x32_bf16, whose lanes take
   // 8 consecutive pixels of their row.
   constexpr bool kBf16 = sizeof(TD) == 2;
   constexpr int kLdPxB = kTilePx + 8;
+  constexpr int kWgA = wg_plain_channels<TD>(), kWgCB = wg_gathered_blocks<TD>();
+  constexpr int MB = kWgA / 64;  // 16-row blocks of plain channels per wave
+  constexpr int kPtFloats = kBf16 ? kWgA * kLdPxB / 2 : kWgA * kLdPx;
+  constexpr int kTapFloats = 2 * kWgKT * kTilePx * NA;
+  constexpr bool kCacheTaps = kTapFloats <= kPtFloats + 1024;
+  __shared__ __attribute__((aligned(16))) float PtMem[kCacheTaps && kTapFloats > kPtFloats ? kTapFloats : kPtFloats];
+  __shared__ __attribute__((aligned(16))) float SMem[kBf16 ? kGC * kLdPxB : 2 * kGC * kLdPx];
+  float(*Pt)[kLdPx] = reinterpret_cast<float(*)[kLdPx]>(PtMem);
+  float(*S)[kGC][kLdPx] = reinterpret_cast<float(*)[kGC][kLdPx]>(SMem);
   uint16_t(*PtB)[kLdPxB] = reinterpret_cast<uint16_t(*)[kLdPxB]>(PtMem);
-  uint16_t(*SB)[kGC][kLdPxB] = reinterpret_cast<uint16_t(*)[kGC][kLdPxB]>(&S[0][0][0]);
+  uint16_t(*SB)[kGC][kLdPxB] = reinterpret_cast<uint16_t(*)[kGC][kLdPxB]>(SMem);
   // (NA pairs per pixel: with two, a lane's offsets are one 8-byte word and the lanes of a
   // wave read consecutive words)
   unsigned(*TapOff)[kTilePx][NA] = reinterpret_cast<unsigned(*)[kTilePx][NA]>(PtMem);
@@ -541,16 +550,20 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
   const bool vec_ok = (MW & (16 / (int)sizeof(TD) - 1)) == 0 &&
                       (reinterpret_cast<uintptr_t>(plain) & 15) == 0;
 
-  floatx4 acc[kWgKT][kWgCB];
+  floatx4 acc[kWgKT][kWgCB][MB];
 #pragma unroll
   for (int k = 0; k < kWgKT; k++)
 #pragma unroll
-    for (int cb = 0; cb < kWgCB; cb++) acc[k][cb] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int cb = 0; cb < kWgCB; cb++)
+#pragma unroll
+      for (int mb = 0; mb < MB; mb++) acc[k][cb][mb] = floatx4{0.f, 0.f, 0.f, 0.f};
   // Sum of the plain operand over pixels (the bias gradient of a convolution), taken from
   // the staged tiles by the workgroups of the first channel group and tap pass: thread
-  // (row tid/4, quarter tid%4) adds 32 pixels of its row per tile.
+  // (row tid/4 of each 64, quarter tid%4) adds 32 pixels of its row per tile.
   const bool sum_plain = plain_sum_part != nullptr && cg == 0 && blockIdx.z == 0;
-  float plain_sum = 0.f;
+  float plain_sum[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; mb++) plain_sum[mb] = 0.f;
 
   for (int tile = t_begin; tile < t_end; ++tile) {
     const int b = tile / tiles_per_img;
@@ -597,12 +610,15 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
     }
     __syncthreads();
     float areg[kBf16 ? 1 : 32];
-    bf16x8 aregb[kBf16 ? 4 : 1];
+    bf16x8 aregb[MB][kBf16 ? 4 : 1];
     if constexpr (kBf16) {
 #pragma unroll
-      for (int s = 0; s < 4; s++)
-        aregb[s] = __builtin_bit_cast(
-            bf16x8, *reinterpret_cast<const uint4 *>(&PtB[wave * 16 + l15][32 * s + 8 * lq]));
+      for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int s = 0; s < 4; s++)
+          aregb[mb][s] = __builtin_bit_cast(
+              bf16x8, *reinterpret_cast<const uint4 *>(
+                          &PtB[(wave * MB + mb) * 16 + l15][32 * s + 8 * lq]));
     } else {
 #pragma unroll
       for (int s4 = 0; s4 < 8; s4++) {
@@ -618,15 +634,21 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
     if (sum_plain) {
       float t = 0.f;
       if constexpr (kBf16) {
-        const uint4 *row = reinterpret_cast<const uint4 *>(&PtB[tid >> 2][(tid & 3) * 32]);
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-          const uint4 q = row[r];
-          const unsigned w4[4] = {q.x, q.y, q.z, q.w};
+        for (int mb = 0; mb < MB; mb++) {
+          const uint4 *row =
+              reinterpret_cast<const uint4 *>(&PtB[64 * mb + (tid >> 2)][(tid & 3) * 32]);
+          t = 0.f;
 #pragma unroll
-          for (int j = 0; j < 4; j++)
-            t += __builtin_bit_cast(float, w4[j] << 16) +
-                 __builtin_bit_cast(float, w4[j] & 0xffff0000u);
+          for (int r = 0; r < 4; r++) {
+            const uint4 q = row[r];
+            const unsigned w4[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+              t += __builtin_bit_cast(float, w4[j] << 16) +
+                   __builtin_bit_cast(float, w4[j] & 0xffff0000u);
+          }
+          if (mb + 1 < MB) plain_sum[mb] += t;
         }
       } else {
         const float4 *row = reinterpret_cast<const float4 *>(&Pt[tid >> 2][(tid & 3) * 32]);
@@ -636,7 +658,7 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
           t += (q.x + q.y) + (q.z + q.w);
         }
       }
-      plain_sum += t;
+      plain_sum[MB - 1] += t;
     }
 
     const int gi = i0 + (p >> tw_shift), gj = j0 + (p & tw_mask);
@@ -771,17 +793,19 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
             for (int s = 0; s < 4; s++) {
               const bf16x8 bq = __builtin_bit_cast(
                   bf16x8, *reinterpret_cast<const uint4 *>(&SB[buf][l15][32 * s + 8 * lq]));
-              acc[k][cb] =
-                  __builtin_amdgcn_mfma_f32_16x16x32_bf16(aregb[s], bq, acc[k][cb], 0, 0, 0);
+#pragma unroll
+              for (int mb = 0; mb < MB; mb++)
+                acc[k][cb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aregb[mb][s], bq,
+                                                                         acc[k][cb][mb], 0, 0, 0);
             }
           } else
 #pragma unroll
           for (int s4 = 0; s4 < 8; s4++) {
             const float4 bq = *reinterpret_cast<const float4 *>(&S[buf][l15][16 * s4 + 4 * lq]);
-            acc[k][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[4 * s4 + 0], bq.x, acc[k][cb], 0, 0, 0);
-            acc[k][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[4 * s4 + 1], bq.y, acc[k][cb], 0, 0, 0);
-            acc[k][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[4 * s4 + 2], bq.z, acc[k][cb], 0, 0, 0);
-            acc[k][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[4 * s4 + 3], bq.w, acc[k][cb], 0, 0, 0);
+            acc[k][cb][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[4 * s4 + 0], bq.x, acc[k][cb][0], 0, 0, 0);
+            acc[k][cb][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[4 * s4 + 1], bq.y, acc[k][cb][0], 0, 0, 0);
+            acc[k][cb][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[4 * s4 + 2], bq.z, acc[k][cb][0], 0, 0, 0);
+            acc[k][cb][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[4 * s4 + 3], bq.w, acc[k][cb][0], 0, 0, 0);
           }
         }
       }
@@ -789,13 +813,17 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
   }
 
   if (sum_plain) {  // the four quarters of a row sit in neighbouring lanes
-    plain_sum += __shfl_xor(plain_sum, 1);
-    plain_sum += __shfl_xor(plain_sum, 2);
-    const int a = a0 + (tid >> 2);
-    if ((tid & 3) == 0 && a < A) plain_sum_part[(int64_t)range * A + a] = plain_sum;
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) {
+      float t = plain_sum[mb];
+      t += __shfl_xor(t, 1);
+      t += __shfl_xor(t, 2);
+      const int a = a0 + 64 * mb + (tid >> 2);
+      if ((tid & 3) == 0 && a < A) plain_sum_part[(int64_t)range * A + a] = t;
+    }
   }
   // partial gW of this workgroup: lane holds gathered channel l15 of each block and
-  // plain channels a0 + 16*wave + 4*lq + i
+  // plain channels a0 + 16*(wave*MB + mb) + 4*lq + i
   float *pr = part + (int64_t)range * A * G * K;
 #pragma unroll
   for (int k = 0; k < kWgKT; k++) {
@@ -804,10 +832,12 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
       for (int cb = 0; cb < kWgCB; cb++) {
         const int g = g_first + cb * kGC + l15;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-          const int a = a0 + wave * 16 + lq * 4 + i;
-          if (a < A && g < G) pr[((int64_t)a * G + g) * K + k_base + k] = acc[k][cb][i];
-        }
+        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            const int a = a0 + (wave * MB + mb) * 16 + lq * 4 + i;
+            if (a < A && g < G) pr[((int64_t)a * G + g) * K + k_base + k] = acc[k][cb][mb][i];
+          }
       }
     }
   }
@@ -1205,7 +1235,9 @@ inline PixelTiling make_tiling(int64_t B, int64_t H, int64_t W) {
   return t;
 }
 
+template <typename TD>
 inline int weight_grad_ranges(int64_t total_tiles, int64_t A, int64_t G, int64_t K) {
+  constexpr int kWgA = wg_plain_channels<TD>(), kWgCB = wg_gathered_blocks<TD>();
   const int64_t per_range = ((G + kWgCB * kGC - 1) / (kWgCB * kGC)) * ((A + kWgA - 1) / kWgA) *
                             ((K + kWgKT - 1) / kWgKT);
   int64_t r = std::max<int64_t>(8, (768 / per_range) / 8 * 8);  // about three workgroups per CU
@@ -1416,7 +1448,9 @@ int mfma_gather_product(const TD *src, const float *map, const float *iw, const 
 size_t mfma_weight_grad_bytes(int64_t B, int64_t A, int64_t G, int64_t MH, int64_t MW, int64_t K,
                               int64_t GH, int64_t GW) {
   const PixelTiling t = make_tiling(B, MH, MW);
-  const size_t ranges = (size_t)weight_grad_ranges(t.total, A, G, K);
+  // (sized for either storage type: the number of ranges depends on it)
+  const size_t ranges = (size_t)std::max(weight_grad_ranges<float>(t.total, A, G, K),
+                                         weight_grad_ranges<bf16_t>(t.total, A, G, K));
   size_t n = align256(ranges * (size_t)(A * G * K) * sizeof(float));
   n += align256(ranges * (size_t)A * sizeof(float));
   n += 256;  // the map's pair mask
@@ -1435,7 +1469,8 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
   const PixelTiling t = make_tiling(B, MH, MW);
   if (t.total > 0x7fffffffLL) return MCX_E_SHAPE;
   if (GH * GW * (int64_t)sizeof(TD) > 0xffffffffLL) return MCX_E_SHAPE;  // 32-bit tap offsets
-  const int ranges = weight_grad_ranges(t.total, A, G, K);
+  constexpr int kWgA = wg_plain_channels<TD>(), kWgCB = wg_gathered_blocks<TD>();
+  const int ranges = weight_grad_ranges<TD>(t.total, A, G, K);
   const int cgroups = (int)((G + kWgCB * kGC - 1) / (kWgCB * kGC));
   const int64_t Gpad = round_up(G, kGC);
   const bool cl = use_channel_last(GH, interp) &&
