@@ -52,7 +52,7 @@ int fill_zero<double>(double *p, int64_t n, hipStream_t s) { return fill_f64(p, 
 // ---- scratch sizes of the three operators -------------------------------------------
 size_t gather_product_ws(int dtype, int64_t G, int64_t O, int64_t K, int64_t P, int64_t B,
                          int64_t SH, int64_t SW) {
-  return use_mfma(dtype, P) ? mfma_gather_product_bytes(O, G, K, B, SH, SW) : 0;
+  return use_mfma(dtype, P) ? mfma_gather_product_bytes(O, G, K, B, SH, SW, (int)elem_size(dtype)) : 0;
 }
 size_t weight_grad_ws(int dtype, int64_t B, int64_t A, int64_t G, int64_t MH, int64_t MW,
                       int64_t K, int64_t P, int64_t GH, int64_t GW) {
@@ -150,7 +150,7 @@ int gather_product<float>(bool mfma, const void *src, const void *map, const voi
     return generic_gather_product<float>((const float *)src, (const float *)map,
                                          (const float *)iw, (const float *)w, (const float *)bias,
                                          (float *)y, B, G, O, SH, SW, MH * MW, K, P, interp, s);
-  if (!ws || ws_bytes < mfma_gather_product_bytes(O, G, K, B, SH, SW)) return MCX_E_WORKSPACE;
+  if (!ws || ws_bytes < mfma_gather_product_bytes(O, G, K, B, SH, SW, 4)) return MCX_E_WORKSPACE;
   return mfma_gather_product<float>((const float *)src, (const float *)map, (const float *)iw,
                                     (const float *)w, (const float *)bias, (float *)y, ws, B, G, O,
                                     SH, SW, MH, MW, K, P, interp, s);
@@ -208,7 +208,7 @@ int gather_product<bf16_t>(bool mfma, const void *src, const void *map, const vo
                            int64_t B, int64_t G, int64_t O, int64_t SH, int64_t SW, int64_t MH,
                            int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s) {
   if (!mfma) return MCX_E_DTYPE;
-  if (!ws || ws_bytes < mfma_gather_product_bytes(O, G, K, B, SH, SW)) return MCX_E_WORKSPACE;
+  if (!ws || ws_bytes < mfma_gather_product_bytes(O, G, K, B, SH, SW, 2)) return MCX_E_WORKSPACE;
   return mfma_gather_product<bf16_t>((const bf16_t *)src, (const float *)map, (const float *)iw,
                                      (const bf16_t *)w, (const bf16_t *)bias, (bf16_t *)y, ws, B,
                                      G, O, SH, SW, MH, MW, K, P, interp, s);

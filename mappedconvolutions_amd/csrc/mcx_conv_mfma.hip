@@ -119,6 +119,24 @@ __global__ __launch_bounds__(256) void to_channel_last_kernel(const TD *__restri
   }
 }
 
+// x[b][g][n] -> xt[b][g/8][n][g%8] (channels past G zero): a thread gathers the 8 channels of
+// one pixel (each of the 8 loads is contiguous across the wave) and writes them as one vector.
+template <typename TD>
+__global__ __launch_bounds__(256) void to_channel_blocks_kernel(const TD *__restrict__ x,
+                                                                TD *__restrict__ xt, int G,
+                                                                int64_t plane) {
+  const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int g8 = blockIdx.y, b = blockIdx.z;
+  if (n >= plane) return;
+  struct alignas(8 * sizeof(TD)) Block { TD c[8]; } v;
+#pragma unroll
+  for (int c = 0; c < 8; c++) {
+    const int g = g8 * 8 + c;
+    v.c[c] = g < G ? x[((int64_t)b * G + g) * plane + n] : TD{};
+  }
+  reinterpret_cast<Block *>(xt)[((int64_t)b * gridDim.y + g8) * plane + n] = v;
+}
+
 // LDS operand tiles of the gather-product kernel, double-buffered.
 template <typename TD>
 struct OperandTiles {  // fp32: samples S[chunk channel][pixel], weights Wt[chunk channel][o]
@@ -136,7 +154,10 @@ struct OperandTiles<bf16_t> {  // bf16: 16-byte groups of 8 channels, [kg][pixel
 // CL: `src` is a channel-last copy [B][SH*SW][Gpad] of the source (made by
 // to_channel_last_kernel): a sample's 8 channels are then one or two 16-byte loads from
 // one cache line instead of 8 loads from 8 lines.  Used for single-row sources (mesh
-// signals), whose maps point anywhere.
+// signals), whose maps point anywhere.  With `cl_blocked` the copy is [B][Gpad/8][SH*SW][8]
+// (made by to_channel_blocks_kernel): neighbouring pixels stay neighbours, so image-like
+// sources keep their coalescing and a sample's 8 channels are still one load; used with bf16
+// storage, where the number of load instructions bounds the kernel.
 // NA: leading (offset, weight) pairs of a tap that are loaded and added.  NA == NP * NCORN is
 // the general form, which skips the pairs a tile's mask shows to be zero across the tile.
 // NA == 2 (four-pair taps) is the branch-free form for maps that use nothing but the first
@@ -150,13 +171,13 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
     int O, int Opad, int Gpad, int SH, int SW, int OH, int OW, int K, int weighted, int wrap,
     int tiles_x, int tiles_per_img, int tw_shift, const int *__restrict__ gate, int run_if_zero,
     const float *__restrict__ addend, const int *__restrict__ pair_mask, int run_if_leading,
-    int packed_map, int accumulate) {
+    int packed_map, int accumulate, int cl_blocked) {
   constexpr int NE = NP * NCORN;         // (offset, weight) pairs per pixel and tap
   static_assert(NA >= 1 && NA <= NE, "NA counts leading pairs");
   constexpr bool kMasked = NA == NE;
   // taps cached in LDS at a time: 12 pairs per pixel, or 6 where that leaves room for a
   // fifth workgroup on the CU
-  constexpr int kPairs = NA <= 2 ? kTapCache / 2 : kTapCache;
+  constexpr int kPairs = (NA <= 2 && OG == 1) ? kTapCache / 2 : kTapCache;
   constexpr int TG = NA <= 2 ? kPairs / NA : (kTapCache / NE > 0 ? kTapCache / NE : 1);
   constexpr bool kBf16 = sizeof(TD) == 2;
   __shared__ __attribute__((aligned(16))) OperandTiles<TD> T;
@@ -219,7 +240,8 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
   auto set_chunk = [&](int c) {
     const int g0 = c * kGC + half * 8;
     if constexpr (CL) {
-      pl[0] = src_b + g0;  // the 8 channels are contiguous; offsets select the pixel row
+      // the 8 channels are contiguous; offsets select the pixel
+      pl[0] = cl_blocked ? src_b + (int64_t)(g0 >> 3) * plane * 8 : src_b + g0;
     } else if (g0 + 8 <= G) {  // all eight planes exist: one product, then additions
       const char *q = reinterpret_cast<const char *>(src_b) + (int64_t)g0 * plane_bytes;
 #pragma unroll
@@ -341,7 +363,8 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
 #pragma unroll
         for (int i = 0; i < NCORN; i++) {
           if (sp * NCORN + i >= NA) continue;
-          TapOff[kl][p][sp * NCORN + i] = CL ? t.off[i] * (unsigned)Gpad : t.off[i];
+          TapOff[kl][p][sp * NCORN + i] =
+              CL ? t.off[i] * (unsigned)(cl_blocked ? 8 : Gpad) : t.off[i];
           TapWt[kl][p][sp * NCORN + i] = t.wt[i];
           if (kMasked && __builtin_amdgcn_ballot_w64(t.wt[i] != 0.f)) m |= 1u << (sp * NCORN + i);
         }
@@ -353,6 +376,102 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
     // Units run chunk-major with the tap fastest: the source rows a 16-channel chunk
     // touches are reused by all taps of the group while they are still in cache.
     const int units = chunks * kn;
+    if constexpr (CL && kBf16) {
+      // bf16 storage, staged source: a unit is NA 16-byte loads per thread and four short
+      // MFMAs per wave, far too little work to cover the latency of the next unit's loads.
+      // The loads of kDepth units are kept in flight instead (a ring of registers; the unit
+      // loop is unrolled by kDepth so that every ring slot has a fixed register).
+      constexpr int kDepth = NA <= 2 ? 4 : NA <= 4 ? 2 : 1;
+      typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+      u32x4 ring[kDepth][NA];
+      u32x4 wring[kDepth];  // this thread's share of the unit's weights (8 * OG bytes)
+      int ki = 0, ci = 0;   // the unit whose loads are issued next
+      int ks = 0;           // tap of the unit that is staged next
+      // (issued unconditionally, past the last unit too, where it reads the last chunk
+      // again: a load that depends on a branch would make every later wait a full one)
+      auto issue_slot = [&](int d) {
+        const int cc = min(ci, chunks - 1);
+        const int g0 = cc * kGC + half * 8;
+        const char *base = reinterpret_cast<const char *>(
+            cl_blocked ? src_b + (int64_t)(g0 >> 3) * plane * 8 : src_b + g0);
+#pragma unroll
+        for (int i = 0; i < NA; i++)
+          ring[d][i] = *reinterpret_cast<const u32x4 *>(base + TapOff[ki][p][i]);
+        const char *wchunk = reinterpret_cast<const char *>(wp) +
+                             ((((int64_t)(k0 + ki) * chunks + cc) * 2 + (tid >> 7)) * Opad + o0) * 16;
+        if constexpr (OG == 1) {
+          const uint2 t2 = *reinterpret_cast<const uint2 *>(wchunk + (tid & 127) * 8);
+          wring[d] = u32x4{t2.x, t2.y, 0u, 0u};
+        } else {
+          wring[d] = *reinterpret_cast<const u32x4 *>(wchunk + (tid & 127) * 16);
+        }
+        if (++ki == kn) {
+          ki = 0;
+          ++ci;
+        }
+      };
+      auto stage_slot = [&](int d, int b) {
+        float sv[8];
+#pragma unroll
+        for (int ch = 0; ch < 8; ch++) sv[ch] = 0.f;
+#pragma unroll
+        for (int i = 0; i < NA; i++) {
+          const float wgt = TapWt[ks][p][i];
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            const unsigned w2 = ring[d][i][j];
+            sv[2 * j] = __builtin_fmaf(wgt, __builtin_bit_cast(float, w2 << 16), sv[2 * j]);
+            sv[2 * j + 1] = __builtin_fmaf(wgt, __builtin_bit_cast(float, w2 & 0xffff0000u),
+                                           sv[2 * j + 1]);
+          }
+        }
+        u32x4 q;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          q[j] = __builtin_bit_cast(
+              unsigned, __builtin_convertvector(floatx2{sv[2 * j], sv[2 * j + 1]}, bf16x2));
+        *reinterpret_cast<u32x4 *>(&T.S[b][half][p]) = q;
+        if constexpr (OG == 1)
+          reinterpret_cast<uint2 *>(&T.Wt[b][tid >> 7][0])[tid & 127] =
+              uint2{wring[d][0], wring[d][1]};
+        else
+          *reinterpret_cast<u32x4 *>(&T.Wt[b][tid >> 7][tid & 127]) = wring[d];
+        if (++ks == kn) ks = 0;
+      };
+      auto products = [&](int b) {
+        const bf16x8 bq = __builtin_bit_cast(bf16x8, T.S[b][lhi][wave * 32 + l31]);
+        bf16x8 aq[2 * OG];
+#pragma unroll
+        for (int m = 0; m < 2 * OG; m++)
+          aq[m] = __builtin_bit_cast(bf16x8, T.Wt[b][lhi][32 * m + l31]);
+#pragma unroll
+        for (int m = 0; m < 2 * OG; m++)
+          acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aq[m], bq, acc[m], 0, 0, 0);
+      };
+#pragma unroll
+      for (int d = 0; d < kDepth; d++) issue_slot(d);
+      int u = 0;
+      for (; u + kDepth <= units; u += kDepth) {  // whole rounds of the ring, branch-free
+#pragma unroll
+        for (int d = 0; d < kDepth; d++) {
+          stage_slot(d, buf);
+          __syncthreads();
+          issue_slot(d);
+          products(buf);
+          buf ^= 1;
+        }
+      }
+#pragma unroll
+      for (int d = 0; d < kDepth - 1; d++) {  // the last units, already in flight
+        if (u + d < units) {
+          stage_slot(d, buf);
+          __syncthreads();
+          products(buf);
+          buf ^= 1;
+        }
+      }
+      continue;
+    }
     load_tap(0);
     set_chunk(0);
     issue(k0, 0);
@@ -1224,10 +1343,13 @@ struct PixelTiling {
   int64_t total;
 };
 
-// 2-D pixel tiles of 128: 4 x 32 when the map has at least 4 rows, else 1 x 128.
-inline PixelTiling make_tiling(int64_t B, int64_t H, int64_t W) {
+// 2-D pixel tiles of 128: 4 x 32 when the map has at least 4 rows, else 1 x 128.  With 2-byte
+// elements and wide images the tiles are 1 x 128 as well: a wave's 64 samples of a row then
+// span 128 bytes instead of two runs of 64.
+inline PixelTiling make_tiling(int64_t B, int64_t H, int64_t W, int elem) {
   PixelTiling t;
   t.tw_shift = H >= 4 ? 5 : 7;
+  if (elem == 2 && W >= 256) t.tw_shift = 7;
   const int tw = 1 << t.tw_shift, th = kTilePx >> t.tw_shift;
   t.tiles_x = (int)((W + tw - 1) / tw);
   t.tiles_per_img = t.tiles_x * (int)((H + th - 1) / th);
@@ -1295,6 +1417,19 @@ inline ModeArgs mode_args(int interp, int64_t P) {
 inline bool use_channel_last(int64_t SH, int interp) {
   return SH == 1 && canonical_interp(interp) == kInterpNearest;
 }
+// Blocked staging ([B][Gpad/8][pixels][8]) of an image-like source: bf16 storage only.
+inline bool use_channel_blocks(int64_t SH, int interp, size_t elem) {
+  return elem == 2 && !use_channel_last(SH, interp) && SH > 1;
+}
+template <typename TD>
+int launch_channel_blocks(const TD *src, TD *stage, int64_t B, int64_t G, int64_t plane,
+                          hipStream_t s) {
+  const int64_t Gpad = round_up(G, kGC);
+  dim3 tg((unsigned)((plane + 255) / 256), (unsigned)(Gpad / 8), (unsigned)B);
+  hipLaunchKernelGGL(to_channel_blocks_kernel<TD>, tg, dim3(256), 0, s, src, stage, (int)G, plane);
+  MCX_HIP_CHECK_LAUNCH();
+  return 0;
+}
 
 // `stage`: room for the channel-last copy (B * SH * SW * Gpad elements) when
 // use_channel_last(SH, interp), unused otherwise.
@@ -1307,10 +1442,15 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
                           const int *pair_mask = nullptr, bool packed_map = false,
                           bool accumulate = false) {
   const int Opad = (int)round_up(O, kOT), Gpad = (int)round_up(G, kGC);
-  const bool cl = stage != nullptr && use_channel_last(SH, interp) &&
-                  SH * SW * Gpad * (int64_t)sizeof(TD) <= 0xffffffffLL;
+  const bool blocked = stage != nullptr && use_channel_blocks(SH, interp, sizeof(TD)) &&
+                       SH * SW * 8 * (int64_t)sizeof(TD) <= 0xffffffffLL;
+  const bool cl = blocked || (stage != nullptr && use_channel_last(SH, interp) &&
+                              SH * SW * Gpad * (int64_t)sizeof(TD) <= 0xffffffffLL);
   if (cl && staged) {
-    src = stage;  // the caller has made the channel-last copy already
+    src = stage;  // the caller has made the copy already
+  } else if (blocked) {
+    if (int rc = launch_channel_blocks<TD>(src, stage, B, G, SH * SW, s)) return rc;
+    src = stage;
   } else if (cl) {
     dim3 tg((unsigned)((SH * SW + 63) / 64), (unsigned)((Gpad + 63) / 64), (unsigned)B);
     hipLaunchKernelGGL(to_channel_last_kernel<TD>, tg, dim3(256), 0, s, src, stage, (int)G, Gpad,
@@ -1318,7 +1458,7 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
     MCX_HIP_CHECK_LAUNCH();
     src = stage;
   }
-  const PixelTiling t = make_tiling(B, OH, OW);
+  const PixelTiling t = make_tiling(B, OH, OW, (int)sizeof(TD));
   if (t.total > 0x7fffffffLL) return MCX_E_SHAPE;
   // tap offsets are 32-bit byte offsets inside a source plane
   if (SH * SW * (int64_t)sizeof(TD) > 0xffffffffLL) return MCX_E_SHAPE;
@@ -1332,7 +1472,7 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
                      dim3(kThreads), 0, s, src, map, iw, wp, bias, y, (int)G, (int)O, Opad,      \
                      Gpad, (int)SH, (int)SW, (int)OH, (int)OW, (int)K, m.weighted, m.wrap,       \
                      t.tiles_x, t.tiles_per_img, t.tw_shift, gate, run_if_zero, addend, MASK,    \
-                     LEAD, packed_map ? 1 : 0, accumulate ? 1 : 0)
+                     LEAD, packed_map ? 1 : 0, accumulate ? 1 : 0, blocked ? 1 : 0)
 #define MCX_LAUNCH_CL(NCORN, NP, OG, CL)                                      \
   if constexpr (NCORN * NP == 4) {                                            \
     if (pair_mask) {                                                          \
@@ -1345,7 +1485,7 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
     MCX_LAUNCH_NA(NCORN, NP, OG, CL, NCORN * NP, (const int *)nullptr, 0);    \
   }
 #define MCX_LAUNCH_OG(NCORN, NP, OG)           \
-  if constexpr (NCORN == 1) {                  \
+  if constexpr (NCORN == 1 || sizeof(TD) == 2) { \
     if (cl) {                                  \
       MCX_LAUNCH_CL(NCORN, NP, OG, true);      \
     } else {                                   \
@@ -1415,10 +1555,11 @@ int launch_pair_mask(const float *map, const float *iw, int *mask, const ModeArg
 // Packed weights, then (single-row sources) the channel-last copy of the source, sized
 // for 4-byte elements.
 size_t mfma_gather_product_bytes(int64_t O, int64_t G, int64_t K, int64_t B, int64_t SH,
-                                 int64_t SW) {
+                                 int64_t SW, int elem) {
   size_t n = align256((size_t)(K * round_up(G, kGC) * round_up(O, kOT)) * sizeof(float));
   n += 256;  // the map's pair mask
-  if (SH == 1) n += align256((size_t)(B * SH * SW * round_up(G, kGC)) * sizeof(float));
+  if (SH == 1 || elem == 2)
+    n += align256((size_t)(B * SH * SW * round_up(G, kGC)) * sizeof(float));
   return n;
 }
 
@@ -1431,7 +1572,8 @@ int mfma_gather_product(const TD *src, const float *map, const float *iw, const 
   float *wp = (float *)scratch;
   int *pair_mask = reinterpret_cast<int *>(
       (char *)scratch + align256((size_t)(K * round_up(G, kGC) * round_up(O, kOT)) * 4));
-  TD *stage = SH == 1 ? reinterpret_cast<TD *>((char *)pair_mask + 256) : nullptr;
+  TD *stage = (SH == 1 || sizeof(TD) == 2) ? reinterpret_cast<TD *>((char *)pair_mask + 256)
+                                           : nullptr;
   if (int rc = launch_pack_weights<TD>(w, wp, O, G, K, 0, s, pair_mask)) return rc;
   const ModeArgs m = mode_args(interp, P);
   const bool four_pairs = m.np * (m.mode == kInterpNearest ? 1 : 4) == 4;
@@ -1447,10 +1589,10 @@ int mfma_gather_product(const TD *src, const float *map, const float *iw, const 
 // (single-row gathered operands) their channel-last copy.
 size_t mfma_weight_grad_bytes(int64_t B, int64_t A, int64_t G, int64_t MH, int64_t MW, int64_t K,
                               int64_t GH, int64_t GW) {
-  const PixelTiling t = make_tiling(B, MH, MW);
-  // (sized for either storage type: the number of ranges depends on it)
-  const size_t ranges = (size_t)std::max(weight_grad_ranges<float>(t.total, A, G, K),
-                                         weight_grad_ranges<bf16_t>(t.total, A, G, K));
+  // (sized for either storage type: the tiling and the number of ranges depend on it)
+  const size_t ranges =
+      (size_t)std::max(weight_grad_ranges<float>(make_tiling(B, MH, MW, 4).total, A, G, K),
+                       weight_grad_ranges<bf16_t>(make_tiling(B, MH, MW, 2).total, A, G, K));
   size_t n = align256(ranges * (size_t)(A * G * K) * sizeof(float));
   n += align256(ranges * (size_t)A * sizeof(float));
   n += 256;  // the map's pair mask
@@ -1466,7 +1608,7 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
                      int64_t MH, int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s,
                      TD *plain_sum, const void *plan) {
   float *part = (float *)scratch;
-  const PixelTiling t = make_tiling(B, MH, MW);
+  const PixelTiling t = make_tiling(B, MH, MW, (int)sizeof(TD));
   if (t.total > 0x7fffffffLL) return MCX_E_SHAPE;
   if (GH * GW * (int64_t)sizeof(TD) > 0xffffffffLL) return MCX_E_SHAPE;  // 32-bit tap offsets
   constexpr int kWgA = wg_plain_channels<TD>(), kWgCB = wg_gathered_blocks<TD>();
@@ -1752,8 +1894,11 @@ ScatterScratch scatter_scratch(int64_t B, int64_t S, int64_t D, int64_t K, int64
     sc.ovf_cap = std::min<int64_t>(MH * MW * K * (P ? P : 1) * 2, 0x3fffffffLL);
     off += align256((size_t)sc.ovf_cap * sizeof(OverflowEntry));
   }
-  sc.stage = off;  // channel-last copy of a single-row source (see launch_gather_product)
-  if (sc.transposed_path && MH == 1) off += align256((size_t)(B * MH * MW * round_up(S, kGC)) * 4);
+  // channel-last copy of a single-row source, channel-block copy of a bf16 one (see
+  // launch_gather_product)
+  sc.stage = off;
+  if (sc.transposed_path && (MH == 1 || elem == 2))
+    off += align256((size_t)(B * MH * MW * round_up(S, kGC)) * 4);
   sc.total = off;
   return sc;
 }
@@ -1847,7 +1992,7 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
     int *flag = cnt + cells;
     gate = flag;
     OverflowEntry *ovf = (OverflowEntry *)(pbase + sc.ovf);
-    TD *stage = MH == 1 ? (TD *)(base + sc.stage) : nullptr;
+    TD *stage = (MH == 1 || sizeof(TD) == 2) ? (TD *)(base + sc.stage) : nullptr;
     if (!plan)
       if (int rc = build_transposed_map(sc, map, iw, cnt, m, DH, DW, MH, MW, K, s)) return rc;
     if (int rc = launch_pack_weights<TD>(w, wpt, D, S, K, 1, s)) return rc;
