@@ -480,6 +480,28 @@ def test_conv_bf16_wide_outputs(co, device):
         assert rel_err(a.float(), r) < 2e-2, nm
 
 
+@pytest.mark.parametrize("interp", [0, 1])
+@pytest.mark.parametrize("w_img", [256, 300])
+def test_conv_bf16_wide_rows(interp, w_img, device):
+    """bf16 storage on images at least 256 pixels wide: 1 x 128 pixel tiles (ragged at the
+    right edge for W = 300), the channel-block copy of the gathered operand with channels
+    padded (Ci = 24, Co = 40) and the ring of in-flight gathers."""
+    B, Ci, Co, H, K = 2, 24, 40, 6, 9
+    g = torch.Generator().manual_seed(900 + interp + w_img)
+    smap = synthetic.latitude_map(H, w_img, 1)
+    x = torch.randn(B, Ci, H, w_img, generator=g).bfloat16()
+    w = (torch.randn(Co, Ci, K, generator=g) / (Ci * K) ** 0.5).bfloat16()
+    b = torch.randn(Co, generator=g).bfloat16()
+    gy = torch.randn(B, Co, H, w_img, generator=g).bfloat16()
+    y_o = O.mapped_conv_forward(x.float(), smap, w.float(), b.float(), K, interp)
+    g_o = O.mapped_conv_backward(gy.float(), smap, x.float(), w.float(), b.float(), K, interp)
+    y = _C.mapped_conv_forward(*dev(x, smap, w, b), K, interp)
+    gr = _C.mapped_conv_backward(*dev(gy, smap, x, w, b), K, interp)
+    assert rel_err(y.float(), y_o) < 2e-2
+    for a, r, nm in zip(gr, g_o, ("grad_input", "grad_weight", "grad_bias")):
+        assert rel_err(a.float(), r) < 2e-2, nm
+
+
 def test_scatter_forms_many_to_one(device):
     """Every source pixel lands on the same few destination pixels: destination lists far
     longer than the length up to which they are sorted, empty lists everywhere else."""
