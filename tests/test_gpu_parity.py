@@ -327,7 +327,7 @@ def test_conv_bf16_latitude_map_uses_both_backward_paths(device):
 
 
 # ------------------------------------------------------------------ map plans
-@pytest.mark.parametrize("case", ["latitude_fp32", "random_fp32", "mesh_bf16"])
+@pytest.mark.parametrize("case", ["latitude_fp32", "random_fp32", "mesh_bf16", "latitude_bf16"])
 def test_conv_backward_with_map_plan(case, device):
     """A plan built once from the map (conv_map_plan) replaces the per-call build of the
     transposed map and of the pair masks: same gradients as without it, and as the oracle."""
@@ -339,11 +339,13 @@ def test_conv_backward_with_map_plan(case, device):
     else:
         B, Ci, Co, H, W, K = 2, 24, 40, 24, 48, 9
         iw = None
-        if case == "latitude_fp32":
+        if case.startswith("latitude"):
             smap = synthetic.latitude_map(H, W, 1)
         else:
             smap, _ = helpers.random_map(g, H, W, K, 0, H, W, torch.float32)
         shape_in, shape_out, interp, dtype, tol = (B, Ci, H, W), (B, Co, H, W), 1, torch.float32, 1e-5
+        if case == "latitude_bf16":  # the gathered operand goes through its channel-block copy
+            dtype, tol = torch.bfloat16, 2e-2
     x = torch.randn(shape_in, generator=g).to(dtype)
     gy = torch.randn(shape_out, generator=g).to(dtype)
     w = (torch.randn(Co, Ci, K, generator=g) / 8).to(dtype)
