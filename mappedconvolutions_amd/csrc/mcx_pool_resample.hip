@@ -348,19 +348,19 @@ __global__ __launch_bounds__(kThreads) void scan_sums_kernel(uint32_t *__restric
 // at the same step.  Lists longer than kSortMax stay as filled.
 constexpr uint32_t kSortMax = 512;
 
-// Batcher's odd-even merge sort for kNetN keys as a list of compare-exchange pairs, made at
-// compile time so that the unrolled network indexes registers statically.
+// Batcher's odd-even merge sort for N keys (16 or 32) as a list of compare-exchange pairs, made
+// at compile time so that the unrolled network indexes registers statically.
 constexpr int kNetN = 32;
 struct SortNetwork {
   int n;
   unsigned char a[256], b[256];
 };
-constexpr SortNetwork make_network() {
+constexpr SortNetwork make_network(int N) {
   SortNetwork net{};
-  for (int p = 1; p < kNetN; p *= 2)
+  for (int p = 1; p < N; p *= 2)
     for (int k = p; k >= 1; k /= 2)
-      for (int j = k % p; j + k < kNetN; j += 2 * k)
-        for (int i = 0; i < k && i + j + k < kNetN; i++)
+      for (int j = k % p; j + k < N; j += 2 * k)
+        for (int i = 0; i < k && i + j + k < N; i++)
           if ((i + j) / (2 * p) == (i + j + k) / (2 * p)) {
             net.a[net.n] = (unsigned char)(i + j);
             net.b[net.n] = (unsigned char)(i + j + k);
@@ -368,7 +368,39 @@ constexpr SortNetwork make_network() {
           }
   return net;
 }
-constexpr SortNetwork kNet = make_network();
+constexpr SortNetwork kNet32 = make_network(32), kNet16 = make_network(16);
+
+// Sorts the list [start, end) of this lane (at most N entries) in registers: read once, run
+// through the network, written back.  Order: by source, ties by weight.
+template <typename T, int N>
+__device__ inline void network_sort(uint32_t *__restrict__ e_src, T *__restrict__ e_wt,
+                                    uint32_t start, uint32_t end) {
+  constexpr const SortNetwork &net = N == 16 ? kNet16 : kNet32;
+  uint32_t code[N];
+  T w[N];
+#pragma unroll
+  for (int u = 0; u < N; u++) {
+    const bool in = start + u < end;
+    code[u] = in ? e_src[start + u] : 0xffffffffu;  // padding sorts to the end
+    w[u] = in ? e_wt[start + u] : T(0);
+  }
+#pragma unroll
+  for (int c = 0; c < net.n; c++) {
+    const int ia = net.a[c], ib = net.b[c];
+    const bool swap = code[ia] > code[ib] || (code[ia] == code[ib] && w[ia] > w[ib]);
+    const uint32_t ca = swap ? code[ib] : code[ia], cb = swap ? code[ia] : code[ib];
+    const T wa = swap ? w[ib] : w[ia], wb = swap ? w[ia] : w[ib];
+    code[ia] = ca; code[ib] = cb;
+    w[ia] = wa; w[ib] = wb;
+  }
+#pragma unroll
+  for (int u = 0; u < N; u++) {
+    if (start + u < end) {
+      e_src[start + u] = code[u];
+      e_wt[start + u] = w[u];
+    }
+  }
+}
 
 template <typename T>
 __global__ __launch_bounds__(kThreads) void sort_entries_kernel(
@@ -384,30 +416,10 @@ __global__ __launch_bounds__(kThreads) void sort_entries_kernel(
   // (a wave most of whose lists are very short is quicker with the insertion sort)
   if (__builtin_amdgcn_ballot_w64(end - start > (uint32_t)kNetN) == 0 &&
       __builtin_popcountll(__builtin_amdgcn_ballot_w64(end - start > 8u)) >= 32) {
-    uint32_t code[kNetN];
-    T w[kNetN];
-#pragma unroll
-    for (int u = 0; u < kNetN; u++) {
-      const bool in = start + u < end;
-      code[u] = in ? e_src[start + u] : 0xffffffffu;  // padding sorts to the end
-      w[u] = in ? e_wt[start + u] : T(0);
-    }
-#pragma unroll
-    for (int c = 0; c < kNet.n; c++) {
-      const int ia = kNet.a[c], ib = kNet.b[c];
-      const bool swap = code[ia] > code[ib] || (code[ia] == code[ib] && w[ia] > w[ib]);
-      const uint32_t ca = swap ? code[ib] : code[ia], cb = swap ? code[ia] : code[ib];
-      const T wa = swap ? w[ib] : w[ia], wb = swap ? w[ia] : w[ib];
-      code[ia] = ca; code[ib] = cb;
-      w[ia] = wa; w[ib] = wb;
-    }
-#pragma unroll
-    for (int u = 0; u < kNetN; u++) {
-      if (start + u < end) {
-        e_src[start + u] = code[u];
-        e_wt[start + u] = w[u];
-      }
-    }
+    if (__builtin_amdgcn_ballot_w64(end - start > 16u) == 0)
+      network_sort<T, 16>(e_src, e_wt, start, end);
+    else
+      network_sort<T, 32>(e_src, e_wt, start, end);
     return;
   }
   if (!live) return;
