@@ -555,6 +555,30 @@ def test_config4_cube_resample_and_pools(interp, device):
                    O.mapped_avg_unpool(gy, lmap, H, W, 9, 1)) < 1e-5
 
 
+@pytest.mark.parametrize("radius,interp", [(1, 1), (2, 0), (2, 1)])
+def test_unpool_list_lengths_for_both_sorting_networks(radius, interp, device):
+    """Unpooling through latitude maps whose per-pixel contribution lists are 9 to 16 entries
+    long (3x3 bilinear: the 16-key sorting network) and 17 to 32 (5x5 nearest: 25 entries,
+    the 32-key network) or longer (5x5 bilinear: 50, insertion sort): same values as the
+    oracle, and the same bits on every call."""
+    B, C, H, W = 2, 3, 24, 128
+    K = (2 * radius + 1) ** 2
+    g = torch.Generator().manual_seed(40 + radius + interp)
+    lmap = synthetic.latitude_map(H, W, radius)
+    x = torch.randn(B, C, H, W, generator=g)
+    gy = torch.randn(B, C, H, W, generator=g)
+    _, mi = O.mapped_max_pool(x, lmap, K, interp)
+    want_a = O.mapped_avg_unpool(gy, lmap, H, W, K, interp)
+    want_m = O.mapped_max_unpool(gy, mi, lmap, H, W, K, interp)
+    gyd, ld, mid = gy.cuda(), lmap.cuda(), mi.cuda()
+    got_a = _C.mapped_avg_unpool(gyd, ld, H, W, K, interp)
+    got_m = _C.mapped_max_unpool(gyd, mid, ld, H, W, K, interp)
+    assert rel_err(got_a, want_a) < 1e-5
+    assert rel_err(got_m, want_m) < 1e-5
+    assert torch.equal(got_a, _C.mapped_avg_unpool(gyd, ld, H, W, K, interp))
+    assert torch.equal(got_m, _C.mapped_max_unpool(gyd, mid, ld, H, W, K, interp))
+
+
 def test_config4_full_size_scatter_properties(device):
     """Full spatial size of the cube -> equirect resampling (256x1536 -> 512x1024) and of the
     512x1024 unpoolings, fewer planes: the gather form against the atomic form, and
