@@ -11,6 +11,9 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kCH = 8;  // channels per thread
+// Channels per thread of the pooling gather that keeps its taps in registers: resolving 9 taps
+// costs about as much as sampling 6 channels, so it is spread over more of them.
+constexpr int kPoolCH = 32;
 // Map locations per workgroup: a 32 x 8 patch for resampling (arbitrary maps: neighbouring
 // rows of the map read neighbouring source pixels), one 256-long row segment for pooling
 // (taps already reach into the rows above and below; longer rows mean fewer cache lines
@@ -50,11 +53,12 @@ template <typename T, int MODE, int OP>
 __device__ inline void direct_gather(const T *__restrict__ in, const T *__restrict__ map,
                                      const T *__restrict__ iw, T *__restrict__ out,
                                      int64_t *__restrict__ idx, int C, int IH, int IW, int N,
-                                     int K, int P, int n, int c0, int b) {
+                                     int K, int P, int n, int c0, int b, int cpt) {
+  // cpt: channels per thread, kPoolCH on the register-tap path below and kCH otherwise
   const int64_t plane = (int64_t)IH * IW;
   const T *src = in + ((int64_t)b * C + c0) * plane;
   const int pm = P == 0 ? 1 : P;
-  const int nc = min(kCH, C - c0);
+  const int nc = min(cpt, C - c0);
 
   if constexpr (OP != OP_RESAMPLE) {
     // Pooling with few unweighted taps: resolve them all first and walk the channels in the
@@ -163,7 +167,7 @@ template <typename T, int MODE, int OP>
 __global__ __launch_bounds__(kThreads) void gather_kernel(
     const T *__restrict__ in, const T *__restrict__ map, const T *__restrict__ iw,
     T *__restrict__ out, int64_t *__restrict__ idx, int C, int IH, int IW, int N, int MW, int K,
-    int P) {
+    int P, int cpt) {
   constexpr int kTileW = Patch<OP>::kW, kTileH = Patch<OP>::kH;
   const int tiles_x = (MW + kTileW - 1) / kTileW;
   // (pooling only: a resampling map's rows need not read neighbouring source rows, and the
@@ -173,8 +177,8 @@ __global__ __launch_bounds__(kThreads) void gather_kernel(
   const int ty = (tile / tiles_x) * kTileH + threadIdx.x / kTileW;
   const int n = ty * MW + tx;
   if (tx >= MW || n >= N) return;
-  direct_gather<T, MODE, OP>(in, map, iw, out, idx, C, IH, IW, N, K, P, n, blockIdx.y * kCH,
-                             blockIdx.z);
+  direct_gather<T, MODE, OP>(in, map, iw, out, idx, C, IH, IW, N, K, P, n, blockIdx.y * cpt,
+                             blockIdx.z, cpt);
 }
 
 // Scatter form (adjoint of the gather).  OP_RESAMPLE: K == 1, pushes the value;
@@ -442,7 +446,11 @@ __global__ __launch_bounds__(kThreads) void sort_entries_kernel(
   }
 }
 
-constexpr int kTCH = 8;  // planes per thread of the transposed gather
+// Planes per thread of the transposed gather.  The unpoolings read their list of about 15
+// entries once per thread: more planes per thread spread that over more work (8 -> 32 planes
+// took a third off the kernel); resampling lists are short and 8 planes measured best.
+template <int OP>
+constexpr int planes_per_thread() { return OP == UN_RESAMPLE ? 8 : 32; }
 
 // One thread per destination pixel and kTCH planes.  UN_MAX keeps a contribution
 // only where the recorded winner of that source element is this tap.
@@ -452,6 +460,7 @@ __global__ __launch_bounds__(kThreads) void transposed_gather_kernel(
     const uint32_t *__restrict__ local, const uint32_t *__restrict__ bsum,
     const uint32_t *__restrict__ e_src, const T *__restrict__ e_wt, int64_t planes, int nsrc,
     int ndst, int K, int idx_scale, int groups) {
+  constexpr int kTCH = planes_per_thread<OP>();
   const int pg = blockIdx.x % groups;
   const int p = (blockIdx.x / groups) * kThreads + threadIdx.x;
   if (p >= ndst) return;
@@ -563,11 +572,13 @@ int launch_gather(const void *in, const void *map, const void *iw, void *out, in
                   int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t MH, int64_t MW, int64_t K,
                   int64_t P, int interp, hipStream_t s) {
   const int64_t N = MH * MW;
-  dim3 grid(div_up(MW, Patch<OP>::kW) * div_up(MH, Patch<OP>::kH), div_up(C, kCH), (unsigned)B);
+  // (the same test as in direct_gather: unweighted pooling with at most 9 taps)
+  const int cpt = (OP != OP_RESAMPLE && P == 0 && K <= 9) ? kPoolCH : kCH;
+  dim3 grid(div_up(MW, Patch<OP>::kW) * div_up(MH, Patch<OP>::kH), div_up(C, cpt), (unsigned)B);
   MCX_DISPATCH_MODE(interp, hipLaunchKernelGGL((gather_kernel<T, MODE, OP>), grid, dim3(kThreads),
                                                0, s, (const T *)in, (const T *)map,
                                                (const T *)iw, (T *)out, idx, (int)C, (int)IH,
-                                               (int)IW, (int)N, (int)MW, (int)K, (int)P));
+                                               (int)IW, (int)N, (int)MW, (int)K, (int)P, cpt));
   MCX_HIP_CHECK_LAUNCH();
   return 0;
 }
@@ -613,6 +624,7 @@ int launch_transposed(const void *src, const int64_t *idx, const void *map, cons
   const int64_t samples = nsrc * K * pm, ndst = DH * DW;
   const TransposedLayout l = transposed_layout(ndst, samples, corners_of(interp), sizeof(T));
   if (!ws || !l.ok || ws_bytes < l.total || nsrc * K > 0xffffffffLL) return kNotApplicable;
+  constexpr int kTCH = planes_per_thread<OP>();
   const int64_t groups = (planes + kTCH - 1) / kTCH;
   const int64_t blocks = groups * ((ndst + kThreads - 1) / kThreads);
   if (blocks > 0x7fffffffLL) return kNotApplicable;
