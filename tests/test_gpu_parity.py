@@ -555,6 +555,28 @@ def test_config4_cube_resample_and_pools(interp, device):
                    O.mapped_avg_unpool(gy, lmap, H, W, 9, 1)) < 1e-5
 
 
+@pytest.mark.parametrize("interp", [0, 1])
+def test_pools_with_more_channels_than_one_thread_takes(interp, device):
+    """3x3 pooling and unpooling with 40 channels and 2 images: the pooling gather takes 32
+    channels per thread and the unpooling gather 32 planes (80 = 32 + 32 + 16), so both see
+    full and ragged groups.  Bit-exact pooling outputs and argmax, 1e-5 on the unpoolings."""
+    B, C, H, W, K = 2, 40, 8, 64, 9
+    g = torch.Generator().manual_seed(60 + interp)
+    lmap = synthetic.latitude_map(H, W, 1)
+    x = torch.randn(B, C, H, W, generator=g)
+    gy = torch.randn(B, C, H, W, generator=g)
+    mo, mi = O.mapped_max_pool(x, lmap, K, interp)
+    ao = O.mapped_avg_pool(x, lmap, K, interp)
+    xd, ld, gyd = x.cuda(), lmap.cuda(), gy.cuda()
+    m, i = _C.mapped_max_pool(xd, ld, K, interp)
+    a = _C.mapped_avg_pool(xd, ld, K, interp)
+    assert torch.equal(m.cpu(), mo) and torch.equal(i.cpu(), mi) and torch.equal(a.cpu(), ao)
+    assert rel_err(_C.mapped_avg_unpool(gyd, ld, H, W, K, interp),
+                   O.mapped_avg_unpool(gy, lmap, H, W, K, interp)) < 1e-5
+    assert rel_err(_C.mapped_max_unpool(gyd, i, ld, H, W, K, interp),
+                   O.mapped_max_unpool(gy, mi, lmap, H, W, K, interp)) < 1e-5
+
+
 @pytest.mark.parametrize("radius,interp", [(1, 1), (2, 0), (2, 1)])
 def test_unpool_list_lengths_for_both_sorting_networks(radius, interp, device):
     """Unpooling through latitude maps whose per-pixel contribution lists are 9 to 16 entries
