@@ -377,8 +377,7 @@ constexpr SortNetwork kNet32 = make_network(32), kNet16 = make_network(16);
 // Sorts the list [start, end) of this lane (at most N entries) in registers: read once, run
 // through the network, written back.  Order: by source, ties by weight.
 template <typename T, int N>
-__device__ inline void network_sort(uint32_t *__restrict__ e_src, T *__restrict__ e_wt,
-                                    uint32_t start, uint32_t end) {
+__device__ inline void network_sort(uint32_t *e_src, T *e_wt, uint32_t start, uint32_t end) {
   constexpr const SortNetwork &net = N == 16 ? kNet16 : kNet32;
   uint32_t code[N];
   T w[N];
@@ -420,10 +419,33 @@ __global__ __launch_bounds__(kThreads) void sort_entries_kernel(
   // (a wave most of whose lists are very short is quicker with the insertion sort)
   if (__builtin_amdgcn_ballot_w64(end - start > (uint32_t)kNetN) == 0 &&
       __builtin_popcountll(__builtin_amdgcn_ballot_w64(end - start > 8u)) >= 32) {
-    if (__builtin_amdgcn_ballot_w64(end - start > 16u) == 0)
-      network_sort<T, 16>(e_src, e_wt, start, end);
-    else
+    if (__builtin_amdgcn_ballot_w64(end - start > 16u) == 0) {
+      // The lists of a wave's 64 pixels are one contiguous run of at most 1024 entries: it
+      // is copied to LDS and back with coalesced accesses, and each lane sorts its piece
+      // there (a lane's own list starts 15 or so words after its neighbour's: separate
+      // cache lines in memory, separate banks in LDS).
+      __shared__ uint32_t run_src[kThreads / 64][64 * 16];
+      __shared__ T run_wt[kThreads / 64][64 * 16];
+      const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
+      const uint32_t first = __builtin_amdgcn_readfirstlane(start);  // lane 0 is live here
+      uint32_t last = end;
+      for (int d = 32; d > 0; d >>= 1) last = max(last, (uint32_t)__shfl_xor((int)last, d));
+      const uint32_t total = __builtin_amdgcn_readfirstlane(last) - first;
+      for (uint32_t t = lane; t < total; t += 64) {
+        run_src[wv][t] = e_src[first + t];
+        run_wt[wv][t] = e_wt[first + t];
+      }
+      __builtin_amdgcn_wave_barrier();
+      const uint32_t off = live ? start - first : 0u;
+      network_sort<T, 16>(run_src[wv], run_wt[wv], off, off + (end - start));
+      __builtin_amdgcn_wave_barrier();
+      for (uint32_t t = lane; t < total; t += 64) {
+        e_src[first + t] = run_src[wv][t];
+        e_wt[first + t] = run_wt[wv][t];
+      }
+    } else {
       network_sort<T, 32>(e_src, e_wt, start, end);
+    }
     return;
   }
   if (!live) return;
