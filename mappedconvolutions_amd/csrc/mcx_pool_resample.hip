@@ -13,7 +13,7 @@ constexpr int kThreads = 256;
 constexpr int kCH = 8;  // channels per thread
 // Channels per thread of the pooling gather that keeps its taps in registers: resolving 9 taps
 // costs about as much as sampling 6 channels, so it is spread over more of them.
-constexpr int kPoolCH = 32;
+constexpr int kPoolCH = 64;
 // Map locations per workgroup: a 32 x 8 patch for resampling (arbitrary maps: neighbouring
 // rows of the map read neighbouring source pixels), one 256-long row segment for pooling
 // (taps already reach into the rows above and below; longer rows mean fewer cache lines
@@ -469,10 +469,10 @@ __global__ __launch_bounds__(kThreads) void sort_entries_kernel(
 }
 
 // Planes per thread of the transposed gather.  The unpoolings read their list of about 15
-// entries once per thread: more planes per thread spread that over more work (8 -> 32 planes
+// entries once per thread: more planes per thread spread that over more work (8 -> 64 planes
 // took a third off the kernel); resampling lists are short and 8 planes measured best.
 template <int OP>
-constexpr int planes_per_thread() { return OP == UN_RESAMPLE ? 8 : 32; }
+constexpr int planes_per_thread() { return OP == UN_RESAMPLE ? 8 : 64; }
 
 // One thread per destination pixel and kTCH planes.  UN_MAX keeps a contribution
 // only where the recorded winner of that source element is this tap.

@@ -557,10 +557,11 @@ def test_config4_cube_resample_and_pools(interp, device):
 
 @pytest.mark.parametrize("interp", [0, 1])
 def test_pools_with_more_channels_than_one_thread_takes(interp, device):
-    """3x3 pooling and unpooling with 40 channels and 2 images: the pooling gather takes 32
-    channels per thread and the unpooling gather 32 planes (80 = 32 + 32 + 16), so both see
-    full and ragged groups.  Bit-exact pooling outputs and argmax, 1e-5 on the unpoolings."""
-    B, C, H, W, K = 2, 40, 8, 64, 9
+    """3x3 pooling and unpooling with 72 channels and 2 images: the pooling gather takes 64
+    channels per thread (72 = 64 + 8) and the unpooling gather 64 planes (144 = 64 + 64 + 16),
+    so both see full and ragged groups.  Bit-exact pooling outputs and argmax, 1e-5 on the
+    unpoolings."""
+    B, C, H, W, K = 2, 72, 8, 64, 9
     g = torch.Generator().manual_seed(60 + interp)
     lmap = synthetic.latitude_map(H, W, 1)
     x = torch.randn(B, C, H, W, generator=g)
