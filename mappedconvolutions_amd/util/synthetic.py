@@ -88,3 +88,31 @@ def sphere_points(n, seed=0, dtype=torch.float32):
     p = rng.standard_normal((3, n))
     p /= np.linalg.norm(p, axis=0, keepdims=True)
     return torch.from_numpy(p[None]).to(dtype).contiguous()
+
+
+def upsampling_map(src_height, src_width, factor, radius=1, latitude=False, aligned=False,
+                   dtype=torch.float32):
+    """Square kernel of an output grid `factor` times finer than the source image it samples:
+    [factor*H, factor*W, (2r+1)^2, 2].  Output pixel (i, j) sits at source position
+    ((j + 0.5) / f - 0.5, (i + 0.5) / f - 0.5), or (j / f, i / f) with `aligned` (coordinates
+    are then multiples of 1/f: integral, .5, ...).  Taps are dy-major at unit source spacing;
+    with `latitude` the x offsets are stretched by 1 / max(cos lat, 0.05) and wrap around.
+    About factor^2 output pixels share every source pixel: the strongly many-to-one case of a
+    scatter through the map."""
+    oh, ow = src_height * factor, src_width * factor
+    i = np.arange(oh, dtype=np.float64)[:, None, None]
+    j = np.arange(ow, dtype=np.float64)[None, :, None]
+    cy = i / factor if aligned else (i + 0.5) / factor - 0.5
+    cx = j / factor if aligned else (j + 0.5) / factor - 0.5
+    offs = np.arange(-radius, radius + 1, dtype=np.float64)
+    dy, dx = np.meshgrid(offs, offs, indexing='ij')
+    dy, dx = dy.reshape(1, 1, -1), dx.reshape(1, 1, -1)
+    if latitude:
+        lat = ((i + 0.5) / oh) * math.pi - math.pi / 2
+        x = np.mod(cx + dx / np.maximum(np.cos(lat), 0.05), src_width)
+        y = np.clip(cy + dy, 0, src_height - 1) + 0 * j
+    else:
+        x = cx + dx + 0 * i
+        y = cy + dy + 0 * j
+    out = np.stack([np.broadcast_to(x, y.shape), y], axis=-1)
+    return torch.from_numpy(np.ascontiguousarray(out)).to(dtype)

@@ -97,3 +97,59 @@ def rel_err(a, b):
     """max |a-b| / max(|b|, tiny): error relative to the magnitude of the result."""
     a, b = a.double().cpu(), b.double().cpu()
     return ((a - b).abs().max() / b.abs().max().clamp_min(1e-30)).item()
+
+
+def assert_close_elementwise(a, b, tol, what=""):
+    """Every element: |a - b| <= tol * (|b| + rms(b)).  Unlike rel_err, an element that is small
+    against the largest one still has to be right to `tol` of the result's typical size."""
+    a, b = a.double().cpu(), b.double().cpu()
+    rms = b.pow(2).mean().sqrt().clamp_min(1e-30)
+    excess = (a - b).abs() - tol * (b.abs() + rms)
+    worst = excess.max().item()
+    assert worst <= 0, "%s: element off by %.3g beyond tol %.1e (rms %.3g)" % (
+        what, worst + tol * rms.item(), tol, rms.item())
+
+
+def map_contributions(smap, iw, dh, dw, interp):
+    """Destination cells (pixel * K + tap) of every contribution with a nonzero weight that a
+    scatter through `smap` [MH, MW, K, (P,) 2] makes into a dh x dw image: the entries of the
+    map turned around.  Returns a 1-D int64 tensor of cell indices (with repeats)."""
+    K = smap.shape[2]
+    m = smap.double()
+    if iw is None:
+        m = m.unsqueeze(3)
+        w = torch.ones(m.shape[:-1], dtype=torch.float64)
+    else:
+        w = iw.double()
+    x, y = m[..., 0], m[..., 1]
+    tap = torch.arange(K).view(1, 1, K, 1).expand_as(x)
+    cells = []
+    if interp == 0:
+        xi = torch.where(x >= 0, (x + 0.5).floor(), (x - 0.5).ceil()).long()
+        yi = torch.where(y >= 0, (y + 0.5).floor(), (y - 0.5).ceil()).long()
+        corners = [(xi, yi, w)]
+    else:
+        x1, y1 = x.floor(), y.floor()
+        corners = []
+        for cx, cy, cw in ((x1, y1, (y1 + 1 - y) * (x1 + 1 - x)), (x1 + 1, y1, (y1 + 1 - y) * (x - x1)),
+                           (x1, y1 + 1, (y - y1) * (x1 + 1 - x)), (x1 + 1, y1 + 1, (y - y1) * (x - x1))):
+            corners.append((cx.long(), cy.long(), cw * w))
+    for cx, cy, cw in corners:
+        if interp == 2:
+            cx = cx % dw
+        ok = (cx >= 0) & (cx < dw) & (cy >= 0) & (cy < dh) & (cw != 0)
+        cells.append(((cy * dw + cx) * K + tap)[ok])
+    return torch.cat(cells)
+
+
+def transposed_map_overflows(smap, iw, dh, dw, interp):
+    """True when the convolution's slotted transposed map cannot hold this map: more
+    contributions beyond the slots of their cells (4, or 8 for single-row maps) than the
+    overflow list has room for (2 per map sample).  The product then runs through the
+    scatter kernel with its LDS windows and atomics."""
+    cells = map_contributions(smap, iw, dh, dw, interp)
+    slots = 8 if smap.shape[0] == 1 else 4
+    counts = torch.bincount(cells, minlength=dh * dw * smap.shape[2])
+    spill = (counts - slots).clamp_min(0).sum().item()
+    cap = smap[..., 0].numel() * 2
+    return spill > cap
