@@ -24,8 +24,11 @@
  *     fully overwritten: the library clears them itself before accumulating.
  *   - Return value: 0 on success; a positive hipError_t if a launch failed; a
  *     negative MCX_E_* for rejected arguments.  Nothing aborts the process.
- *   - Thread safety: no global mutable state; concurrent calls on different
- *     streams are independent as long as their output buffers are.
+ *   - Thread safety: concurrent calls on different streams are independent as long as
+ *     their output and workspace buffers are.  Two pieces of state live in the library: a
+ *     per-thread timing request (mcx_profile_dominant_kernel; consumed or dropped by the
+ *     next convolution call of that thread) and the per-GPU scratch array of
+ *     mcx_conv_forward_static (calls of that one entry point that overlap on one GPU race).
  */
 #ifndef MCX_H_
 #define MCX_H_
@@ -44,7 +47,8 @@ enum {
   MCX_E_DTYPE = -1,     /* dtype not supported by this entry point */
   MCX_E_SHAPE = -2,     /* a size is negative, zero where it may not be, or too large */
   MCX_E_NULL = -3,      /* a required pointer is NULL (or iw/P disagree) */
-  MCX_E_WORKSPACE = -4  /* workspace missing or too small */
+  MCX_E_WORKSPACE = -4, /* workspace missing or too small */
+  MCX_E_STATIC_LIMIT = -5 /* needs more scratch than mcx_conv_forward_static's fixed buffer */
 };
 
 /* Library identification; bumps when a signature changes. */
@@ -132,6 +136,23 @@ int mcx_conv_forward(const void *x, const void *map, const void *iw, const void 
                      const void *bias, void *y, void *workspace, size_t workspace_bytes,
                      int64_t B, int64_t Ci, int64_t Co, int64_t IH, int64_t IW, int64_t OH,
                      int64_t OW, int64_t K, int64_t P, int interp, int dtype, void *stream);
+
+/* mcx_conv_forward for callers that cannot allocate device memory or hand over a workspace
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It
+ * has no counterpart in the reference.  Same arguments and results as mcx_conv_forward, but
+ * the scratch (repacked weights, the map's pair mask, staging copies) lives in an array of
+ * MCX_STATIC_SCRATCH_BYTES inside the library's code object, one copy per GPU, held until the
+ * process ends; the call makes no hipMalloc / hipFree.  Problems whose
+ * mcx_conv_forward_workspace() exceeds that size (bf16 storage and single-row sources need a
+ * staging copy as large as the input) return MCX_E_STATIC_LIMIT.  All calls on one GPU share
+ * the array: calls that overlap on one GPU (different streams or threads) race; calls on one
+ * stream are ordered and safe.  The first call on a device looks up the array's address
+ * (hipGetSymbolAddress), so make it outside any graph capture. */
+#define MCX_STATIC_SCRATCH_BYTES ((size_t)8 << 20)
+int mcx_conv_forward_static(const void *x, const void *map, const void *iw, const void *w,
+                            const void *bias, void *y, int64_t B, int64_t Ci, int64_t Co,
+                            int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P,
+                            int interp, int dtype, void *stream);
 
 /* Bytes of device scratch the matching call needs for these sizes (may be 0).
  * The scratch holds repacked weights and partial sums; its contents need not

@@ -30,6 +30,7 @@ SIGNATURES = {
     "mcx_avg_pool": (_i, [_p] * 4 + [_i64] * 8 + [_i, _i, _p]),
     "mcx_avg_unpool": (_i, [_p] * 5 + [_sz] + [_i64] * 8 + [_i, _i, _p]),
     "mcx_conv_forward": (_i, [_p] * 7 + [_sz] + [_i64] * 9 + [_i, _i, _p]),
+    "mcx_conv_forward_static": (_i, [_p] * 6 + [_i64] * 9 + [_i, _i, _p]),
     "mcx_conv_forward_workspace": (_sz, [_i64] * 9 + [_i]),
     "mcx_conv_backward_workspace": (_sz, [_i64] * 9 + [_i]),
     "mcx_conv_backward": (_i, [_p] * 9 + [_sz] + [_i64] * 9 + [_i, _i, _p]),

@@ -6,6 +6,7 @@
 // with more points).
 #include <algorithm>
 #include <initializer_list>
+#include <mutex>
 
 #include "mcx.h"
 #include "mcx_conv.h"
@@ -13,7 +14,50 @@
 
 using namespace mcx;
 
+// Scratch of mcx_conv_forward_static: one array per GPU, part of the loaded code object, so
+// the entry point never allocates.  Host code must not use the array's name as an address
+// (it is a host-side stand-in); the device address is looked up once per device with
+// hipGetSymbolAddress and kept in g_static_scratch.
+constexpr size_t kStaticScratchBytes = MCX_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+void *g_static_scratch[kMaxDevices] = {};
+std::mutex g_static_scratch_mutex;
+
+// Device address of `scratch` on the current device (looked up at the first call on that
+// device); nullptr and *rc set on failure.
+void *static_scratch_of_current_device(int *rc) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    *rc = (int)e;
+    return nullptr;
+  }
+  if (dev < 0 || dev >= kMaxDevices) {
+    *rc = MCX_E_SHAPE;
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+  if (!g_static_scratch[dev]) {
+    void *ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      *rc = e != hipSuccess ? (int)e : (int)hipErrorInvalidSymbol;
+      return nullptr;
+    }
+    g_static_scratch[dev] = ptr;
+  }
+  return g_static_scratch[dev];
+}
+
+// A timing request (mcx_profile_dominant_kernel) is consumed by the kernel launch it asks
+// for; an entry point that returns before that launch must not leave it armed.
+struct ProfileRequestScope {
+  ~ProfileRequestScope() { mcx::set_profile_events(nullptr, nullptr); }
+};
 
 struct ConvDims {
   int64_t B, Ci, Co, IH, IW, OH, OW, K, P;
@@ -322,6 +366,7 @@ extern "C" int mcx_conv_forward(const void *x, const void *map, const void *iw, 
                                 size_t workspace_bytes, int64_t B, int64_t Ci, int64_t Co,
                                 int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
                                 int64_t P, int interp, int dtype, void *stream) {
+  ProfileRequestScope profile_scope;
   const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
   if (int rc = check_dims(d, OH, OW)) return rc;
   if (int rc = check_ptrs(x, map, iw, w, P)) return rc;
@@ -330,6 +375,30 @@ extern "C" int mcx_conv_forward(const void *x, const void *map, const void *iw, 
   const bool mfma = use_mfma(dtype, P);
   MCX_DISPATCH_DTYPE(dtype, conv_forward_t<T>(mfma, x, map, iw, w, bias, y, workspace,
                                               workspace_bytes, d, interp, s));
+}
+
+extern "C" int mcx_conv_forward_static(const void *x, const void *map, const void *iw,
+                                       const void *w, const void *bias, void *y, int64_t B,
+                                       int64_t Ci, int64_t Co, int64_t IH, int64_t IW, int64_t OH,
+                                       int64_t OW, int64_t K, int64_t P, int interp, int dtype,
+                                       void *stream) {
+  ProfileRequestScope profile_scope;
+  const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
+  if (int rc = check_dims(d, OH, OW)) return rc;
+  if (int rc = check_ptrs(x, map, iw, w, P)) return rc;
+  if (!bias || !y) return MCX_E_NULL;
+  if (dtype != MCX_F32 && dtype != MCX_F64 && dtype != MCX_BF16) return MCX_E_DTYPE;
+  const size_t need = gather_product_ws(dtype, Ci, Co, K, P, B, IH, IW);
+  if (need > kStaticScratchBytes) return MCX_E_STATIC_LIMIT;
+  int rc = 0;
+  void *ws = static_scratch_of_current_device(&rc);
+  if (!ws) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  const bool mfma = use_mfma(dtype, P);
+  // the kernels overwrite every word of the scratch they read (the weight-packing kernel
+  // clears the flag word beside the packed weights), so nothing of the last call survives
+  MCX_DISPATCH_DTYPE(dtype, conv_forward_t<T>(mfma, x, map, iw, w, bias, y, ws,
+                                              kStaticScratchBytes, d, interp, s));
 }
 
 extern "C" size_t mcx_conv_backward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t IH,
@@ -346,6 +415,7 @@ extern "C" int mcx_conv_backward(const void *gy, const void *map, const void *iw
                                  size_t workspace_bytes, int64_t B, int64_t Ci, int64_t Co,
                                  int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
                                  int64_t P, int interp, int dtype, void *stream) {
+  ProfileRequestScope profile_scope;
   const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
   if (int rc = check_dims(d, OH, OW)) return rc;
   if (int rc = check_ptrs(gy, map, iw, w, P)) return rc;
@@ -382,6 +452,7 @@ extern "C" int mcx_conv_backward_planned(const void *gy, const void *map, const 
                                          int64_t Ci, int64_t Co, int64_t IH, int64_t IW,
                                          int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
                                          int dtype, void *stream) {
+  ProfileRequestScope profile_scope;
   const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
   if (int rc = check_dims(d, OH, OW)) return rc;
   if (int rc = check_ptrs(gy, map, iw, w, P)) return rc;
@@ -408,6 +479,7 @@ extern "C" int mcx_tconv_forward(const void *x, const void *map, const void *iw,
                                  size_t workspace_bytes, int64_t B, int64_t Ci, int64_t Co,
                                  int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
                                  int64_t P, int interp, int dtype, void *stream) {
+  ProfileRequestScope profile_scope;
   const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
   if (int rc = check_dims(d, IH, IW)) return rc;
   if (int rc = check_ptrs(x, map, iw, w, P)) return rc;
@@ -433,6 +505,7 @@ extern "C" int mcx_tconv_backward(const void *gy, const void *map, const void *i
                                   size_t workspace_bytes, int64_t B, int64_t Ci, int64_t Co,
                                   int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
                                   int64_t P, int interp, int dtype, void *stream) {
+  ProfileRequestScope profile_scope;
   const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
   if (int rc = check_dims(d, IH, IW)) return rc;
   if (int rc = check_ptrs(gy, map, iw, w, P)) return rc;
@@ -443,7 +516,7 @@ extern "C" int mcx_tconv_backward(const void *gy, const void *map, const void *i
                                                 workspace_bytes, d, interp, s));
 }
 
-extern "C" int mcx_abi_version(void) { return 7; }
+extern "C" int mcx_abi_version(void) { return 8; }
 
 extern "C" int mcx_profile_dominant_kernel(void *start_event, void *stop_event) {
   mcx::set_profile_events(start_event, stop_event);
@@ -457,6 +530,9 @@ extern "C" const char *mcx_error_string(int code) {
     case MCX_E_SHAPE: return "mcx: invalid or too large dimension";
     case MCX_E_NULL: return "mcx: required pointer is NULL, or interp_weights and P disagree";
     case MCX_E_WORKSPACE: return "mcx: workspace missing or too small";
+    case MCX_E_STATIC_LIMIT:
+      return "mcx: this problem needs more scratch than the library's static buffer holds; "
+             "use the entry point that takes a workspace";
     default: return code > 0 ? hipGetErrorString((hipError_t)code) : "mcx: unknown error";
   }
 }
