@@ -357,6 +357,8 @@ def weighted_mapped_transposed_conv_backward(grad_output, sample_map, interp_wei
 
 # ------------------------------------------------------------------------ pooling
 def _pool_dims(input, sample_map, interp_weights, kernel_size):
+    if input.dim() != 4:
+        raise RuntimeError("expected a 4-D [B, C, H, W] tensor, got %d dimensions" % input.dim())
     P = _weighted_dims(sample_map, interp_weights, True)
     K = int(kernel_size)
     if sample_map.shape[2] != K:
@@ -393,6 +395,8 @@ def _max_unpool(grad_output, idx_mask, sample_map, interp_weights, input_height,
         raise RuntimeError("idx_mask must be int64 with grad_output's shape")
     P, K = _pool_dims(grad_output, sample_map, interp_weights, kernel_size)
     B, C, OH, OW = grad_output.shape
+    if tuple(sample_map.shape[:2]) != (OH, OW):
+        raise RuntimeError("sample_map spatial size must match grad_output")
     IH, IW = int(input_height), int(input_width)
     gin = torch.empty((B, C, IH, IW), dtype=grad_output.dtype, device=grad_output.device)
     lib = _lib.load()
@@ -501,6 +505,8 @@ def _resample_to_map(input, sample_map, interp_weights, output_height, output_wi
     _on_gpu("input", input, sample_map=sample_map, interp_weights=interp_weights)
     dt = _dtype(input, maps=(sample_map, interp_weights))
     P = _weighted_dims(sample_map, interp_weights, False)
+    if input.dim() != 4:
+        raise RuntimeError("expected a 4-D [B, C, H, W] tensor, got %d dimensions" % input.dim())
     B, C, IH, IW = input.shape
     if tuple(sample_map.shape[:2]) != (IH, IW):
         raise RuntimeError("sample_map spatial size must match the input")
@@ -523,6 +529,8 @@ def _resample_from_map(input, sample_map, interp_weights, interpolation):
     _on_gpu("input", input, sample_map=sample_map, interp_weights=interp_weights)
     dt = _dtype(input, maps=(sample_map, interp_weights))
     P = _weighted_dims(sample_map, interp_weights, False)
+    if input.dim() != 4:
+        raise RuntimeError("expected a 4-D [B, C, H, W] tensor, got %d dimensions" % input.dim())
     B, C, SH, SW = input.shape
     MH, MW = sample_map.shape[0], sample_map.shape[1]
     out = torch.empty((B, C, MH, MW), dtype=input.dtype, device=input.device)

@@ -65,7 +65,10 @@ struct ConvDims {
 
 // map_h x map_w is the spatial size of the sample map (output for convolution,
 // input for transposed convolution).
-int check_dims(const ConvDims &d, int64_t map_h, int64_t map_w) {
+int check_dims(const ConvDims &d, int64_t map_h, int64_t map_w, int dtype) {
+  // samples are addressed with 32-bit byte offsets inside a plane
+  const int64_t elem = dtype == MCX_F64 ? 8 : dtype == MCX_BF16 ? 2 : 4;
+  if (d.IH * d.IW * elem > 0xffffffffLL || d.OH * d.OW * elem > 0xffffffffLL) return MCX_E_SHAPE;
   for (int64_t v : {d.B, d.Ci, d.Co, d.IH, d.IW, d.OH, d.OW, d.K, d.IH * d.IW, d.OH * d.OW})
     if (v <= 0 || v > 0x7fffffffLL) return MCX_E_SHAPE;
   if (d.P < 0 || d.P > 0x7fffffffLL || d.B > 65535) return MCX_E_SHAPE;
@@ -368,7 +371,7 @@ extern "C" int mcx_conv_forward(const void *x, const void *map, const void *iw, 
                                 int64_t P, int interp, int dtype, void *stream) {
   ProfileRequestScope profile_scope;
   const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
-  if (int rc = check_dims(d, OH, OW)) return rc;
+  if (int rc = check_dims(d, OH, OW, dtype)) return rc;
   if (int rc = check_ptrs(x, map, iw, w, P)) return rc;
   if (!bias || !y) return MCX_E_NULL;
   hipStream_t s = (hipStream_t)stream;
@@ -384,7 +387,7 @@ extern "C" int mcx_conv_forward_static(const void *x, const void *map, const voi
                                        void *stream) {
   ProfileRequestScope profile_scope;
   const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
-  if (int rc = check_dims(d, OH, OW)) return rc;
+  if (int rc = check_dims(d, OH, OW, dtype)) return rc;
   if (int rc = check_ptrs(x, map, iw, w, P)) return rc;
   if (!bias || !y) return MCX_E_NULL;
   if (dtype != MCX_F32 && dtype != MCX_F64 && dtype != MCX_BF16) return MCX_E_DTYPE;
@@ -417,7 +420,7 @@ extern "C" int mcx_conv_backward(const void *gy, const void *map, const void *iw
                                  int64_t P, int interp, int dtype, void *stream) {
   ProfileRequestScope profile_scope;
   const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
-  if (int rc = check_dims(d, OH, OW)) return rc;
+  if (int rc = check_dims(d, OH, OW, dtype)) return rc;
   if (int rc = check_ptrs(gy, map, iw, w, P)) return rc;
   if (gw && !x) return MCX_E_NULL;
   hipStream_t s = (hipStream_t)stream;
@@ -454,7 +457,7 @@ extern "C" int mcx_conv_backward_planned(const void *gy, const void *map, const 
                                          int dtype, void *stream) {
   ProfileRequestScope profile_scope;
   const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
-  if (int rc = check_dims(d, OH, OW)) return rc;
+  if (int rc = check_dims(d, OH, OW, dtype)) return rc;
   if (int rc = check_ptrs(gy, map, iw, w, P)) return rc;
   if (gw && !x) return MCX_E_NULL;
   hipStream_t s = (hipStream_t)stream;
@@ -481,7 +484,7 @@ extern "C" int mcx_tconv_forward(const void *x, const void *map, const void *iw,
                                  int64_t P, int interp, int dtype, void *stream) {
   ProfileRequestScope profile_scope;
   const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
-  if (int rc = check_dims(d, IH, IW)) return rc;
+  if (int rc = check_dims(d, IH, IW, dtype)) return rc;
   if (int rc = check_ptrs(x, map, iw, w, P)) return rc;
   if (!bias || !y) return MCX_E_NULL;
   hipStream_t s = (hipStream_t)stream;
@@ -507,7 +510,7 @@ extern "C" int mcx_tconv_backward(const void *gy, const void *map, const void *i
                                   int64_t P, int interp, int dtype, void *stream) {
   ProfileRequestScope profile_scope;
   const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
-  if (int rc = check_dims(d, IH, IW)) return rc;
+  if (int rc = check_dims(d, IH, IW, dtype)) return rc;
   if (int rc = check_ptrs(gy, map, iw, w, P)) return rc;
   if (gw && !x) return MCX_E_NULL;
   hipStream_t s = (hipStream_t)stream;

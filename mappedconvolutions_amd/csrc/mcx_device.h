@@ -66,6 +66,44 @@ __device__ inline void atomic_add(double *p, double v) {
   __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// Element `off` of a plane, or element 0 when off < 0 (the caller discards that value).  The
+// load itself is unconditional: a load behind a per-lane test becomes a branch, and a chain of
+// such branches keeps a thread's loads from being in flight together.  The address is the
+// plane pointer (wave-uniform where the plane is chosen per workgroup) plus a 32-bit byte
+// offset, so planes are limited to 4 GiB.
+template <typename TD>
+__device__ inline TD load_elem(const TD *plane, int off) {
+  const unsigned byte_off = (off < 0 ? 0u : (unsigned)off) * (unsigned)sizeof(TD);
+  return *reinterpret_cast<const TD *>(reinterpret_cast<const char *>(plane) + byte_off);
+}
+
+// A plane as a buffer resource: base pointer and size in bytes.  A load whose byte offset
+// lies beyond the size returns 0 and touches no memory, so a tap's corners outside the plane
+// (or with weight zero) are given the offset kOobOffset: no test, no select, no traffic.  The
+// descriptor lives in scalar registers; planes are limited to kOobOffset bytes.
+typedef __amdgpu_buffer_rsrc_t plane_buf_t;
+constexpr unsigned kOobOffset = 0xffffff00u;
+__device__ inline plane_buf_t plane_buf(const void *plane, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(plane), (short)0, (int)bytes,
+                                           0x00020000);
+}
+__device__ inline float buf_load(plane_buf_t r, unsigned byte_off, float) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)byte_off, 0, 0));
+}
+__device__ inline double buf_load(plane_buf_t r, unsigned byte_off, double) {
+  return __builtin_bit_cast(double, __builtin_amdgcn_raw_buffer_load_b64(r, (int)byte_off, 0, 0));
+}
+// Two neighbouring elements with one load (the address need only be element-aligned).
+struct float_pair { float x, y; };
+struct double_pair { double x, y; };
+__device__ inline float_pair buf_load_pair(plane_buf_t r, unsigned byte_off, float) {
+  return __builtin_bit_cast(float_pair, __builtin_amdgcn_raw_buffer_load_b64(r, (int)byte_off, 0, 0));
+}
+__device__ inline double_pair buf_load_pair(plane_buf_t r, unsigned byte_off, double) {
+  return __builtin_bit_cast(double_pair,
+                            __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0));
+}
+
 // ---- taps -----------------------------------------------------------------
 // A tap is one (x, y) sample location resolved against an H x W plane: up to
 // four in-plane element offsets and their weights.  Offsets are -1 for corners
@@ -86,7 +124,21 @@ struct Tap<T, kInterpNearest> {
   }
   template <typename TD>
   __device__ inline T gather(const TD *plane) const {
-    return off >= 0 ? (T)plane[off] : T(0);
+    const T d = (T)load_elem(plane, off);
+    return off >= 0 ? d : T(0);
+  }
+  __device__ inline T gather(plane_buf_t plane) const {
+    return buf_load(plane, off < 0 ? kOobOffset : (unsigned)off * (unsigned)sizeof(T), T());
+  }
+  // gather() in two steps, so that a caller can issue the loads of many taps before it
+  // uses any of them
+  __device__ inline void load(plane_buf_t plane, T *d) const { d[0] = gather(plane); }
+  __device__ inline T combine(const T *d) const { return d[0]; }
+  // (interface of the four-corner taps; a single corner has no rows to skip or pair)
+  __device__ inline bool row_in_use(int) const { return off >= 0; }
+  __device__ inline bool pairable() const { return false; }
+  __device__ inline void load_rows(plane_buf_t plane, T *d, bool, bool, bool) const {
+    load(plane, d);
   }
   __device__ inline void scatter(T *plane, T v) const {
     if (off >= 0) atomic_add(plane + off, v);
@@ -103,6 +155,10 @@ template <typename T, int MODE>
 struct Tap {
   int off[4];
   T wt[4];
+  // The two corners of a row are neighbours in memory (x2 == x1 + 1, both inside the plane)
+  // or both outside: one load of two elements can fetch them.  False next to the left and
+  // right border and at the seam of a wrapped column index.
+  bool pair_ok;
   __device__ inline void set(T x, T y, int h, int w) {
     const T x1f = mcx_floor(x), y1f = mcx_floor(y);
     const T x2f = x1f + T(1), y2f = y1f + T(1);
@@ -119,6 +175,7 @@ struct Tap {
     }
     const bool y1ok = y1 >= 0 && y1 <= h - 1;
     const bool y2ok = y2 >= 0 && y2 <= h - 1;
+    pair_ok = (x1ok && x2ok && x2 == x1 + 1) || (!x1ok && !x2ok);
     const T A = y2f - y, B = x2f - x, C = x - x1f, D = y - y1f;
     wt[0] = A * B;
     wt[1] = A * C;
@@ -133,11 +190,53 @@ struct Tap {
   }
   template <typename TD>
   __device__ inline T gather(const TD *plane) const {
-    const T d0 = off[0] >= 0 ? (T)plane[off[0]] : T(0);
-    const T d1 = off[1] >= 0 ? (T)plane[off[1]] : T(0);
-    const T d2 = off[2] >= 0 ? (T)plane[off[2]] : T(0);
-    const T d3 = off[3] >= 0 ? (T)plane[off[3]] : T(0);
-    return wt[0] * d0 + wt[1] * d1 + wt[2] * d2 + wt[3] * d3;
+    T d[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) d[i] = (T)load_elem(plane, off[i]);
+#pragma unroll
+    for (int i = 0; i < 4; i++) d[i] = off[i] >= 0 ? d[i] : T(0);
+    return wt[0] * d[0] + wt[1] * d[1] + wt[2] * d[2] + wt[3] * d[3];
+  }
+  __device__ inline void load(plane_buf_t plane, T *d) const {
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      d[i] = buf_load(plane, off[i] < 0 ? kOobOffset : (unsigned)off[i] * (unsigned)sizeof(T), T());
+  }
+  __device__ inline T combine(const T *d) const {
+    return wt[0] * d[0] + wt[1] * d[1] + wt[2] * d[2] + wt[3] * d[3];
+  }
+  // Row r (0: y1, 1: y2) holds a corner that is inside the plane and weighs something.
+  __device__ inline bool row_in_use(int r) const { return off[2 * r] >= 0 || off[2 * r + 1] >= 0; }
+  __device__ inline bool pairable() const { return pair_ok; }
+  // load() with three wave-uniform switches: rows no lane of the wave uses are not loaded
+  // at all, and when every lane's tap is pairable a row is one two-element load (its second
+  // element then is real data even where its weight is exactly zero, as in the reference's
+  // own arithmetic).  The texture addresser, which bounds these gathers, sees a quarter to a
+  // half of the instructions.
+  __device__ inline void load_rows(plane_buf_t plane, T *d, bool row0, bool row1,
+                                   bool pairs) const {
+    const bool rows[2] = {row0, row1};
+#pragma unroll
+    for (int r = 0; r < 2; r++) {
+      if (!rows[r]) {
+        d[2 * r] = d[2 * r + 1] = T(0);
+      } else if (pairs) {
+        const auto v = buf_load_pair(
+            plane, off[2 * r] < 0 ? kOobOffset : (unsigned)off[2 * r] * (unsigned)sizeof(T), T());
+        d[2 * r] = v.x;
+        d[2 * r + 1] = v.y;
+      } else {
+#pragma unroll
+        for (int i = 2 * r; i < 2 * r + 2; i++)
+          d[i] = buf_load(plane, off[i] < 0 ? kOobOffset : (unsigned)off[i] * (unsigned)sizeof(T),
+                          T());
+      }
+    }
+  }
+  __device__ inline T gather(plane_buf_t plane) const {
+    T d[4];
+    load(plane, d);
+    return combine(d);
   }
   __device__ inline void scatter(T *plane, T v) const {
 #pragma unroll

@@ -54,11 +54,16 @@ __device__ inline void direct_gather(const T *__restrict__ in, const T *__restri
                                      const T *__restrict__ iw, T *__restrict__ out,
                                      int64_t *__restrict__ idx, int C, int IH, int IW, int N,
                                      int K, int P, int n, int c0, int b, int cpt) {
-  // cpt: channels per thread, kPoolCH on the register-tap path below and kCH otherwise
+  // cpt: channels per thread, kPoolCH on the register-tap path below and kCH otherwise.
+  // Every loop below is free of per-lane branches: loads are unconditional (see load_elem),
+  // channels past the last one re-read the last plane (wave-uniform clamp) and are dropped
+  // at the store, so that all loads of a step are in flight together.
   const int64_t plane = (int64_t)IH * IW;
+  const unsigned plane_bytes = (unsigned)(plane * (int64_t)sizeof(T));
   const T *src = in + ((int64_t)b * C + c0) * plane;
   const int pm = P == 0 ? 1 : P;
   const int nc = min(cpt, C - c0);
+  const int64_t o = ((int64_t)b * C + c0) * N + n;
 
   if constexpr (OP != OP_RESAMPLE) {
     // Pooling with few unweighted taps: resolve them all first and walk the channels in the
@@ -73,25 +78,37 @@ __device__ inline void direct_gather(const T *__restrict__ in, const T *__restri
         const int64_t e = (int64_t)n * K + min(k, K - 1);
         taps[k].set(map[e * 2], map[e * 2 + 1], IH, IW);
       }
-      const int64_t o = ((int64_t)b * C + c0) * N + n;
+      // wave-uniform: bit k set when some lane uses row 0 / row 1 of tap k, and when every
+      // lane's tap k can fetch a row's two corners with one load
+      unsigned rows0 = 0, rows1 = 0, pairs = 0;
+#pragma unroll
+      for (int k = 0; k < kTaps; k++) {
+        rows0 |= __builtin_amdgcn_ballot_w64(taps[k].row_in_use(0)) ? 1u << k : 0u;
+        rows1 |= __builtin_amdgcn_ballot_w64(taps[k].row_in_use(1)) ? 1u << k : 0u;
+        pairs |= __builtin_amdgcn_ballot_w64(!taps[k].pairable()) ? 0u : 1u << k;
+      }
       for (int c = 0; c < nc; c++) {
-        const T *pl = src + c * plane;
+        const plane_buf_t pl = plane_buf(src + c * plane, plane_bytes);
+        // every load of the channel is issued before the first one is used (left to itself
+        // the compiler interleaves loads and waits to save registers, one load in flight)
+        T d[kTaps][Tap<T, MODE>::kCorners];
+#pragma unroll
+        for (int k = 0; k < kTaps; k++)
+          taps[k].load_rows(pl, d[k], (rows0 >> k) & 1u, (rows1 >> k) & 1u, (pairs >> k) & 1u);
+        __builtin_amdgcn_sched_barrier(0);
         T val[kTaps];
 #pragma unroll
-        for (int k = 0; k < kTaps; k++) val[k] = taps[k].gather(pl);
+        for (int k = 0; k < kTaps; k++) val[k] = taps[k].combine(d[k]);
         T a = OP == OP_MAX ? T(-3.402823466e+38F) : T(0);
         int bk = -1;
 #pragma unroll
         for (int k = 0; k < kTaps; k++) {
-          if (k < K) {
-            if (OP == OP_MAX) {
-              if (val[k] > a) {
-                a = val[k];
-                bk = k;
-              }
-            } else {
-              a += val[k];
-            }
+          if (OP == OP_MAX) {
+            const bool better = k < K && val[k] > a;
+            a = better ? val[k] : a;
+            bk = better ? k : bk;
+          } else {
+            a = k < K ? a + val[k] : a;
           }
         }
         out[o + (int64_t)c * N] = OP == OP_AVG ? a / (T)K : a;
@@ -101,6 +118,9 @@ __device__ inline void direct_gather(const T *__restrict__ in, const T *__restri
       return;
     }
   }
+  plane_buf_t pl[kCH];
+#pragma unroll
+  for (int c = 0; c < kCH; c++) pl[c] = plane_buf(src + min(c, nc - 1) * plane, plane_bytes);
   T acc[kCH];
   int64_t best[kCH];
 #pragma unroll
@@ -124,9 +144,15 @@ __device__ inline void direct_gather(const T *__restrict__ in, const T *__restri
         nx = map[(e + 1) * 2];
         ny = map[(e + 1) * 2 + 1];
       }
+      const bool row0 = __builtin_amdgcn_ballot_w64(tap.row_in_use(0)) != 0;
+      const bool row1 = __builtin_amdgcn_ballot_w64(tap.row_in_use(1)) != 0;
+      const bool pairs = __builtin_amdgcn_ballot_w64(!tap.pairable()) == 0;
+      T d[kCH][Tap<T, MODE>::kCorners];
 #pragma unroll
-      for (int c = 0; c < kCH; c++)
-        if (c < nc) val[c] = tap.gather(src + c * plane);
+      for (int c = 0; c < kCH; c++) tap.load_rows(pl[c], d[c], row0, row1, pairs);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int c = 0; c < kCH; c++) val[c] = tap.combine(d[c]);
     } else {
 #pragma unroll
       for (int c = 0; c < kCH; c++) val[c] = T(0);
@@ -134,19 +160,23 @@ __device__ inline void direct_gather(const T *__restrict__ in, const T *__restri
         Tap<T, MODE> tap;
         tap.set(map[(e + p) * 2], map[(e + p) * 2 + 1], IH, IW);
         const T w = iw[e + p];
+        const bool row0 = __builtin_amdgcn_ballot_w64(tap.row_in_use(0)) != 0;
+        const bool row1 = __builtin_amdgcn_ballot_w64(tap.row_in_use(1)) != 0;
+        const bool pairs = __builtin_amdgcn_ballot_w64(!tap.pairable()) == 0;
+        T d[kCH][Tap<T, MODE>::kCorners];
 #pragma unroll
-        for (int c = 0; c < kCH; c++)
-          if (c < nc) val[c] += w * tap.gather(src + c * plane);
+        for (int c = 0; c < kCH; c++) tap.load_rows(pl[c], d[c], row0, row1, pairs);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int c = 0; c < kCH; c++) val[c] += w * tap.combine(d[c]);
       }
     }
 #pragma unroll
     for (int c = 0; c < kCH; c++) {
-      if (c >= nc) continue;
       if (OP == OP_MAX) {
-        if (val[c] > acc[c]) {
-          acc[c] = val[c];
-          best[c] = e * 2;
-        }
+        const bool better = val[c] > acc[c];
+        acc[c] = better ? val[c] : acc[c];
+        best[c] = better ? e * 2 : best[c];
       } else if (OP == OP_AVG) {
         acc[c] += val[c];
       } else {
@@ -154,7 +184,6 @@ __device__ inline void direct_gather(const T *__restrict__ in, const T *__restri
       }
     }
   }
-  const int64_t o = ((int64_t)b * C + c0) * N + n;
 #pragma unroll
   for (int c = 0; c < kCH; c++) {
     if (c >= nc) continue;
@@ -525,7 +554,13 @@ __global__ __launch_bounds__(kThreads) void transposed_gather_kernel(
             const uint32_t cd = code[g * kGroup + j];
             const uint32_t n = OP == UN_MAX ? cd / (uint32_t)K : cd;
             v[j] = sc[n];
-            keep[j] = OP == UN_MAX ? ic[n] == (int64_t)cd * idx_scale : true;
+            // Entries past the end of a lane's list are dropped by a test, not by their zero
+            // weight (an Inf or NaN in an unrelated source element must not reach the
+            // destination).  Max unpooling keeps the recorded-winner test alone: its padded
+            // entries repeat the lane's own first entry with weight zero, and the extra test
+            // cost it a third of its speed.
+            keep[j] = OP == UN_MAX ? ic[n] == (int64_t)cd * idx_scale
+                                   : (uint32_t)(g * kGroup + j) < len;
           }
 #pragma unroll
           for (int j = 0; j < kGroup; j++)
@@ -540,17 +575,19 @@ __global__ __launch_bounds__(kThreads) void transposed_gather_kernel(
 #pragma unroll
   for (int c = 0; c < kTCH; c++) acc[c] = T(0);
   // kUnroll entries per trip so that their loads are in flight together; entries past
-  // the end repeat the last valid one with weight zero.
+  // the end repeat the last valid one and are dropped (by a test, not by a zero weight: an Inf
+  // or NaN in an unrelated source element must not reach the destination).
   constexpr int kUnroll = OP == UN_RESAMPLE ? 2 : 4;
   for (uint32_t e = start; e < end; e += kUnroll) {
     uint32_t code[kUnroll];
     T w[kUnroll];
+    bool in[kUnroll];
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
-      const bool in = e + u < end;
-      const uint32_t ee = in ? e + u : e;
+      in[u] = e + u < end;
+      const uint32_t ee = in[u] ? e + u : e;
       code[u] = e_src[ee];
-      w[u] = in ? e_wt[ee] : T(0);
+      w[u] = e_wt[ee];
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
@@ -560,10 +597,10 @@ __global__ __launch_bounds__(kThreads) void transposed_gather_kernel(
       for (int c = 0; c < kTCH; c++) {
         if (c >= nc) continue;
         if (OP == UN_MAX) {
-          if (i0[(int64_t)c * nsrc + n] == want)
-            acc[c] = mcx_fma(w[u], s0[(int64_t)c * nsrc + n], acc[c]);
+          const bool hit = i0[(int64_t)c * nsrc + n] == want;
+          if (in[u] & hit) acc[c] = mcx_fma(w[u], s0[(int64_t)c * nsrc + n], acc[c]);
         } else {
-          acc[c] = mcx_fma(w[u], s0[(int64_t)c * nsrc + n], acc[c]);
+          if (in[u]) acc[c] = mcx_fma(w[u], s0[(int64_t)c * nsrc + n], acc[c]);
         }
       }
     }
@@ -698,6 +735,11 @@ int launch_scatter(const void *in, const void *map, const void *iw, void *out, i
   return 0;
 }
 
+// Samples are addressed with 32-bit byte offsets inside a plane (see plane_buf).
+bool plane_beyond_4gib(int64_t pixels, int dtype) {
+  return pixels * (dtype == MCX_F64 ? 8 : 4) > (int64_t)kOobOffset;
+}
+
 int check_common(const void *a, const void *map, const void *iw, const void *o, int64_t P,
                  int dtype) {
   if (dtype != MCX_F32 && dtype != MCX_F64) return MCX_E_DTYPE;
@@ -721,7 +763,8 @@ extern "C" int mcx_resample_from_map(const void *src, const void *map, const voi
                                      int64_t B, int64_t C, int64_t SH, int64_t SW, int64_t MH,
                                      int64_t MW, int64_t P, int interp, int dtype, void *stream) {
   if (int rc = check_common(src, map, iw, dst, P, dtype)) return rc;
-  if (bad_dims({B, C, SH, SW, MH, MW, SH * SW, MH * MW, MH * MW * (P ? P : 1) * 2}) || B > 65535)
+  if (bad_dims({B, C, SH, SW, MH, MW, SH * SW, MH * MW, MH * MW * (P ? P : 1) * 2}) || B > 65535 ||
+      plane_beyond_4gib(SH * SW, dtype))
     return MCX_E_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == MCX_F32)
@@ -785,7 +828,9 @@ extern "C" int mcx_max_pool(const void *in, const void *map, const void *iw, voi
                             void *stream) {
   if (int rc = check_common(in, map, iw, out, P, dtype)) return rc;
   if (!idx) return MCX_E_NULL;
-  if (bad_dims({B, C, IH, IW, OH, OW, K, IH * IW, OH * OW}) || B > 65535) return MCX_E_SHAPE;
+  if (bad_dims({B, C, IH, IW, OH, OW, K, IH * IW, OH * OW}) || B > 65535 ||
+      plane_beyond_4gib(IH * IW, dtype))
+    return MCX_E_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == MCX_F32)
     return launch_gather<float, OP_MAX>(in, map, iw, out, idx, B, C, IH, IW, OH, OW, K, P, interp,
@@ -798,7 +843,9 @@ extern "C" int mcx_avg_pool(const void *in, const void *map, const void *iw, voi
                             int64_t C, int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
                             int64_t P, int interp, int dtype, void *stream) {
   if (int rc = check_common(in, map, iw, out, P, dtype)) return rc;
-  if (bad_dims({B, C, IH, IW, OH, OW, K, IH * IW, OH * OW}) || B > 65535) return MCX_E_SHAPE;
+  if (bad_dims({B, C, IH, IW, OH, OW, K, IH * IW, OH * OW}) || B > 65535 ||
+      plane_beyond_4gib(IH * IW, dtype))
+    return MCX_E_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == MCX_F32)
     return launch_gather<float, OP_AVG>(in, map, iw, out, nullptr, B, C, IH, IW, OH, OW, K, P,

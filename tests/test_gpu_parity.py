@@ -785,3 +785,24 @@ def test_knn_sphere_invariants(device):
     full = torch.cdist(qry[0][:, sample].t().double(), ref[0].t().double())
     kth = full.sort(-1).values[:, 7]
     torch.testing.assert_close(dist[0, 7, sample].double(), kth, rtol=1e-5, atol=1e-6)
+
+
+def test_scatter_as_gather_keeps_infinities_where_they_belong(device):
+    """A non-finite source value reaches the destinations its own taps touch and no others:
+    destinations that receive nothing stay exactly zero (padded list entries are dropped, not
+    multiplied by a zero weight)."""
+    B, C, IH, IW, OH, OW = 1, 3, 12, 20, 9, 11
+    x = torch.ones(B, C, IH, IW)
+    x[:, :, 0, 0] = float("inf")       # source element 0: what an empty list would re-read
+    smap = torch.zeros(IH, IW, 2)
+    smap[..., 0] = 4.25
+    smap[..., 1] = 5.5                  # everything lands around (5..6, 4..5)
+    want = O.resample_to_map(x, smap, OH, OW, 1)
+    got = _C.resample_to_map(x.cuda(), smap.cuda(), OH, OW, 1).cpu()
+    assert torch.equal(torch.isinf(got), torch.isinf(want))
+    assert (got[~torch.isinf(want)] == 0).all() and not torch.isnan(got).any()
+    K = 2
+    pmap = smap[:, :, None, :].repeat(1, 1, K, 1).contiguous()
+    want = O.mapped_avg_unpool(x, pmap, OH, OW, K, 1)
+    got = _C.mapped_avg_unpool(x.cuda(), pmap.cuda(), OH, OW, K, 1).cpu()
+    assert torch.equal(torch.isinf(got), torch.isinf(want)) and not torch.isnan(got).any()
