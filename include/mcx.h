@@ -268,6 +268,27 @@ int mcx_cube_projection_map(float *out, int64_t cube_dim, int64_t kh, int64_t kw
 int mcx_cube2rect(const void *cubemap, void *rect, int64_t C, int64_t cube_dim, int64_t RH,
                   int64_t RW, int interp, int dtype, void *stream);
 
+/* ---- icosphere map operators -------------------------------------------------- */
+
+/* get_planar_conv_operator_from_samples: package/ext_modules/include/util/cpp/sphere.h:131-175
+ * (binding), package/ext_modules/src/util/cpp/sphere.cpp:1117-1270 (driver), :1055-1105
+ * (Sphere::_isPointInFace), :1007-1053 (face search); Python caller
+ * package/layers/util/icosphere_functions.py:226-262.  For each of N sample directions
+ * samples [N, 2] = (longitude, latitude) in radians: the face of the triangle mesh
+ * (vertices [V, 3] float, faces [F, 3] int64, a closed mesh around the origin) that the ray
+ * pierces -> face_idx [N] int64 (-1: none), vertex_idx [N, 3] int64 (the face's vertices in
+ * reverse order, as the reference lists them) and weights [N, 3] float (barycentric s, t, u of
+ * the pierced point; `nearest` != 0: one-hot at the largest).  The mesh is the caller's: the
+ * reference's own module walks its private icosphere hierarchy on the host; to reproduce it
+ * pass the vertices and faces of that icosphere.  Where a sample is within the face test's
+ * tolerance (1e-3) of an edge, several faces pass; this library returns the one it lies
+ * deepest inside.  workspace: mcx_planar_conv_operator_workspace(F) bytes. */
+size_t mcx_planar_conv_operator_workspace(int64_t F);
+int mcx_planar_conv_operator(const float *samples, const float *vertices, const int64_t *faces,
+                             int64_t *face_idx, int64_t *vertex_idx, float *weights,
+                             void *workspace, size_t workspace_bytes, int64_t N, int64_t V,
+                             int64_t F, int nearest, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

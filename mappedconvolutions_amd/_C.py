@@ -639,3 +639,43 @@ def cube2rect(cubemap, rect_height, rect_width, interpolation):
                                        _stream(cubemap))
     _lib.check(rc, "cube2rect")
     return rect
+
+
+# ------------------------------------------------------------ icosphere map operators
+def planar_conv_operator_from_samples(samples, vertices, faces, keepdim=True, nearest=False):
+    """Sphere.get_planar_conv_operator_from_samples of the reference's `_sphere` module
+    (package/ext_modules/src/util/cpp/sphere.cpp:1117-1270) over a caller-supplied mesh.
+
+    samples [OH, OW, K, 2] or [OH, OW, 2] (longitude, latitude), float32, on the GPU;
+    vertices [V, 3] float32 and faces [F, 3] int64 of a closed triangle mesh around the
+    origin.  Returns [face_idx [OH, OW, K] int64, vertex_idx [OH, OW, K, 3] int64,
+    weights [OH, OW, K, 3] float32]; a [OH, OW, 2] input without `keepdim` drops the K axis,
+    as in the reference."""
+    _contig(samples=samples, vertices=vertices, faces=faces)
+    _on_gpu("samples", samples, vertices=vertices, faces=faces)
+    if samples.dtype != torch.float32 or vertices.dtype != torch.float32:
+        raise RuntimeError("samples and vertices must be float32")
+    if faces.dtype != torch.int64:
+        raise RuntimeError("faces must be int64")
+    if samples.dim() not in (3, 4) or samples.shape[-1] != 2:
+        raise RuntimeError("samples must be [OH, OW, K, 2] or [OH, OW, 2]")
+    if vertices.dim() != 2 or vertices.shape[1] != 3 or faces.dim() != 2 or faces.shape[1] != 3:
+        raise RuntimeError("vertices must be [V, 3] and faces [F, 3]")
+    lead = tuple(samples.shape[:-1])
+    if samples.dim() == 3 and keepdim:
+        lead = lead + (1,)
+    N, V, F = samples.numel() // 2, vertices.shape[0], faces.shape[0]
+    dev = samples.device
+    face_idx = torch.empty(lead, dtype=torch.int64, device=dev)
+    vertex_idx = torch.empty(lead + (3,), dtype=torch.int64, device=dev)
+    weights = torch.empty(lead + (3,), dtype=torch.float32, device=dev)
+    lib = _lib.load()
+    ws_bytes = lib.mcx_planar_conv_operator_workspace(F)
+    ws = _workspace(ws_bytes, dev)
+    with torch.cuda.device(dev):
+        rc = lib.mcx_planar_conv_operator(_ptr(samples), _ptr(vertices), _ptr(faces),
+                                          _ptr(face_idx), _ptr(vertex_idx), _ptr(weights),
+                                          _ptr(ws), ws_bytes, N, V, F, 1 if nearest else 0,
+                                          _stream(samples))
+    _lib.check(rc, "planar_conv_operator_from_samples")
+    return [face_idx, vertex_idx, weights]

@@ -36,6 +36,65 @@ _EXT_MODULES = {
 }
 
 
+# Modules of the reference's extension package that lie outside this backend's path.  The
+# plain convolution pair is the reference's timing baseline, a re-implementation of the library
+# convolution (package/ext_modules/include/nn/layers/convolution_layer.h:64-143,
+# transposed_convolution_layer.h): registered as thin calls of that library routine so that
+# the reference's `nn/__init__` imports and its baseline layers run.  `_sphere` is a host-side
+# half-edge mesh class (include/util/cpp/sphere.h:131-175): its name resolves, its use raises.
+def _plain_conv_module():
+    import torch
+    import torch.nn.functional as F
+    m = types.ModuleType("_mapped_convolution_ext._convolution")
+
+    def conv_forward(input, weight, bias, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w,
+                     dilation_h, dilation_w):
+        return F.conv2d(input, weight, bias, (stride_h, stride_w), (pad_h, pad_w),
+                        (dilation_h, dilation_w))
+
+    def conv_backward(grad_output, input, weight, bias, kernel_h, kernel_w, stride_h, stride_w,
+                      pad_h, pad_w, dilation_h, dilation_w):
+        gi, gw, gb = torch.ops.aten.convolution_backward(
+            grad_output, input, weight, [bias.numel()], [stride_h, stride_w], [pad_h, pad_w],
+            [dilation_h, dilation_w], False, [0, 0], 1, [True, True, True])
+        return [gi, gw, gb]
+
+    m.conv_forward, m.conv_backward = conv_forward, conv_backward
+    return m
+
+
+def _plain_transposed_conv_module():
+    import torch
+    import torch.nn.functional as F
+    m = types.ModuleType("_mapped_convolution_ext._transposed_convolution")
+
+    def transposed_conv_forward(input, weight, bias, kernel_h, kernel_w, stride_h, stride_w,
+                                pad_h, pad_w, dilation_h, dilation_w):
+        return F.conv_transpose2d(input, weight, bias, (stride_h, stride_w), (pad_h, pad_w), 0,
+                                  1, (dilation_h, dilation_w))
+
+    def transposed_conv_backward(grad_output, input, weight, bias, kernel_h, kernel_w, stride_h,
+                                 stride_w, pad_h, pad_w, dilation_h, dilation_w):
+        gi, gw, gb = torch.ops.aten.convolution_backward(
+            grad_output, input, weight, [bias.numel()], [stride_h, stride_w], [pad_h, pad_w],
+            [dilation_h, dilation_w], True, [0, 0], 1, [True, True, True])
+        return [gi, gw, gb]
+
+    m.transposed_conv_forward = transposed_conv_forward
+    m.transposed_conv_backward = transposed_conv_backward
+    return m
+
+
+class _HostOnlyModule(types.ModuleType):
+    def __getattr__(self, name):
+        if name.startswith("__"):
+            raise AttributeError(name)
+        raise RuntimeError(
+            "%s.%s: the reference's host-side mesh tools are not part of this GPU backend; "
+            "pass mesh tensors to mappedconvolutions_amd.util.vertex_to_vertex_kernel_map / "
+            "_C.planar_conv_operator_from_samples instead" % (self.__name__, name))
+
+
 def install_aliases(ext_only=False):
     """Make `import mapped_convolution.nn` and
     `import _mapped_convolution_ext._mapped_convolution` resolve to this package.
@@ -59,3 +118,7 @@ def install_aliases(ext_only=False):
             setattr(m, op, getattr(_C, op))
         sys.modules.setdefault(m.__name__, m)
         setattr(sys.modules["_mapped_convolution_ext"], mod_name, m)
+    for m in (_plain_conv_module(), _plain_transposed_conv_module(),
+              _HostOnlyModule("_mapped_convolution_ext._sphere")):
+        sys.modules.setdefault(m.__name__, m)
+        setattr(sys.modules["_mapped_convolution_ext"], m.__name__.rsplit(".", 1)[1], m)

@@ -45,6 +45,8 @@ SIGNATURES = {
     "mcx_projection_map": (_i, [_p] + [_i64] * 4 + [_i] + [_i64] * 2 + [_p]),
     "mcx_cube_projection_map": (_i, [_p] + [_i64] * 4 + [_p]),
     "mcx_cube2rect": (_i, [_p] * 2 + [_i64] * 4 + [_i, _i, _p]),
+    "mcx_planar_conv_operator_workspace": (_sz, [_i64]),
+    "mcx_planar_conv_operator": (_i, [_p] * 7 + [_sz] + [_i64] * 3 + [_i, _p]),
 }
 
 _lib = None

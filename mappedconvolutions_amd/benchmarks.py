@@ -139,6 +139,16 @@ def maps(dev):
     _line("cube projection map dim 256 3x3",
           _time(lambda: get_reverse_cube_projection_map(256, (3, 3), device=dev)),
           nbytes=256 * 1536 * 9 * 2 * 4)
+    # the real maps of a mesh convolution at config 3's size: 7 taps at each of 40962 vertices
+    from .util import gnomonic_kernel, convert_3d_to_spherical
+    verts, faces = synthetic.subdivided_icosahedron(6)
+    verts, faces = verts.to(dev), faces.to(dev)
+    samples = gnomonic_kernel(convert_3d_to_spherical(verts), 1, 7, 0.02, 0.02).contiguous()
+    n, f = samples.numel() // 2, faces.shape[0]
+    _line("planar conv operator: %d samples x %d faces" % (n, f),
+          _time(lambda: _C.planar_conv_operator_from_samples(samples, verts, faces, True, False),
+                iters=3, warmup=1),
+          flops=6.0 * n * f, peak_tflops=FP32_VALU_TFLOPS, bound="valu")
     cube = torch.rand(64, 256, 6 * 256, device=dev)
     for interp in ("nearest", "bilinear"):
         _line("cube2rect %s C=64 dim 256 -> 512x1024" % interp,

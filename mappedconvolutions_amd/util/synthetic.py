@@ -116,3 +116,32 @@ def upsampling_map(src_height, src_width, factor, radius=1, latitude=False, alig
         y = cy + dy + 0 * j
     out = np.stack([np.broadcast_to(x, y.shape), y], axis=-1)
     return torch.from_numpy(np.ascontiguousarray(out)).to(dtype)
+
+
+def subdivided_icosahedron(order):
+    """Triangle mesh of the unit sphere: midpoint subdivision of the icosahedron, every new
+    vertex pushed onto the sphere (10 * 4^order + 2 vertices, 20 * 4^order faces).  Not the
+    reference's Loop-subdivided icosphere, whose vertex order differs.  Returns
+    (vertices [V, 3] float32, faces [F, 3] int64)."""
+    r = (1.0 + 5 ** 0.5) / 2
+    v = [(-1, r, 0), (1, r, 0), (-1, -r, 0), (1, -r, 0), (0, -1, r), (0, 1, r), (0, -1, -r),
+         (0, 1, -r), (r, 0, -1), (r, 0, 1), (-r, 0, -1), (-r, 0, 1)]
+    f = [(0, 11, 5), (0, 5, 1), (0, 1, 7), (0, 7, 10), (0, 10, 11), (1, 5, 9), (5, 11, 4),
+         (11, 10, 2), (10, 7, 6), (7, 1, 8), (3, 9, 4), (3, 4, 2), (3, 2, 6), (3, 6, 8),
+         (3, 8, 9), (4, 9, 5), (2, 4, 11), (6, 2, 10), (8, 6, 7), (9, 8, 1)]
+    v = [np.array(p, np.float64) / np.linalg.norm(p) for p in v]
+    for _ in range(order):
+        cache, nf = {}, []
+
+        def mid(a, b):
+            key = (min(a, b), max(a, b))
+            if key not in cache:
+                m = v[a] + v[b]
+                v.append(m / np.linalg.norm(m))
+                cache[key] = len(v) - 1
+            return cache[key]
+        for a, b, c in f:
+            ab, bc, ca = mid(a, b), mid(b, c), mid(c, a)
+            nf += [(a, ab, ca), (b, bc, ab), (c, ca, bc), (ab, bc, ca)]
+        f = nf
+    return (torch.from_numpy(np.array(v, np.float32)), torch.from_numpy(np.array(f, np.int64)))

@@ -35,10 +35,14 @@ MODULES = {
 }
 
 
-def _compile(ref_root, name, base, verbose):
+# the host-side icosphere tools (package/setup.py:86-94): one source under src/util/cpp
+UTIL_MODULES = {"_sphere": "sphere"}
+
+
+def _compile(ref_root, name, base, verbose, subdir="nn"):
     import torch
     from torch.utils import cpp_extension as ce
-    src = os.path.join(ref_root, "package/ext_modules/src/nn/cpp", base + ".cpp")
+    src = os.path.join(ref_root, "package/ext_modules/src", subdir, "cpp", base + ".cpp")
     inc = os.path.join(ref_root, "package/ext_modules/include")
     out = os.path.join(OUT, name + ".so")
     torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
@@ -63,6 +67,8 @@ def build(ref_root="/root/reference", verbose=False, jobs=4):
     os.makedirs(OUT, exist_ok=True)
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         futs = [ex.submit(_compile, ref_root, n, b, verbose) for n, b in MODULES.items()]
+        futs += [ex.submit(_compile, ref_root, n, b, verbose, "util")
+                 for n, b in UTIL_MODULES.items()]
         return [f.result() for f in futs]
 
 
