@@ -203,14 +203,19 @@ int mcx_tconv_backward(const void *gy, const void *map, const void *iw, const vo
                        int dtype, void *stream);
 
 /* Map plan: no counterpart in the reference, which decodes sample_map inside its kernels at
- * every call.  A training loop applies the same sample_map at every step, so what the
- * backward derives from the map alone - the transposed map of its input gradient and the
- * "which pairs are in use" masks - can be built once and reused.  A plan belongs to one
- * (sample_map, interp_weights, interp, IH x IW, OH x OW, K, P); the caller rebuilds it when
- * the map's contents change.  mcx_conv_plan_bytes is 0 where no plan exists (F64, P > 4):
- * pass NULL, 0 then.  mcx_conv_backward_planned is mcx_conv_backward with the plan in place
- * of the per-call build (plan NULL: identical to mcx_conv_backward); it only reads the plan,
- * so one plan may serve concurrent calls. */
+ * every call.  A network applies the same sample_map at every step, so everything that depends
+ * on the map alone can be built once and reused: the transposed map of the scatter direction
+ * (convolution backward-input, transposed-convolution forward), the taps of the gather
+ * direction resolved to (offset, weight) pairs (convolution forward, transposed-convolution
+ * backward-input; maps of at most four pairs per tap), and the "which pairs are in use" masks
+ * (all of them and the weight gradients).  A plan belongs to one (sample_map, interp_weights,
+ * interp, sampled image, map size, K, P).  In mcx_conv_plan_bytes / _build, IH x IW is the image
+ * the map samples and OH x OW the map's spatial size: a convolution passes its input and
+ * output sizes, a transposed convolution its OUTPUT size as (IH, IW) and its INPUT size as
+ * (OH, OW).  The caller rebuilds the plan when the map's contents change.  mcx_conv_plan_bytes
+ * is 0 where no plan exists (F64, P > 4): pass NULL, 0 then.  The _planned entry points are the
+ * plain ones with the plan in place of the per-call build (plan NULL: identical to the plain
+ * call); they only read the plan, so one plan may serve concurrent calls. */
 size_t mcx_conv_plan_bytes(int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P,
                            int dtype);
 int mcx_conv_plan_build(const void *map, const void *iw, void *plan, size_t plan_bytes,
@@ -222,6 +227,48 @@ int mcx_conv_backward_planned(const void *gy, const void *map, const void *iw, c
                               int64_t B, int64_t Ci, int64_t Co, int64_t IH, int64_t IW,
                               int64_t OH, int64_t OW, int64_t K, int64_t P, int interp, int dtype,
                               void *stream);
+
+/* Scatter plans: no counterpart in the reference.  resample_to_map and the two unpoolings run
+ * as gathers through the transposed form of their sample map (per destination pixel the sorted
+ * list of (source, weight) contributions); built per call that is a third of a call's time, and
+ * it depends on the map alone.  mcx_scatter_plan_build writes it once into a caller-owned buffer
+ * of mcx_scatter_plan_bytes(); the _planned entry points take it in place of (map, iw,
+ * workspace) and only read it.  MH x MW: the sample map's spatial size (the source of the
+ * scatter); DH x DW: the image scattered into; K = 1 for resample_to_map.  A plan built with
+ * for_max_unpool != 0 records the tap of every contribution and serves mcx_max_unpool_planned
+ * only; one built with 0 serves the other two.  F32 and F64. */
+size_t mcx_scatter_plan_bytes(int64_t MH, int64_t MW, int64_t DH, int64_t DW, int64_t K, int64_t P,
+                              int interp, int dtype);
+int mcx_scatter_plan_build(const void *map, const void *iw, void *plan, size_t plan_bytes,
+                           int64_t MH, int64_t MW, int64_t DH, int64_t DW, int64_t K, int64_t P,
+                           int interp, int dtype, int for_max_unpool, void *stream);
+int mcx_resample_to_map_planned(const void *in, const void *plan, size_t plan_bytes, void *out,
+                                int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t OH,
+                                int64_t OW, int64_t P, int interp, int dtype, void *stream);
+int mcx_avg_unpool_planned(const void *gout, const void *plan, size_t plan_bytes, void *gin,
+                           int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t OH, int64_t OW,
+                           int64_t K, int64_t P, int interp, int dtype, void *stream);
+int mcx_max_unpool_planned(const void *gout, const int64_t *idx, const void *plan,
+                           size_t plan_bytes, void *gin, int64_t B, int64_t C, int64_t IH,
+                           int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
+                           int dtype, void *stream);
+
+int mcx_conv_forward_planned(const void *x, const void *map, const void *iw, const void *w,
+                             const void *bias, void *y, void *workspace, size_t workspace_bytes,
+                             const void *plan, size_t plan_bytes, int64_t B, int64_t Ci,
+                             int64_t Co, int64_t IH, int64_t IW, int64_t OH, int64_t OW,
+                             int64_t K, int64_t P, int interp, int dtype, void *stream);
+int mcx_tconv_forward_planned(const void *x, const void *map, const void *iw, const void *w,
+                              const void *bias, void *y, void *workspace, size_t workspace_bytes,
+                              const void *plan, size_t plan_bytes, int64_t B, int64_t Ci,
+                              int64_t Co, int64_t IH, int64_t IW, int64_t OH, int64_t OW,
+                              int64_t K, int64_t P, int interp, int dtype, void *stream);
+int mcx_tconv_backward_planned(const void *gy, const void *map, const void *iw, const void *x,
+                               const void *w, void *gx, void *gw, void *gb, void *workspace,
+                               size_t workspace_bytes, const void *plan, size_t plan_bytes,
+                               int64_t B, int64_t Ci, int64_t Co, int64_t IH, int64_t IW,
+                               int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
+                               int dtype, void *stream);
 
 /* ---- KNN -------------------------------------------------------------------- */
 

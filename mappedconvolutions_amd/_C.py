@@ -114,7 +114,8 @@ def _weighted_dims(sample_map, interp_weights, kernel):
 
 
 # --------------------------------------------------------------------------- conv
-def _conv_forward(input, sample_map, interp_weights, weight, bias, kernel_size, interpolation):
+def _conv_forward(input, sample_map, interp_weights, weight, bias, kernel_size, interpolation,
+                  plan=None):
     _contig(input=input, sample_map=sample_map, interp_weights=interp_weights, weight=weight,
             bias=bias)
     _on_gpu("input", input, sample_map=sample_map, interp_weights=interp_weights, weight=weight,
@@ -133,22 +134,27 @@ def _conv_forward(input, sample_map, interp_weights, weight, bias, kernel_size, 
     lib = _lib.load()
     ws_bytes = lib.mcx_conv_forward_workspace(B, Ci, Co, IH, IW, OH, OW, K, P, dt)
     ws = _workspace(ws_bytes, input.device)
+    if plan is None and map_plan_cache is not None:
+        plan = _cached_plan(sample_map, interp_weights, IH, IW, interpolation, input.dtype)
+    plan_bytes = 0 if plan is None else plan.numel()
     with torch.cuda.device(input.device):
-        rc = _timed("conv_forward", input.device, lambda: lib.mcx_conv_forward(
+        rc = _timed("conv_forward", input.device, lambda: lib.mcx_conv_forward_planned(
             _ptr(input), _ptr(sample_map), _ptr(interp_weights), _ptr(weight), _ptr(bias),
-            _ptr(out), _ptr(ws), ws_bytes, B, Ci, Co, IH, IW, OH, OW, K, P, int(interpolation),
-            dt, _stream(input)))
+            _ptr(out), _ptr(ws), ws_bytes, _ptr(plan), plan_bytes, B, Ci, Co, IH, IW, OH, OW, K,
+            P, int(interpolation), dt, _stream(input)))
     _lib.check(rc, "mapped_conv_forward")
     return out
 
 
 # ---- map plans (no counterpart in the reference) ------------------------------------
-# What the convolution backward derives from sample_map alone (the transposed map of the
-# input gradient and the masks of pairs in use) can be built once and reused while the map
-# does not change.  `conv_map_plan` builds such a plan explicitly; with `map_plan_cache` set
-# to a dict (see enable_map_plan_cache) the backward ops keep the plans of the maps they
-# have seen, keyed by the tensors' storage and in-place version counters.  Off by default:
-# every call then rebuilds what it needs, like the reference.
+# What the operators derive from sample_map alone can be built once and reused while the map
+# does not change: for the (transposed) convolutions the transposed map of the scatter
+# direction, the resolved taps of the gather direction and the masks of pairs in use
+# (`conv_map_plan`); for resample_to_map and the unpoolings the sorted per-destination lists of
+# contributions (`scatter_map_plan`).  With `map_plan_cache` set to a dict (see
+# enable_map_plan_cache) the ops keep the plans of the maps they have seen, keyed by the
+# tensors' storage and in-place version counters.  Off by default: every call then rebuilds
+# what it needs, like the reference.
 map_plan_cache = None
 _MAP_PLAN_CACHE_ENTRIES = 16
 
@@ -161,10 +167,11 @@ def enable_map_plan_cache(enabled=True):
 
 def conv_map_plan(sample_map, interp_weights, input_height, input_width, interpolation,
                   data_dtype=torch.float32):
-    """Plan of a MappedConvolution's backward for one sample_map [OH, OW, K, (P,) 2] over an
-    input of input_height x input_width; None where the library has no plan for the case
-    (float64 data, P > 4).  Pass it as `plan=` to mapped_conv_backward /
-    weighted_mapped_conv_backward for as long as the map's contents stay the same."""
+    """Plan of one sample_map [MH, MW, K, (P,) 2] that samples an image of input_height x
+    input_width: a MappedConvolution's input, or a MappedTransposedConvolution's OUTPUT.  None
+    where the library has no plan for the case (float64 data, P > 4).  Pass it as `plan=` to
+    the forward and backward ops of that layer for as long as the map's contents stay the
+    same."""
     _contig(sample_map=sample_map, interp_weights=interp_weights)
     _on_gpu("sample_map", sample_map, interp_weights=interp_weights)
     P = _weighted_dims(sample_map, interp_weights, True)
@@ -187,16 +194,21 @@ def conv_map_plan(sample_map, interp_weights, input_height, input_width, interpo
     return plan
 
 
-def _cached_plan(sample_map, interp_weights, IH, IW, interpolation, data_dtype):
+def _cached_plan(sample_map, interp_weights, IH, IW, interpolation, data_dtype, kind="conv",
+                 **scatter_args):
     """Plan from the cache, rebuilt when a tensor was modified in place or replaced."""
     def ident(t):
         return None if t is None else (t.data_ptr(), t._version, tuple(t.shape))
-    key = (ident(sample_map), ident(interp_weights), IH, IW, int(interpolation), data_dtype,
+    key = (kind, ident(sample_map), ident(interp_weights), IH, IW, int(interpolation), data_dtype,
            sample_map.device.index)
     hit = map_plan_cache.get(key)
     if hit is not None:
         return hit[0]
-    plan = conv_map_plan(sample_map, interp_weights, IH, IW, interpolation, data_dtype)
+    if kind == "conv":
+        plan = conv_map_plan(sample_map, interp_weights, IH, IW, interpolation, data_dtype)
+    else:
+        plan = scatter_map_plan(sample_map, interp_weights, IH, IW, interpolation,
+                                for_max_unpool=kind == "max_unpool", **scatter_args)
     if len(map_plan_cache) >= _MAP_PLAN_CACHE_ENTRIES:
         map_plan_cache.pop(next(iter(map_plan_cache)))
     # the entry keeps the tensors alive, so their addresses cannot be handed to other maps
@@ -243,9 +255,10 @@ def _conv_backward(grad_output, sample_map, interp_weights, input, weight, bias,
     return [grad_input, grad_weight, grad_bias]
 
 
-def mapped_conv_forward(input, sample_map, weight, bias, kernel_size, interpolation):
-    """include/nn/layers/mapped_convolution_layer.h:64-66."""
-    return _conv_forward(input, sample_map, None, weight, bias, kernel_size, interpolation)
+def mapped_conv_forward(input, sample_map, weight, bias, kernel_size, interpolation, plan=None):
+    """include/nn/layers/mapped_convolution_layer.h:64-66.  `plan` (optional, not in the
+    reference): see conv_map_plan."""
+    return _conv_forward(input, sample_map, None, weight, bias, kernel_size, interpolation, plan)
 
 
 def mapped_conv_backward(grad_output, sample_map, input, weight, bias, kernel_size, interpolation,
@@ -257,10 +270,10 @@ def mapped_conv_backward(grad_output, sample_map, input, weight, bias, kernel_si
 
 
 def weighted_mapped_conv_forward(input, sample_map, interp_weights, weight, bias, kernel_size,
-                                 interpolation):
-    """include/nn/layers/weighted_mapped_convolution_layer.h:65-68."""
+                                 interpolation, plan=None):
+    """include/nn/layers/weighted_mapped_convolution_layer.h:65-68.  `plan`: see conv_map_plan."""
     return _conv_forward(input, sample_map, interp_weights, weight, bias, kernel_size,
-                         interpolation)
+                         interpolation, plan)
 
 
 def weighted_mapped_conv_backward(grad_output, sample_map, interp_weights, input, weight, bias,
@@ -272,7 +285,7 @@ def weighted_mapped_conv_backward(grad_output, sample_map, interp_weights, input
 
 # ---------------------------------------------------------------- transposed conv
 def _tconv_forward(input, sample_map, interp_weights, weight, bias, output_height, output_width,
-                   kernel_size, interpolation):
+                   kernel_size, interpolation, plan=None):
     _contig(input=input, sample_map=sample_map, interp_weights=interp_weights, weight=weight,
             bias=bias)
     _on_gpu("input", input, sample_map=sample_map, interp_weights=interp_weights, weight=weight,
@@ -288,17 +301,20 @@ def _tconv_forward(input, sample_map, interp_weights, weight, bias, output_heigh
     lib = _lib.load()
     ws_bytes = lib.mcx_tconv_forward_workspace(B, Ci, Co, IH, IW, OH, OW, K, P, dt)
     ws = _workspace(ws_bytes, input.device)
+    if plan is None and map_plan_cache is not None:
+        plan = _cached_plan(sample_map, interp_weights, OH, OW, interpolation, input.dtype)
+    plan_bytes = 0 if plan is None else plan.numel()
     with torch.cuda.device(input.device):
-        rc = lib.mcx_tconv_forward(_ptr(input), _ptr(sample_map), _ptr(interp_weights),
-                                   _ptr(weight), _ptr(bias), _ptr(out), _ptr(ws), ws_bytes, B, Ci,
-                                   Co, IH, IW, OH, OW, K, P, int(interpolation), dt,
-                                   _stream(input))
+        rc = lib.mcx_tconv_forward_planned(_ptr(input), _ptr(sample_map), _ptr(interp_weights),
+                                           _ptr(weight), _ptr(bias), _ptr(out), _ptr(ws),
+                                           ws_bytes, _ptr(plan), plan_bytes, B, Ci, Co, IH, IW,
+                                           OH, OW, K, P, int(interpolation), dt, _stream(input))
     _lib.check(rc, "mapped_transposed_conv_forward")
     return out
 
 
 def _tconv_backward(grad_output, sample_map, interp_weights, input, weight, bias, kernel_size,
-                    interpolation):
+                    interpolation, plan=None):
     _contig(input=input, sample_map=sample_map, interp_weights=interp_weights, weight=weight,
             bias=bias)
     grad_output = grad_output.contiguous()
@@ -317,42 +333,84 @@ def _tconv_backward(grad_output, sample_map, interp_weights, input, weight, bias
     lib = _lib.load()
     ws_bytes = lib.mcx_tconv_backward_workspace(B, Ci, Co, IH, IW, OH, OW, K, P, dt)
     ws = _workspace(ws_bytes, input.device)
+    if plan is None and map_plan_cache is not None:
+        plan = _cached_plan(sample_map, interp_weights, OH, OW, interpolation, input.dtype)
+    plan_bytes = 0 if plan is None else plan.numel()
     with torch.cuda.device(input.device):
-        rc = lib.mcx_tconv_backward(_ptr(grad_output), _ptr(sample_map), _ptr(interp_weights),
-                                    _ptr(input), _ptr(weight), _ptr(grad_input), _ptr(grad_weight),
-                                    _ptr(grad_bias), _ptr(ws), ws_bytes, B, Ci, Co, IH, IW, OH, OW,
-                                    K, P, int(interpolation), dt, _stream(input))
+        rc = lib.mcx_tconv_backward_planned(
+            _ptr(grad_output), _ptr(sample_map), _ptr(interp_weights), _ptr(input), _ptr(weight),
+            _ptr(grad_input), _ptr(grad_weight), _ptr(grad_bias), _ptr(ws), ws_bytes, _ptr(plan),
+            plan_bytes, B, Ci, Co, IH, IW, OH, OW, K, P, int(interpolation), dt, _stream(input))
     _lib.check(rc, "mapped_transposed_conv_backward")
     return [grad_input, grad_weight, grad_bias]
 
 
 def mapped_transposed_conv_forward(input, sample_map, weight, bias, output_height, output_width,
-                                   kernel_size, interpolation):
-    """include/nn/layers/mapped_transposed_convolution_layer.h:64-69."""
+                                   kernel_size, interpolation, plan=None):
+    """include/nn/layers/mapped_transposed_convolution_layer.h:64-69.  `plan` (optional, not in
+    the reference): conv_map_plan(sample_map, None, output_height, output_width, ...)."""
     return _tconv_forward(input, sample_map, None, weight, bias, output_height, output_width,
-                          kernel_size, interpolation)
+                          kernel_size, interpolation, plan)
 
 
 def mapped_transposed_conv_backward(grad_output, sample_map, input, weight, bias, kernel_size,
-                                    interpolation):
+                                    interpolation, plan=None):
     """include/nn/layers/mapped_transposed_convolution_layer.h:97-100."""
     return _tconv_backward(grad_output, sample_map, None, input, weight, bias, kernel_size,
-                           interpolation)
+                           interpolation, plan)
 
 
 def weighted_mapped_transposed_conv_forward(input, sample_map, interp_weights, weight, bias,
                                             output_height, output_width, kernel_size,
-                                            interpolation):
+                                            interpolation, plan=None):
     """include/nn/layers/weighted_mapped_transposed_convolution_layer.h:64-67."""
     return _tconv_forward(input, sample_map, interp_weights, weight, bias, output_height,
-                          output_width, kernel_size, interpolation)
+                          output_width, kernel_size, interpolation, plan)
 
 
 def weighted_mapped_transposed_conv_backward(grad_output, sample_map, interp_weights, input,
-                                             weight, bias, kernel_size, interpolation):
+                                             weight, bias, kernel_size, interpolation, plan=None):
     """include/nn/layers/weighted_mapped_transposed_convolution_layer.h:98-100."""
     return _tconv_backward(grad_output, sample_map, interp_weights, input, weight, bias,
-                           kernel_size, interpolation)
+                           kernel_size, interpolation, plan)
+
+
+def scatter_map_plan(sample_map, interp_weights, dest_height, dest_width, interpolation,
+                     for_max_unpool=False, kernel=None):
+    """Plan of resample_to_map (sample_map [IH, IW, (P,) 2]) or of an unpooling (sample_map
+    [OH, OW, K, (P,) 2]) into an image of dest_height x dest_width: the transposed form of the
+    map, built once.  `kernel`: whether the map has a tap axis (default: told from its number of
+    dimensions).  A plan built with `for_max_unpool` serves mapped_max_unpool only, one built
+    without it resample_to_map / mapped_avg_unpool.  Pass it as `plan=` to those ops."""
+    _contig(sample_map=sample_map, interp_weights=interp_weights)
+    _on_gpu("sample_map", sample_map, interp_weights=interp_weights)
+    if kernel is None:
+        kernel = sample_map.dim() == (4 if interp_weights is None else 5)
+    P = _weighted_dims(sample_map, interp_weights, kernel)
+    if sample_map.dtype not in (torch.float32, torch.float64):
+        raise RuntimeError("unsupported dtype %s" % sample_map.dtype)
+    dt = _DTYPES[sample_map.dtype]
+    MH, MW = sample_map.shape[0], sample_map.shape[1]
+    K = sample_map.shape[2] if kernel else 1
+    DH, DW = int(dest_height), int(dest_width)
+    lib = _lib.load()
+    nbytes = lib.mcx_scatter_plan_bytes(MH, MW, DH, DW, K, P, int(interpolation), dt)
+    if nbytes == 0:
+        return None
+    plan = torch.empty((nbytes,), dtype=torch.uint8, device=sample_map.device)
+    with torch.cuda.device(sample_map.device):
+        rc = lib.mcx_scatter_plan_build(_ptr(sample_map), _ptr(interp_weights), _ptr(plan), nbytes,
+                                        MH, MW, DH, DW, K, P, int(interpolation), dt,
+                                        1 if for_max_unpool else 0, _stream(sample_map))
+    _lib.check(rc, "scatter_map_plan")
+    return plan
+
+
+def _scatter_plan_for(kind, plan, sample_map, interp_weights, DH, DW, interpolation, kernel):
+    if plan is None and map_plan_cache is not None and scatter_as_gather:
+        plan = _cached_plan(sample_map, interp_weights, DH, DW, interpolation, sample_map.dtype,
+                            kind=kind, kernel=kernel)
+    return plan
 
 
 # ------------------------------------------------------------------------ pooling
@@ -385,7 +443,7 @@ def _max_pool(input, sample_map, interp_weights, kernel_size, interpolation):
 
 
 def _max_unpool(grad_output, idx_mask, sample_map, interp_weights, input_height, input_width,
-                kernel_size, interpolation):
+                kernel_size, interpolation, plan=None):
     _contig(grad_output=grad_output, idx_mask=idx_mask, sample_map=sample_map,
             interp_weights=interp_weights)
     _on_gpu("grad_output", grad_output, idx_mask=idx_mask, sample_map=sample_map,
@@ -400,6 +458,15 @@ def _max_unpool(grad_output, idx_mask, sample_map, interp_weights, input_height,
     IH, IW = int(input_height), int(input_width)
     gin = torch.empty((B, C, IH, IW), dtype=grad_output.dtype, device=grad_output.device)
     lib = _lib.load()
+    plan = _scatter_plan_for("max_unpool", plan, sample_map, interp_weights, IH, IW,
+                             interpolation, True)
+    if plan is not None:
+        with torch.cuda.device(grad_output.device):
+            rc = lib.mcx_max_unpool_planned(_ptr(grad_output), _ptr(idx_mask), _ptr(plan),
+                                            plan.numel(), _ptr(gin), B, C, IH, IW, OH, OW, K, P,
+                                            int(interpolation), dt, _stream(grad_output))
+        _lib.check(rc, "mapped_max_unpool")
+        return gin
     ws_bytes = lib.mcx_unpool_workspace(IH, IW, OH, OW, K, P, int(interpolation), dt) \
         if scatter_as_gather else 0
     ws = _workspace(ws_bytes, grad_output.device)
@@ -428,7 +495,7 @@ def _avg_pool(input, sample_map, interp_weights, kernel_size, interpolation):
 
 
 def _avg_unpool(grad_output, sample_map, interp_weights, input_height, input_width, kernel_size,
-                interpolation):
+                interpolation, plan=None):
     _contig(grad_output=grad_output, sample_map=sample_map, interp_weights=interp_weights)
     _on_gpu("grad_output", grad_output, sample_map=sample_map, interp_weights=interp_weights)
     dt = _dtype(grad_output, maps=(sample_map, interp_weights))
@@ -439,6 +506,15 @@ def _avg_unpool(grad_output, sample_map, interp_weights, input_height, input_wid
     IH, IW = int(input_height), int(input_width)
     gin = torch.empty((B, C, IH, IW), dtype=grad_output.dtype, device=grad_output.device)
     lib = _lib.load()
+    plan = _scatter_plan_for("avg_unpool", plan, sample_map, interp_weights, IH, IW,
+                             interpolation, True)
+    if plan is not None:
+        with torch.cuda.device(grad_output.device):
+            rc = lib.mcx_avg_unpool_planned(_ptr(grad_output), _ptr(plan), plan.numel(), _ptr(gin),
+                                            B, C, IH, IW, OH, OW, K, P, int(interpolation), dt,
+                                            _stream(grad_output))
+        _lib.check(rc, "mapped_avg_unpool")
+        return gin
     ws_bytes = lib.mcx_unpool_workspace(IH, IW, OH, OW, K, P, int(interpolation), dt) \
         if scatter_as_gather else 0
     ws = _workspace(ws_bytes, grad_output.device)
@@ -456,10 +532,10 @@ def mapped_max_pool(input, sample_map, kernel_size, interpolation):
 
 
 def mapped_max_unpool(grad_output, idx_mask, sample_map, input_height, input_width, kernel_size,
-                      interpolation):
-    """include/nn/layers/mapped_max_pooling_layer.h:69-73."""
+                      interpolation, plan=None):
+    """include/nn/layers/mapped_max_pooling_layer.h:69-73.  `plan`: see scatter_map_plan."""
     return _max_unpool(grad_output, idx_mask, sample_map, None, input_height, input_width,
-                       kernel_size, interpolation)
+                       kernel_size, interpolation, plan)
 
 
 def weighted_mapped_max_pool(input, sample_map, interp_weights, kernel_size, interpolation):
@@ -468,10 +544,10 @@ def weighted_mapped_max_pool(input, sample_map, interp_weights, kernel_size, int
 
 
 def weighted_mapped_max_unpool(grad_output, idx_mask, sample_map, interp_weights, input_height,
-                               input_width, kernel_size, interpolation):
+                               input_width, kernel_size, interpolation, plan=None):
     """include/nn/layers/weighted_mapped_max_pooling_layer.h:67-70."""
     return _max_unpool(grad_output, idx_mask, sample_map, interp_weights, input_height,
-                       input_width, kernel_size, interpolation)
+                       input_width, kernel_size, interpolation, plan)
 
 
 def mapped_avg_pool(input, sample_map, kernel_size, interpolation):
@@ -480,10 +556,10 @@ def mapped_avg_pool(input, sample_map, kernel_size, interpolation):
 
 
 def mapped_avg_unpool(grad_output, sample_map, input_height, input_width, kernel_size,
-                      interpolation):
-    """include/nn/layers/mapped_avg_pooling_layer.h:64-67."""
+                      interpolation, plan=None):
+    """include/nn/layers/mapped_avg_pooling_layer.h:64-67.  `plan`: see scatter_map_plan."""
     return _avg_unpool(grad_output, sample_map, None, input_height, input_width, kernel_size,
-                       interpolation)
+                       interpolation, plan)
 
 
 def weighted_mapped_avg_pool(input, sample_map, interp_weights, kernel_size, interpolation):
@@ -492,15 +568,15 @@ def weighted_mapped_avg_pool(input, sample_map, interp_weights, kernel_size, int
 
 
 def weighted_mapped_avg_unpool(grad_output, sample_map, interp_weights, input_height, input_width,
-                               kernel_size, interpolation):
+                               kernel_size, interpolation, plan=None):
     """include/nn/layers/weighted_mapped_avg_pooling_layer.h:75-78."""
     return _avg_unpool(grad_output, sample_map, interp_weights, input_height, input_width,
-                       kernel_size, interpolation)
+                       kernel_size, interpolation, plan)
 
 
 # ----------------------------------------------------------------------- resample
 def _resample_to_map(input, sample_map, interp_weights, output_height, output_width,
-                     interpolation):
+                     interpolation, plan=None):
     _contig(input=input, sample_map=sample_map, interp_weights=interp_weights)
     _on_gpu("input", input, sample_map=sample_map, interp_weights=interp_weights)
     dt = _dtype(input, maps=(sample_map, interp_weights))
@@ -513,6 +589,15 @@ def _resample_to_map(input, sample_map, interp_weights, output_height, output_wi
     OH, OW = int(output_height), int(output_width)
     out = torch.empty((B, C, OH, OW), dtype=input.dtype, device=input.device)
     lib = _lib.load()
+    plan = _scatter_plan_for("resample", plan, sample_map, interp_weights, OH, OW, interpolation,
+                             False)
+    if plan is not None:
+        with torch.cuda.device(input.device):
+            rc = lib.mcx_resample_to_map_planned(_ptr(input), _ptr(plan), plan.numel(), _ptr(out),
+                                                 B, C, IH, IW, OH, OW, P, int(interpolation), dt,
+                                                 _stream(input))
+        _lib.check(rc, "resample_to_map")
+        return out
     ws_bytes = lib.mcx_resample_to_map_workspace(IH, IW, OH, OW, P, int(interpolation), dt) \
         if scatter_as_gather else 0
     ws = _workspace(ws_bytes, input.device)
@@ -542,9 +627,10 @@ def _resample_from_map(input, sample_map, interp_weights, interpolation):
     return out
 
 
-def resample_to_map(input, sample_map, output_height, output_width, interpolation):
-    """include/nn/layers/resample_layer.h:38-40 (scatter)."""
-    return _resample_to_map(input, sample_map, None, output_height, output_width, interpolation)
+def resample_to_map(input, sample_map, output_height, output_width, interpolation, plan=None):
+    """include/nn/layers/resample_layer.h:38-40 (scatter).  `plan`: see scatter_map_plan."""
+    return _resample_to_map(input, sample_map, None, output_height, output_width, interpolation,
+                            plan)
 
 
 def resample_from_map(input, sample_map, interpolation):
@@ -553,10 +639,10 @@ def resample_from_map(input, sample_map, interpolation):
 
 
 def weighted_resample_to_map(input, sample_map, interp_weights, output_height, output_width,
-                             interpolation):
+                             interpolation, plan=None):
     """include/nn/layers/weighted_resample_layer.h:49-54."""
     return _resample_to_map(input, sample_map, interp_weights, output_height, output_width,
-                            interpolation)
+                            interpolation, plan)
 
 
 def weighted_resample_from_map(input, sample_map, interp_weights, interpolation):

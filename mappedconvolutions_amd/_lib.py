@@ -37,10 +37,18 @@ SIGNATURES = {
     "mcx_conv_plan_bytes": (_sz, [_i64] * 6 + [_i]),
     "mcx_conv_plan_build": (_i, [_p] * 3 + [_sz] + [_i64] * 6 + [_i, _i, _p]),
     "mcx_conv_backward_planned": (_i, [_p] * 9 + [_sz, _p, _sz] + [_i64] * 9 + [_i, _i, _p]),
+    "mcx_conv_forward_planned": (_i, [_p] * 7 + [_sz, _p, _sz] + [_i64] * 9 + [_i, _i, _p]),
+    "mcx_tconv_forward_planned": (_i, [_p] * 7 + [_sz, _p, _sz] + [_i64] * 9 + [_i, _i, _p]),
+    "mcx_tconv_backward_planned": (_i, [_p] * 9 + [_sz, _p, _sz] + [_i64] * 9 + [_i, _i, _p]),
     "mcx_tconv_forward": (_i, [_p] * 7 + [_sz] + [_i64] * 9 + [_i, _i, _p]),
     "mcx_tconv_forward_workspace": (_sz, [_i64] * 9 + [_i]),
     "mcx_tconv_backward_workspace": (_sz, [_i64] * 9 + [_i]),
     "mcx_tconv_backward": (_i, [_p] * 9 + [_sz] + [_i64] * 9 + [_i, _i, _p]),
+    "mcx_scatter_plan_bytes": (_sz, [_i64] * 6 + [_i, _i]),
+    "mcx_scatter_plan_build": (_i, [_p] * 3 + [_sz] + [_i64] * 6 + [_i, _i, _i, _p]),
+    "mcx_resample_to_map_planned": (_i, [_p] * 2 + [_sz, _p] + [_i64] * 7 + [_i, _i, _p]),
+    "mcx_avg_unpool_planned": (_i, [_p] * 2 + [_sz, _p] + [_i64] * 8 + [_i, _i, _p]),
+    "mcx_max_unpool_planned": (_i, [_p] * 3 + [_sz, _p] + [_i64] * 8 + [_i, _i, _p]),
     "mcx_knn": (_i, [_p] * 4 + [_i64] * 5 + [_i, _p]),
     "mcx_projection_map": (_i, [_p] + [_i64] * 4 + [_i] + [_i64] * 2 + [_p]),
     "mcx_cube_projection_map": (_i, [_p] + [_i64] * 4 + [_p]),

@@ -156,8 +156,52 @@ def maps(dev):
               nbytes=cube.numel() * 4 + 64 * H * W * 4)
 
 
+def plans(dev):
+    """The same calls with map plans (built once, outside the timed region): config 4's scatter
+    ops through scatter_map_plan, the headline convolution through conv_map_plan."""
+    B, C, F, H, W = 4, 64, 256, 512, 1024
+    g = torch.Generator().manual_seed(0)
+    cube = torch.rand(B, C, F, 6 * F, generator=g).to(dev)
+    cmap = synthetic.cube_to_equirect_map(F, H, W).to(dev)
+    eq = torch.rand(B, C, H, W, generator=g).to(dev)
+    lmap = synthetic.latitude_map(H, W, 1).to(dev)
+    fb = 4
+    n_cube, n_eq = cube.numel() * fb, eq.numel() * fb
+    plan = _C.scatter_map_plan(cmap, None, H, W, 1)
+    _line("planned config4 resample_to_map bilinear",
+          _time(lambda: _C.resample_to_map(cube, cmap, H, W, 1, plan=plan)),
+          nbytes=n_cube + n_eq + plan.numel())
+    _, idx = _C.mapped_max_pool(eq, lmap, 9, 1)
+    plan_a = _C.scatter_map_plan(lmap, None, H, W, 1)
+    plan_m = _C.scatter_map_plan(lmap, None, H, W, 1, for_max_unpool=True)
+    _line("planned config4 mapped_avg_unpool K9",
+          _time(lambda: _C.mapped_avg_unpool(eq, lmap, H, W, 9, 1, plan=plan_a)),
+          nbytes=2 * n_eq + plan_a.numel())
+    _line("planned config4 mapped_max_unpool K9",
+          _time(lambda: _C.mapped_max_unpool(eq, idx, lmap, H, W, 9, 1, plan=plan_m)),
+          nbytes=2 * n_eq + 2 * n_eq + plan_m.numel())
+    del cube, eq, idx
+    B, C, H, W, K = 8, 64, 256, 512, 9
+    x = torch.randn(B, C, H, W, generator=g).to(dev)
+    gy = torch.randn(B, C, H, W, generator=g).to(dev)
+    w = (torch.randn(C, C, K, generator=g) / (C * K) ** 0.5).to(dev)
+    b = torch.zeros(C, device=dev)
+    smap = synthetic.latitude_map(H, W, 1).to(dev)
+    cplan = _C.conv_map_plan(smap, None, H, W, 1)
+    flop = 2.0 * B * H * W * C * C * K
+    _line("planned headline conv forward fp32",
+          _time(lambda: _C.mapped_conv_forward(x, smap, w, b, K, 1, plan=cplan)), flops=flop)
+    _line("unplanned headline conv forward fp32",
+          _time(lambda: _C.mapped_conv_forward(x, smap, w, b, K, 1)), flops=flop)
+    _line("planned headline conv backward fp32",
+          _time(lambda: _C.mapped_conv_backward(gy, smap, x, w, b, K, 1, plan=cplan)),
+          flops=2 * flop)
+    _line("unplanned headline conv backward fp32",
+          _time(lambda: _C.mapped_conv_backward(gy, smap, x, w, b, K, 1)), flops=2 * flop)
+
+
 WORKLOADS = {"config3": config3, "config4": config4, "knn": knn, "config5": config5,
-             "maps": maps}
+             "maps": maps, "plans": plans}
 
 
 def main(argv):

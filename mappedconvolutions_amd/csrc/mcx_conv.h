@@ -40,7 +40,7 @@ template <typename TD>
 int mfma_gather_product(const TD *src, const float *map, const float *iw, const TD *w,
                         const TD *bias, TD *y, void *scratch, int64_t B, int64_t G, int64_t O,
                         int64_t SH, int64_t SW, int64_t OH, int64_t OW, int64_t K, int64_t P,
-                        int interp, hipStream_t s);
+                        int interp, hipStream_t s, const void *plan = nullptr);
 size_t mfma_weight_grad_bytes(int64_t B, int64_t A, int64_t G, int64_t MH, int64_t MW, int64_t K,
                               int64_t GH, int64_t GW);
 template <typename TD>

@@ -122,7 +122,7 @@ template <typename T>
 int gather_product(bool mfma, const void *src, const void *map, const void *iw, const void *w,
                    const void *bias, void *y, void *ws, size_t ws_bytes, int64_t B, int64_t G,
                    int64_t O, int64_t SH, int64_t SW, int64_t MH, int64_t MW, int64_t K, int64_t P,
-                   int interp, hipStream_t s);
+                   int interp, hipStream_t s, const void *plan = nullptr);  // plan: see mcx.h
 
 // dst[b,d] = bias[d] (or 0) + splat(sum_s W[s,d,k] * src[b,s,n], map[n,k]); n over MH x MW.
 template <typename T>
@@ -149,7 +149,7 @@ int bias_grad(const void *gy, void *gb, void *ws, size_t ws_bytes, int64_t B, in
   int gather_product<T>(bool, const void *src, const void *map, const void *iw, const void *w,     \
                         const void *bias, void *y, void *, size_t, int64_t B, int64_t G,           \
                         int64_t O, int64_t SH, int64_t SW, int64_t MH, int64_t MW, int64_t K,      \
-                        int64_t P, int interp, hipStream_t s) {                                    \
+                        int64_t P, int interp, hipStream_t s, const void *) {                      \
     return generic_gather_product<T>((const T *)src, (const T *)map, (const T *)iw,                \
                                      (const T *)w, (const T *)bias, (T *)y, B, G, O, SH, SW,       \
                                      MH * MW, K, P, interp, s);                                    \
@@ -192,7 +192,8 @@ template <>
 int gather_product<float>(bool mfma, const void *src, const void *map, const void *iw,
                           const void *w, const void *bias, void *y, void *ws, size_t ws_bytes,
                           int64_t B, int64_t G, int64_t O, int64_t SH, int64_t SW, int64_t MH,
-                          int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s) {
+                          int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s,
+                          const void *plan) {
   if (!mfma)
     return generic_gather_product<float>((const float *)src, (const float *)map,
                                          (const float *)iw, (const float *)w, (const float *)bias,
@@ -200,7 +201,7 @@ int gather_product<float>(bool mfma, const void *src, const void *map, const voi
   if (!ws || ws_bytes < mfma_gather_product_bytes(O, G, K, B, SH, SW, 4)) return MCX_E_WORKSPACE;
   return mfma_gather_product<float>((const float *)src, (const float *)map, (const float *)iw,
                                     (const float *)w, (const float *)bias, (float *)y, ws, B, G, O,
-                                    SH, SW, MH, MW, K, P, interp, s);
+                                    SH, SW, MH, MW, K, P, interp, s, plan);
 }
 
 template <>
@@ -253,12 +254,13 @@ template <>
 int gather_product<bf16_t>(bool mfma, const void *src, const void *map, const void *iw,
                            const void *w, const void *bias, void *y, void *ws, size_t ws_bytes,
                            int64_t B, int64_t G, int64_t O, int64_t SH, int64_t SW, int64_t MH,
-                           int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s) {
+                           int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s,
+                           const void *plan) {
   if (!mfma) return MCX_E_DTYPE;
   if (!ws || ws_bytes < mfma_gather_product_bytes(O, G, K, B, SH, SW, 2)) return MCX_E_WORKSPACE;
   return mfma_gather_product<bf16_t>((const bf16_t *)src, (const float *)map, (const float *)iw,
                                      (const bf16_t *)w, (const bf16_t *)bias, (bf16_t *)y, ws, B,
-                                     G, O, SH, SW, MH, MW, K, P, interp, s);
+                                     G, O, SH, SW, MH, MW, K, P, interp, s, plan);
 }
 
 template <>
@@ -300,9 +302,9 @@ int bias_grad<bf16_t>(const void *gy, void *gb, void *ws, size_t ws_bytes, int64
 template <typename T>
 int conv_forward_t(bool mfma, const void *x, const void *map, const void *iw, const void *w,
                    const void *bias, void *y, void *ws, size_t ws_bytes, const ConvDims &d,
-                   int interp, hipStream_t s) {
+                   int interp, hipStream_t s, const void *plan = nullptr) {
   return gather_product<T>(mfma, x, map, iw, w, bias, y, ws, ws_bytes, d.B, d.Ci, d.Co, d.IH, d.IW,
-                           d.OH, d.OW, d.K, d.P, interp, s);
+                           d.OH, d.OW, d.K, d.P, interp, s, plan);
 }
 
 template <typename T>
@@ -327,22 +329,22 @@ int conv_backward_t(bool mfma, const void *gy, const void *map, const void *iw, 
 template <typename T>
 int tconv_forward_t(bool mfma, const void *x, const void *map, const void *iw, const void *w,
                     const void *bias, void *y, void *ws, size_t ws_bytes, const ConvDims &d,
-                    int interp, hipStream_t s) {
+                    int interp, hipStream_t s, const void *plan = nullptr) {
   return product_scatter<T>(mfma, x, map, iw, w, bias, y, ws, ws_bytes, d.B, d.Ci, d.Co, d.OH,
-                            d.OW, d.IH, d.IW, d.K, d.P, interp, s);
+                            d.OW, d.IH, d.IW, d.K, d.P, interp, s, plan);
 }
 
 template <typename T>
 int tconv_backward_t(bool mfma, const void *gy, const void *map, const void *iw, const void *x,
                      const void *w, void *gx, void *gw, void *gb, void *ws, size_t ws_bytes,
-                     const ConvDims &d, int interp, hipStream_t s) {
+                     const ConvDims &d, int interp, hipStream_t s, const void *plan = nullptr) {
   int rc = 0;
   // grad_input[b,ci] = sum_{co,k} W[ci,co,k] * sample(gy[b,co], map[n,k])
   if (gx && (rc = gather_product<T>(mfma, gy, map, iw, w, nullptr, gx, ws, ws_bytes, d.B, d.Co,
-                                    d.Ci, d.OH, d.OW, d.IH, d.IW, d.K, d.P, interp, s)))
+                                    d.Ci, d.OH, d.OW, d.IH, d.IW, d.K, d.P, interp, s, plan)))
     return rc;
   if (gw && (rc = weight_grad<T>(mfma, x, gy, map, iw, gw, ws, ws_bytes, d.B, d.Ci, d.Co, d.OH,
-                                 d.OW, d.IH, d.IW, d.K, d.P, interp, s, nullptr)))
+                                 d.OW, d.IH, d.IW, d.K, d.P, interp, s, nullptr, plan)))
     return rc;
   if (gb) rc = bias_grad<T>(gy, gb, ws, ws_bytes, d.B, d.Co, d.OH * d.OW, s);
   return rc;
@@ -471,6 +473,73 @@ extern "C" int mcx_conv_backward_planned(const void *gy, const void *map, const 
                                                workspace_bytes, d, interp, s, plan));
 }
 
+namespace {
+// A plan, when given, must be one mcx_conv_plan_build made for these sizes (SH x SW: the
+// image the map samples; MH x MW: the map).
+int check_plan(const void *plan, size_t plan_bytes, bool mfma, int64_t SH, int64_t SW, int64_t MH,
+               int64_t MW, int64_t K, int64_t P) {
+  if (!plan) return 0;
+  if (!mfma) return MCX_E_DTYPE;
+  const size_t need = mfma_scatter_plan_bytes(SH, SW, MH, MW, K, P);
+  return (need == 0 || plan_bytes < need) ? MCX_E_WORKSPACE : 0;
+}
+}  // namespace
+
+extern "C" int mcx_conv_forward_planned(const void *x, const void *map, const void *iw,
+                                        const void *w, const void *bias, void *y, void *workspace,
+                                        size_t workspace_bytes, const void *plan,
+                                        size_t plan_bytes, int64_t B, int64_t Ci, int64_t Co,
+                                        int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
+                                        int64_t P, int interp, int dtype, void *stream) {
+  ProfileRequestScope profile_scope;
+  const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
+  if (int rc = check_dims(d, OH, OW, dtype)) return rc;
+  if (int rc = check_ptrs(x, map, iw, w, P)) return rc;
+  if (!bias || !y) return MCX_E_NULL;
+  hipStream_t s = (hipStream_t)stream;
+  const bool mfma = use_mfma(dtype, P);
+  if (int rc = check_plan(plan, plan_bytes, mfma, IH, IW, OH, OW, K, P)) return rc;
+  MCX_DISPATCH_DTYPE(dtype, conv_forward_t<T>(mfma, x, map, iw, w, bias, y, workspace,
+                                              workspace_bytes, d, interp, s, plan));
+}
+
+extern "C" int mcx_tconv_forward_planned(const void *x, const void *map, const void *iw,
+                                         const void *w, const void *bias, void *y,
+                                         void *workspace, size_t workspace_bytes, const void *plan,
+                                         size_t plan_bytes, int64_t B, int64_t Ci, int64_t Co,
+                                         int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
+                                         int64_t P, int interp, int dtype, void *stream) {
+  ProfileRequestScope profile_scope;
+  const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
+  if (int rc = check_dims(d, IH, IW, dtype)) return rc;
+  if (int rc = check_ptrs(x, map, iw, w, P)) return rc;
+  if (!bias || !y) return MCX_E_NULL;
+  hipStream_t s = (hipStream_t)stream;
+  const bool mfma = use_mfma(dtype, P);
+  if (int rc = check_plan(plan, plan_bytes, mfma, OH, OW, IH, IW, K, P)) return rc;
+  MCX_DISPATCH_DTYPE(dtype, tconv_forward_t<T>(mfma, x, map, iw, w, bias, y, workspace,
+                                               workspace_bytes, d, interp, s, plan));
+}
+
+extern "C" int mcx_tconv_backward_planned(const void *gy, const void *map, const void *iw,
+                                          const void *x, const void *w, void *gx, void *gw,
+                                          void *gb, void *workspace, size_t workspace_bytes,
+                                          const void *plan, size_t plan_bytes, int64_t B,
+                                          int64_t Ci, int64_t Co, int64_t IH, int64_t IW,
+                                          int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
+                                          int dtype, void *stream) {
+  ProfileRequestScope profile_scope;
+  const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
+  if (int rc = check_dims(d, IH, IW, dtype)) return rc;
+  if (int rc = check_ptrs(gy, map, iw, w, P)) return rc;
+  if (gw && !x) return MCX_E_NULL;
+  hipStream_t s = (hipStream_t)stream;
+  const bool mfma = use_mfma(dtype, P);
+  if (int rc = check_plan(plan, plan_bytes, mfma, OH, OW, IH, IW, K, P)) return rc;
+  MCX_DISPATCH_DTYPE(dtype, tconv_backward_t<T>(mfma, gy, map, iw, x, w, gx, gw, gb, workspace,
+                                                workspace_bytes, d, interp, s, plan));
+}
+
 extern "C" size_t mcx_tconv_forward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t IH,
                                               int64_t IW, int64_t OH, int64_t OW, int64_t K,
                                               int64_t P, int dtype) {
@@ -519,7 +588,7 @@ extern "C" int mcx_tconv_backward(const void *gy, const void *map, const void *i
                                                 workspace_bytes, d, interp, s));
 }
 
-extern "C" int mcx_abi_version(void) { return 8; }
+extern "C" int mcx_abi_version(void) { return 9; }
 
 extern "C" int mcx_profile_dominant_kernel(void *start_event, void *stop_event) {
   mcx::set_profile_events(start_event, stop_event);

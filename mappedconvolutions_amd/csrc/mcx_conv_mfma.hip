@@ -352,8 +352,11 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
         const int64_t e = (n_g * K + k0 + kl) * NP + sp;
         PairTap<NCORN> t;
         if (NCORN == 1 && packed_map) {
-          // pre-resolved entry (a transposed map): element index of the source, weight
-          const float2 q = reinterpret_cast<const float2 *>(map)[e];
+          // pre-resolved entry (a transposed map or a plan's gather part): element index of the
+          // source and weight, stored [tap][slot][pixel] so that the lanes of a wave, which
+          // hold neighbouring pixels, read neighbouring entries
+          const float2 q = reinterpret_cast<const float2 *>(
+              map)[((int64_t)(k0 + kl) * NP + sp) * N + n_g];
           t.off[0] = __builtin_bit_cast(unsigned, q.x) * (unsigned)sizeof(TD);
           t.wt[0] = live ? q.y : 0.f;
         } else {
@@ -1551,6 +1554,14 @@ int launch_pair_mask(const float *map, const float *iw, int *mask, const ModeArg
 
 }  // namespace
 
+// (defined with the map plans below)
+namespace {
+constexpr int kPlanSlots = 4;  // resolved entries per (location, tap) of a plan's gather part
+bool gather_plan_applies(int interp, int64_t P);
+}  // namespace
+size_t mfma_gather_plan_offset(int64_t DH, int64_t DW, int64_t MH, int64_t MW, int64_t K,
+                               int64_t P);
+
 // ---- gather-product --------------------------------------------------------------
 // Packed weights, then (single-row sources) the channel-last copy of the source, sized
 // for 4-byte elements.
@@ -1568,8 +1579,26 @@ template <typename TD>
 int mfma_gather_product(const TD *src, const float *map, const float *iw, const TD *w,
                         const TD *bias, TD *y, void *scratch, int64_t B, int64_t G, int64_t O,
                         int64_t SH, int64_t SW, int64_t OH, int64_t OW, int64_t K, int64_t P,
-                        int interp, hipStream_t s) {
+                        int interp, hipStream_t s, const void *plan) {
   float *wp = (float *)scratch;
+  if (plan && gather_plan_applies(interp, P) && OH * OW * K * kPlanSlots * 2 <= 0x7fffffffLL) {
+    // the map's taps were resolved when the plan was built: read them as four pre-resolved
+    // pairs per tap; flag word 4 of the plan says whether only the first two are ever in use
+    const char *pb = (const char *)plan;
+    const float *gmap = (const float *)(pb + mfma_gather_plan_offset(SH, SW, OH, OW, K, P));
+    const int *flags = (const int *)plan + SH * SW * K;
+    TD *stage = (SH == 1 || sizeof(TD) == 2)
+                    ? reinterpret_cast<TD *>((char *)scratch + 256 +
+                                             align256((size_t)(K * round_up(G, kGC) *
+                                                               round_up(O, kOT)) * 4))
+                    : nullptr;
+    if (int rc = launch_pack_weights<TD>(w, wp, O, G, K, 0, s)) return rc;
+    const ModeArgs pm = mode_args(interp, P);
+    const bool four_pairs = pm.np * (pm.mode == kInterpNearest ? 1 : 4) == 4;
+    return launch_gather_product<TD>(src, gmap, nullptr, wp, bias, y, stage, B, G, O, SH, SW, OH,
+                                     OW, K, kPlanSlots, kInterpNearest, nullptr, 0, s, nullptr,
+                                     false, four_pairs ? flags + 4 : nullptr, true);
+  }
   int *pair_mask = reinterpret_cast<int *>(
       (char *)scratch + align256((size_t)(K * round_up(G, kGC) * round_up(O, kOT)) * 4));
   TD *stage = (SH == 1 || sizeof(TD) == 2) ? reinterpret_cast<TD *>((char *)pair_mask + 256)
@@ -1688,10 +1717,11 @@ namespace {
 // resolution-preserving maps such as the latitude-distorted kernels), the product-
 // scatter equals a weighted, nearest-neighbour gather-product over the transposed
 // map, which needs no atomics at all and reuses the forward kernel.  This kernel
-// builds that map: tmap[p][k][slot] = (index of source pixel n as bits, corner weight);
+// builds that map: tmap[k][slot][p] = (index of source pixel n as bits, corner weight);
 // a slot counter per (p, k) hands out slots and an overflow flag selects the scatter
 // kernel instead (both kernels are always enqueued; the flag gates them on the device).
 constexpr int kTransSlots = 4;
+constexpr int kTransSlotsConst = kTransSlots;
 
 // A contribution that finds its cell full goes to the overflow list (destination pixel,
 // source pixel, tap, weight), applied afterwards with atomics by overflow_scatter_kernel;
@@ -1714,6 +1744,7 @@ __global__ void build_transposed_map_kernel(const float *__restrict__ map,
   if (e >= total) return;
   const int k = (int)(e % K);
   const int64_t n = e / K;
+  const int64_t DHW = (int64_t)DH * DW;
   const float nbits = __builtin_bit_cast(float, (int)n);
   for (int sp = 0; sp < np; sp++) {
     const int64_t m = e * np + sp;
@@ -1723,12 +1754,15 @@ __global__ void build_transposed_map_kernel(const float *__restrict__ map,
 #pragma unroll
     for (int c = 0; c < NCORN; c++) {
       if (!(t.ok & (1u << c)) || t.wt[c] == 0.f) continue;
-      const int64_t cell = ((int64_t)t.yy[c] * DW + t.xx[c]) * K + k;
+      const int64_t pix = (int64_t)t.yy[c] * DW + t.xx[c];
+      const int64_t cell = pix * K + k;
       const int slot = atomicAdd(&cnt[cell], 1);
+      // slots are stored [tap][slot][pixel] (see the gather-product kernel's packed maps)
       if (slot < kTransSlots) {
-        tmap[cell * kTransSlots + slot] = make_float2(nbits, t.wt[c]);
+        tmap[((int64_t)k * kTransSlots + slot) * DHW + pix] = make_float2(nbits, t.wt[c]);
       } else if (tmap2 && slot < 2 * kTransSlots) {  // second level (a second gather pass)
-        tmap2[cell * kTransSlots + slot - kTransSlots] = make_float2(nbits, t.wt[c]);
+        tmap2[((int64_t)k * kTransSlots + slot - kTransSlots) * DHW + pix] =
+            make_float2(nbits, t.wt[c]);
       } else {
         // overflow[0]: flag, overflow[1]: length of the overflow list
         const int pos = ovf_cap > 0 ? atomicAdd(&overflow[1], 1) : 0;
@@ -1846,6 +1880,42 @@ __global__ void convert_planes_kernel(const float *__restrict__ src, TD *__restr
     dst[i] = from_f32<TD>(src[i]);
 }
 
+// Gather part of a map plan: every (map location, tap) resolved once to four (element index of
+// the sampled image as bits, weight) entries - the four bilinear corners, or up to four
+// nearest points with the rest zero - in the layout the gather-product kernel reads with
+// `packed_map` (the same as a transposed map's cells).
+template <int NCORN>
+__global__ void build_gather_plan_kernel(const float *__restrict__ map,
+                                         const float *__restrict__ iw, float2 *__restrict__ gmap,
+                                         int np, int weighted, int wrap, int SH, int SW, int K,
+                                         int64_t total) {
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // (location, tap)
+  if (e >= total) return;
+  float2 out[kTransSlotsConst];
+#pragma unroll
+  for (int i = 0; i < kTransSlotsConst; i++) out[i] = make_float2(0.f, 0.f);
+  for (int sp = 0; sp < np; sp++) {
+    const int64_t q = e * np + sp;
+    PairTap<NCORN> t;
+    resolve_pairs<NCORN, 1>(map[q * 2], map[q * 2 + 1], SH, SW, wrap != 0,
+                            weighted ? iw[q] : 1.f, t);
+#pragma unroll
+    for (int i = 0; i < NCORN; i++)
+      if (sp * NCORN + i < kTransSlotsConst)
+        out[sp * NCORN + i] = make_float2(__builtin_bit_cast(float, t.off[i]), t.wt[i]);
+  }
+  const int64_t n = e / K, k = e % K, pixels = total / K;  // stored [tap][slot][location]
+#pragma unroll
+  for (int i = 0; i < kTransSlotsConst; i++) gmap[(k * kTransSlotsConst + i) * pixels + n] = out[i];
+}
+
+// A map has a gather part when a tap is at most four (offset, weight) pairs.
+static_assert(kPlanSlots == kTransSlots, "a plan's gather part has the cells of a transposed map");
+bool gather_plan_applies(int interp, int64_t P) {
+  const int64_t np = P > 0 ? P : 1;
+  return np * (canonical_interp(interp) == kInterpNearest ? 1 : 4) <= 4;
+}
+
 struct ScatterScratch {
   size_t wq, wpt, cnt, tmap, tmap2, acc32, ovf, stage, total;  // byte offsets
   bool two_level;  // a second four-slot level, applied by a second gather pass
@@ -1882,7 +1952,7 @@ ScatterScratch scatter_scratch(int64_t B, int64_t S, int64_t D, int64_t K, int64
     off += align256((size_t)(K * round_up(S, kGC) * round_up(D, kOT)) * 4);
     sc.cnt = off;  // counters, the overflow flag and list length; cleared with tmap
     off += align256((size_t)(cells + 8) * 4);
-    sc.tmap = off;  // [cell][slot] (source pixel index as bits, weight)
+    sc.tmap = off;  // [tap][slot][pixel] (source pixel index as bits, weight)
     off += align256((size_t)cells * kTransSlots * 2 * 4);
     sc.tmap2 = off;
     if (sc.two_level) off += align256((size_t)cells * kTransSlots * 2 * 4);
@@ -1934,10 +2004,22 @@ int build_transposed_map(const ScatterScratch &sc, const float *map, const float
 // Layout: the scratch region [cnt, stage) of mfma_product_scatter (counters, eight flag words,
 // slots, second-level slots, overflow list); flag word 4 holds the pair mask of the map itself,
 // for the weight gradient.  Depends on the map, its interpolation and the two image sizes only.
+// (followed, for maps of at most four points per tap, by the gather part: MH * MW * K cells of
+// four resolved entries)
+size_t mfma_gather_plan_offset(int64_t DH, int64_t DW, int64_t MH, int64_t MW, int64_t K,
+                               int64_t P) {
+  const ScatterScratch sc = scatter_scratch(1, 1, 1, K, DH, DW, 4, MH, MW, P);
+  return sc.transposed_path ? align256(sc.stage - sc.cnt) : 0;
+}
+
 size_t mfma_scatter_plan_bytes(int64_t DH, int64_t DW, int64_t MH, int64_t MW, int64_t K,
                                int64_t P) {
   const ScatterScratch sc = scatter_scratch(1, 1, 1, K, DH, DW, 4, MH, MW, P);
-  return sc.transposed_path ? sc.stage - sc.cnt : 0;
+  if (!sc.transposed_path) return 0;
+  size_t n = align256(sc.stage - sc.cnt);
+  if (P <= kTransSlots && MH * MW * K * kTransSlots * 2 <= 0x7fffffffLL)
+    n += align256((size_t)(MH * MW * K) * kTransSlots * sizeof(float2));
+  return n;
 }
 
 int mfma_scatter_plan_build(const float *map, const float *iw, void *plan, int64_t DH, int64_t DW,
@@ -1956,7 +2038,19 @@ int mfma_scatter_plan_build(const float *map, const float *iw, void *plan, int64
                      flag);
   MCX_HIP_CHECK_LAUNCH();
   if (m.np * (m.mode == kInterpNearest ? 1 : 4) == 4)
-    return launch_pair_mask(map, iw, flag + 4, m, DH, DW, MH * MW * K, s, true);
+    if (int rc = launch_pair_mask(map, iw, flag + 4, m, DH, DW, MH * MW * K, s, true)) return rc;
+  if (gather_plan_applies(interp, P) && MH * MW * K * kTransSlots * 2 <= 0x7fffffffLL) {
+    float2 *gmap = (float2 *)((char *)plan + mfma_gather_plan_offset(DH, DW, MH, MW, K, P));
+    const int64_t total = MH * MW * K;
+    const dim3 grid((unsigned)((total + 255) / 256));
+    if (m.mode == kInterpNearest)
+      hipLaunchKernelGGL(build_gather_plan_kernel<1>, grid, dim3(256), 0, s, map, iw, gmap, m.np,
+                         m.weighted, m.wrap, (int)DH, (int)DW, (int)K, total);
+    else
+      hipLaunchKernelGGL(build_gather_plan_kernel<4>, grid, dim3(256), 0, s, map, iw, gmap, m.np,
+                         m.weighted, m.wrap, (int)DH, (int)DW, (int)K, total);
+    MCX_HIP_CHECK_LAUNCH();
+  }
   return 0;
 }
 
@@ -2126,7 +2220,7 @@ int mfma_bias_grad(const TD *g, TD *gb, void *scratch, int64_t B, int64_t C, int
   template int mfma_gather_product<TD>(const TD *, const float *, const float *, const TD *,      \
                                        const TD *, TD *, void *, int64_t, int64_t, int64_t,       \
                                        int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int, \
-                                       hipStream_t);                                              \
+                                       hipStream_t, const void *);                                \
   template int mfma_weight_grad<TD>(const TD *, const TD *, const float *, const float *, TD *,   \
                                     void *, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, \
                                     int64_t, int64_t, int64_t, int, hipStream_t, TD *,            \

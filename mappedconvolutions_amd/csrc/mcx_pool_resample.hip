@@ -675,18 +675,18 @@ inline int corners_of(int interp) { return canonical_interp(interp) == kInterpNe
 // 32-bit entry indices): the caller then runs the atomic scatter instead.
 constexpr int kNotApplicable = -1000;
 
-template <typename T, int OP>
-int launch_transposed(const void *src, const int64_t *idx, const void *map, const void *iw,
-                      void *dst, void *ws, size_t ws_bytes, int64_t planes, int64_t nsrc,
-                      int64_t K, int64_t P, int64_t DH, int64_t DW, int interp, hipStream_t s) {
+// Builds the compressed transposed map of `map` into `ws` (count -> prefix sum -> fill ->
+// per-pixel sort).  `max_codes`: an entry's source code is (location * K + tap), which max
+// unpooling needs to test the recorded winner; otherwise it is the location alone.
+// Returns kNotApplicable when the form does not apply.
+template <typename T>
+int build_transposed(const void *map, const void *iw, void *ws, size_t ws_bytes, int64_t nsrc,
+                     int64_t K, int64_t P, int64_t DH, int64_t DW, int interp, bool max_codes,
+                     hipStream_t s) {
   const int64_t pm = P ? P : 1;
   const int64_t samples = nsrc * K * pm, ndst = DH * DW;
   const TransposedLayout l = transposed_layout(ndst, samples, corners_of(interp), sizeof(T));
   if (!ws || !l.ok || ws_bytes < l.total || nsrc * K > 0xffffffffLL) return kNotApplicable;
-  constexpr int kTCH = planes_per_thread<OP>();
-  const int64_t groups = (planes + kTCH - 1) / kTCH;
-  const int64_t blocks = groups * ((ndst + kThreads - 1) / kThreads);
-  if (blocks > 0x7fffffffLL) return kNotApplicable;
   char *base = (char *)ws;
   uint32_t *local = (uint32_t *)(base + l.local), *cursor = (uint32_t *)(base + l.cursor);
   uint32_t *bsum = (uint32_t *)(base + l.bsum), *e_src = (uint32_t *)(base + l.e_src);
@@ -694,7 +694,7 @@ int launch_transposed(const void *src, const int64_t *idx, const void *map, cons
   int rc = fill<uint32_t>(local, ndst + 1, 0u, s);
   if (rc) return rc;
   if ((rc = fill<uint32_t>(cursor, ndst, 0u, s))) return rc;
-  const int per_code = (int)(OP == UN_MAX ? pm : pm * K);
+  const int per_code = (int)(max_codes ? pm : pm * K);
   const dim3 sgrid(div_up(samples, kThreads)), blk(kThreads);
   MCX_DISPATCH_MODE(interp, hipLaunchKernelGGL((transposed_map_kernel<T, MODE, false>), sgrid, blk,
                                                0, s, (const T *)map, (const T *)iw, samples,
@@ -713,11 +713,43 @@ int launch_transposed(const void *src, const int64_t *idx, const void *map, cons
   hipLaunchKernelGGL((sort_entries_kernel<T>), dim3(div_up(ndst, kThreads)), blk, 0, s, local, bsum,
                      e_src, e_wt, (int)ndst);
   MCX_HIP_CHECK_LAUNCH();
-  hipLaunchKernelGGL((transposed_gather_kernel<T, OP>), dim3((unsigned)blocks), blk, 0, s,
-                     (const T *)src, idx, (T *)dst, local, bsum, e_src, e_wt, planes, (int)nsrc,
-                     (int)ndst, (int)K, (int)(pm * 2), (int)groups);
+  return 0;
+}
+
+// The gather through a built transposed map (in `ws`: a call's workspace or a caller's plan).
+template <typename T, int OP>
+int gather_transposed(const void *src, const int64_t *idx, void *dst, const void *ws,
+                      size_t ws_bytes, int64_t planes, int64_t nsrc, int64_t K, int64_t P,
+                      int64_t DH, int64_t DW, int interp, hipStream_t s) {
+  const int64_t pm = P ? P : 1;
+  const int64_t samples = nsrc * K * pm, ndst = DH * DW;
+  const TransposedLayout l = transposed_layout(ndst, samples, corners_of(interp), sizeof(T));
+  if (!ws || !l.ok || ws_bytes < l.total || nsrc * K > 0xffffffffLL) return kNotApplicable;
+  constexpr int kTCH = planes_per_thread<OP>();
+  const int64_t groups = (planes + kTCH - 1) / kTCH;
+  const int64_t blocks = groups * ((ndst + kThreads - 1) / kThreads);
+  if (blocks > 0x7fffffffLL) return kNotApplicable;
+  const char *base = (const char *)ws;
+  hipLaunchKernelGGL((transposed_gather_kernel<T, OP>), dim3((unsigned)blocks), dim3(kThreads), 0,
+                     s, (const T *)src, idx, (T *)dst, (const uint32_t *)(base + l.local),
+                     (const uint32_t *)(base + l.bsum), (const uint32_t *)(base + l.e_src),
+                     (const T *)(base + l.e_wt), planes, (int)nsrc, (int)ndst, (int)K,
+                     (int)(pm * 2), (int)groups);
   MCX_HIP_CHECK_LAUNCH();
   return 0;
+}
+
+template <typename T, int OP>
+int launch_transposed(const void *src, const int64_t *idx, const void *map, const void *iw,
+                      void *dst, void *ws, size_t ws_bytes, int64_t planes, int64_t nsrc,
+                      int64_t K, int64_t P, int64_t DH, int64_t DW, int interp, hipStream_t s) {
+  const int64_t groups = (planes + planes_per_thread<OP>() - 1) / planes_per_thread<OP>();
+  if (groups * ((DH * DW + kThreads - 1) / kThreads) > 0x7fffffffLL) return kNotApplicable;
+  const int rc = build_transposed<T>(map, iw, ws, ws_bytes, nsrc, K, P, DH, DW, interp,
+                                     OP == UN_MAX, s);
+  if (rc) return rc;
+  return gather_transposed<T, OP>(src, idx, dst, ws, ws_bytes, planes, nsrc, K, P, DH, DW, interp,
+                                  s);
 }
 
 template <typename T, int OP>
@@ -917,4 +949,70 @@ extern "C" int mcx_max_unpool(const void *gout, const int64_t *idx, const void *
                                     IW, OH * OW, K, P, interp, s);
   return launch_max_unpool<double>(gout, idx, map, iw, gin, workspace, workspace_bytes, B, C, IH,
                                    IW, OH * OW, K, P, interp, s);
+}
+
+// ---- scatter plans: the transposed map of one sample map, built once -------------------
+extern "C" size_t mcx_scatter_plan_bytes(int64_t MH, int64_t MW, int64_t DH, int64_t DW, int64_t K,
+                                         int64_t P, int interp, int dtype) {
+  if (bad_dims({MH, MW, MH * MW, K})) return 0;
+  return transposed_workspace(MH * MW, K, P, DH, DW, interp, dtype);
+}
+
+extern "C" int mcx_scatter_plan_build(const void *map, const void *iw, void *plan,
+                                      size_t plan_bytes, int64_t MH, int64_t MW, int64_t DH,
+                                      int64_t DW, int64_t K, int64_t P, int interp, int dtype,
+                                      int for_max_unpool, void *stream) {
+  if (dtype != MCX_F32 && dtype != MCX_F64) return MCX_E_DTYPE;
+  if (!map || !plan || (P > 0) != (iw != nullptr)) return MCX_E_NULL;
+  if (bad_dims({MH, MW, DH, DW, K, MH * MW, DH * DW}) || P < 0) return MCX_E_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  const int rc = dtype == MCX_F32
+                     ? build_transposed<float>(map, iw, plan, plan_bytes, MH * MW, K, P, DH, DW,
+                                               interp, for_max_unpool != 0, s)
+                     : build_transposed<double>(map, iw, plan, plan_bytes, MH * MW, K, P, DH, DW,
+                                                interp, for_max_unpool != 0, s);
+  return rc == kNotApplicable ? MCX_E_WORKSPACE : rc;
+}
+
+namespace {
+template <int OP>
+int planned_gather(const void *src, const int64_t *idx, void *dst, const void *plan,
+                   size_t plan_bytes, int64_t B, int64_t C, int64_t SH, int64_t SW, int64_t DH,
+                   int64_t DW, int64_t K, int64_t P, int interp, int dtype, void *stream) {
+  if (dtype != MCX_F32 && dtype != MCX_F64) return MCX_E_DTYPE;
+  if (!src || !dst || !plan || (OP == UN_MAX && !idx)) return MCX_E_NULL;
+  if (bad_dims({B, C, SH, SW, DH, DW, K, SH * SW, DH * DW}) || P < 0 || B > 65535)
+    return MCX_E_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  const int rc = dtype == MCX_F32
+                     ? gather_transposed<float, OP>(src, idx, dst, plan, plan_bytes, B * C, SH * SW,
+                                                    K, P, DH, DW, interp, s)
+                     : gather_transposed<double, OP>(src, idx, dst, plan, plan_bytes, B * C,
+                                                     SH * SW, K, P, DH, DW, interp, s);
+  return rc == kNotApplicable ? MCX_E_WORKSPACE : rc;
+}
+}  // namespace
+
+extern "C" int mcx_resample_to_map_planned(const void *in, const void *plan, size_t plan_bytes,
+                                           void *out, int64_t B, int64_t C, int64_t IH, int64_t IW,
+                                           int64_t OH, int64_t OW, int64_t P, int interp, int dtype,
+                                           void *stream) {
+  return planned_gather<UN_RESAMPLE>(in, nullptr, out, plan, plan_bytes, B, C, IH, IW, OH, OW, 1, P,
+                                     interp, dtype, stream);
+}
+
+extern "C" int mcx_avg_unpool_planned(const void *gout, const void *plan, size_t plan_bytes,
+                                      void *gin, int64_t B, int64_t C, int64_t IH, int64_t IW,
+                                      int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
+                                      int dtype, void *stream) {
+  return planned_gather<UN_AVG>(gout, nullptr, gin, plan, plan_bytes, B, C, OH, OW, IH, IW, K, P,
+                                interp, dtype, stream);
+}
+
+extern "C" int mcx_max_unpool_planned(const void *gout, const int64_t *idx, const void *plan,
+                                      size_t plan_bytes, void *gin, int64_t B, int64_t C,
+                                      int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
+                                      int64_t P, int interp, int dtype, void *stream) {
+  return planned_gather<UN_MAX>(gout, idx, gin, plan, plan_bytes, B, C, OH, OW, IH, IW, K, P, interp,
+                                dtype, stream);
 }
