@@ -910,6 +910,9 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
             load_tap(0);
             issue(cb + 1);
           }
+          // The products of a unit issue back to back: at the default priority the other
+          // waves of the SIMD slip their vector work in between and the matrix pipe idles.
+          __builtin_amdgcn_s_setprio(1);
           if constexpr (kBf16) {
 #pragma unroll
             for (int s = 0; s < 4; s++) {
@@ -920,15 +923,17 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
                 acc[k][cb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aregb[mb][s], bq,
                                                                          acc[k][cb][mb], 0, 0, 0);
             }
-          } else
+          } else {
 #pragma unroll
-          for (int s4 = 0; s4 < 8; s4++) {
-            const float4 bq = *reinterpret_cast<const float4 *>(&S[buf][l15][16 * s4 + 4 * lq]);
-            acc[k][cb][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[4 * s4 + 0], bq.x, acc[k][cb][0], 0, 0, 0);
-            acc[k][cb][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[4 * s4 + 1], bq.y, acc[k][cb][0], 0, 0, 0);
-            acc[k][cb][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[4 * s4 + 2], bq.z, acc[k][cb][0], 0, 0, 0);
-            acc[k][cb][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[4 * s4 + 3], bq.w, acc[k][cb][0], 0, 0, 0);
+            for (int s4 = 0; s4 < 8; s4++) {
+              const float4 bq = *reinterpret_cast<const float4 *>(&S[buf][l15][16 * s4 + 4 * lq]);
+              acc[k][cb][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[4 * s4 + 0], bq.x, acc[k][cb][0], 0, 0, 0);
+              acc[k][cb][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[4 * s4 + 1], bq.y, acc[k][cb][0], 0, 0, 0);
+              acc[k][cb][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[4 * s4 + 2], bq.z, acc[k][cb][0], 0, 0, 0);
+              acc[k][cb][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[4 * s4 + 3], bq.w, acc[k][cb][0], 0, 0, 0);
+            }
           }
+          __builtin_amdgcn_s_setprio(0);
         }
       }
     }
@@ -944,9 +949,11 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
       if ((tid & 3) == 0 && a < A) plain_sum_part[(int64_t)range * A + a] = t;
     }
   }
-  // partial gW of this workgroup: lane holds gathered channel l15 of each block and
-  // plain channels a0 + 16*(wave*MB + mb) + 4*lq + i
-  float *pr = part + (int64_t)range * A * G * K;
+  // partial gW of this workgroup, stored [tap][gathered channel][plain channel] (rows padded to
+  // a multiple of four): the lane holds gathered channel l15 of each block and four
+  // consecutive plain channels a0 + 16*(wave*MB + mb) + 4*lq + i, one 16-byte store
+  const int A4 = (A + 3) & ~3;
+  float *pr = part + (int64_t)range * A4 * G * K;
 #pragma unroll
   for (int k = 0; k < kWgKT; k++) {
     if (k < ktaps) {
@@ -954,29 +961,32 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
       for (int cb = 0; cb < kWgCB; cb++) {
         const int g = g_first + cb * kGC + l15;
 #pragma unroll
-        for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-          for (int i = 0; i < 4; i++) {
-            const int a = a0 + (wave * MB + mb) * 16 + lq * 4 + i;
-            if (a < A && g < G) pr[((int64_t)a * G + g) * K + k_base + k] = acc[k][cb][mb][i];
-          }
+        for (int mb = 0; mb < MB; mb++) {
+          const int a = a0 + (wave * MB + mb) * 16 + lq * 4;
+          if (a < A && g < G)
+            *reinterpret_cast<floatx4 *>(&pr[((int64_t)(k_base + k) * G + g) * A4 + a]) =
+                acc[k][cb][mb];
+        }
       }
     }
   }
 }
 
-// out[e] = sum over ranges of part[r][e], for two independent jobs in one launch (the second
-// may be empty).  64 x 4 threads: four quarters of the ranges are summed side by side (eight
-// loads in flight each) and combined in a fixed order, so the result does not depend on
-// scheduling.
+// Sums per-range partials, two independent jobs in one launch (the second may be empty):
+//   out[a][g][k] = sum over ranges of part[r][k][g][a]   (rows of A4 >= A entries), and
+//   out2[e]      = sum over ranges of part2[r][e].
+// 64 x 4 threads: four quarters of the ranges are summed side by side (eight loads in flight
+// each) and combined in a fixed order, so the result does not depend on scheduling.
 template <typename TD>
 __global__ __launch_bounds__(256) void reduce_partials_kernel(
-    const float *__restrict__ part, TD *__restrict__ out, int64_t n,
+    const float *__restrict__ part, TD *__restrict__ out, int A, int A4, int G, int K,
     const float *__restrict__ part2, TD *__restrict__ out2, int64_t n2, int ranges) {
   __shared__ float quarter[4][64];
+  int64_t n = (int64_t)K * G * A4;
   const int blocks1 = (int)((n + 63) / 64);
   int64_t e = (int64_t)blockIdx.x * 64 + threadIdx.x;
-  if ((int)blockIdx.x >= blocks1) {  // second job
+  const bool second = (int)blockIdx.x >= blocks1;
+  if (second) {
     e -= (int64_t)blocks1 * 64;
     part = part2;
     out = out2;
@@ -998,9 +1008,18 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(
   }
   quarter[threadIdx.y][threadIdx.x] = s;
   __syncthreads();
-  if (threadIdx.y == 0 && e < n)
-    out[e] = from_f32<TD>(((quarter[0][threadIdx.x] + quarter[1][threadIdx.x]) +
+  if (threadIdx.y == 0 && e < n) {
+    int64_t o = e;
+    if (!second) {
+      const int a = (int)(e % A4);
+      const int64_t kg = e / A4;  // k * G + g
+      const int g = (int)(kg % G), k = (int)(kg / G);
+      if (a >= A) return;
+      o = ((int64_t)a * G + g) * K + k;
+    }
+    out[o] = from_f32<TD>(((quarter[0][threadIdx.x] + quarter[1][threadIdx.x]) +
                            quarter[2][threadIdx.x]) + quarter[3][threadIdx.x]);
+  }
 }
 
 // ---------------------------------------------------------------------------------
@@ -1622,7 +1641,7 @@ size_t mfma_weight_grad_bytes(int64_t B, int64_t A, int64_t G, int64_t MH, int64
   const size_t ranges =
       (size_t)std::max(weight_grad_ranges<float>(make_tiling(B, MH, MW, 4).total, A, G, K),
                        weight_grad_ranges<bf16_t>(make_tiling(B, MH, MW, 2).total, A, G, K));
-  size_t n = align256(ranges * (size_t)(A * G * K) * sizeof(float));
+  size_t n = align256(ranges * (size_t)(round_up(A, 4) * G * K) * sizeof(float));
   n += align256(ranges * (size_t)A * sizeof(float));
   n += 256;  // the map's pair mask
   if (GH == 1) n += align256((size_t)(B * GH * GW * round_up(G, kGC)) * sizeof(float));
@@ -1646,8 +1665,8 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
   const int64_t Gpad = round_up(G, kGC);
   const bool cl = use_channel_last(GH, interp) &&
                   GH * GW * Gpad * (int64_t)sizeof(TD) <= 0xffffffffLL;
-  float *sum_part = reinterpret_cast<float *>((char *)scratch +
-                                              align256((size_t)ranges * (size_t)(A * G * K) * 4));
+  float *sum_part = reinterpret_cast<float *>(
+      (char *)scratch + align256((size_t)ranges * (size_t)(round_up(A, 4) * G * K) * 4));
   int *pair_mask = reinterpret_cast<int *>((char *)sum_part + align256((size_t)ranges * A * 4));
   if (cl) {
     TD *stage = reinterpret_cast<TD *>((char *)pair_mask + 256);
@@ -1700,10 +1719,11 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
 #undef MCX_LAUNCH_NA
 #undef MCX_LAUNCH_CL
   MCX_HIP_CHECK_LAUNCH();
-  const int64_t n = A * G * K;
+  const int64_t n = round_up(A, 4) * G * K;
   const int64_t n2 = plain_sum ? A : 0;
   hipLaunchKernelGGL(reduce_partials_kernel<TD>, dim3((unsigned)((n + 63) / 64 + (n2 + 63) / 64)),
-                     dim3(64, 4), 0, s, part, gw, n, sum_part, plain_sum, n2, ranges);
+                     dim3(64, 4), 0, s, part, gw, (int)A, (int)round_up(A, 4), (int)G, (int)K,
+                     sum_part, plain_sum, n2, ranges);
   MCX_HIP_CHECK_LAUNCH();
   return 0;
 }
