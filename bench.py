@@ -29,20 +29,35 @@ B, CI, CO, H, W, K = 8, 64, 64, 256, 512, 9
 PEAK_FP32_MFMA_TFLOPS = 157.3
 GEMM_FLOP = 2.0 * B * H * W * CO * CI * K  # one of the three products
 
-# Bytes that cross the L2 boundary per launch (bilinear workload), from FETCH_SIZE and WRITE_SIZE
-# counter passes of this script scaled by a copy kernel of known size (x2.0 KiB and x1.0 KiB per
-# count); profiles/conv_fwd_bwd_headline_hbm_traffic.txt holds the runs.  Counters cannot be read
-# from inside the process, so the figures are the recorded ones; other workloads report null.
-MEASURED_TRAFFIC_BYTES = {
-    "conv_forward": 906.1e6 + 268.4e6,
-    "conv_backward_input": 1432.5e6 + 268.4e6,
-    "conv_backward_weight": 1535.9e6 + 89.1e6,
-}
-KERNEL_OF = {
-    "conv_forward": "gather_product_mfma_kernel<float,4,1,1,false,2>",
-    "conv_backward_input": "gather_product_mfma_kernel<float,1,4,1,false,2>",
-    "conv_backward_weight": "weight_grad_mfma_kernel<float,4,1,false,2>",
-}
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "conv_fwd_bwd_headline_hbm_traffic.txt")
+
+
+def recorded_traffic():
+    """Kernel name and bytes crossing the L2 boundary per launch, per timed C-ABI call, from the
+    committed counter summary (FETCH_SIZE / WRITE_SIZE passes of this script, scaled by copy
+    dispatches of known size; mappedconvolutions_amd/traffic_summary.py writes it).  Counters
+    cannot be read from inside the process, so these are recorded figures: they are dropped when
+    the kernel source has changed since the counter run."""
+    import hashlib
+    import re
+    table, fresh = {}, False
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return {}, False
+    for line in text.splitlines():
+        m = re.match(r"@source sha256=(\w+) file=(\S+)", line)
+        if m:
+            try:
+                with open(os.path.join(ROOT, m.group(2)), "rb") as f:
+                    fresh = hashlib.sha256(f.read()).hexdigest() == m.group(1)
+            except OSError:
+                fresh = False
+        m = re.match(r'@traffic label=(\w+) kernel="([^"]+)" read_bytes=(\d+) written_bytes=(\d+)',
+                     line)
+        if m:
+            table[m.group(1)] = (m.group(2), int(m.group(3)) + int(m.group(4)))
+    return table, fresh
 
 
 def make_inputs(device, batch=B):
@@ -143,6 +158,8 @@ def main():
     achieved = GEMM_FLOP / (kernel_ms[dominant] * 1e-3) / 1e12
 
     ms = elapsed / args.steps * 1e3
+    # (the recorded counter runs cover the bilinear headline workload without a plan cache)
+    recorded, fresh = recorded_traffic() if interp == 1 and not args.map_plan_cache else ({}, False)
     out = {
         "metric": "Mapped-conv fwd+bwd Mpix/s (B8,C64,256x512,3x3); % HBM/MFMA roofline",
         "value": round(B * H * W / (ms * 1e-3) / 1e6, 3),
@@ -154,12 +171,14 @@ def main():
         "config": {"workload": "MappedConvolution fwd+bwd B8 Ci64 Co64 256x512 K9 latitude map, "
                                + args.interp, "interpolation": args.interp,
                    "map_plan_cache": bool(args.map_plan_cache)},
-        "roofline": {"bound": "mfma", "kernel": KERNEL_OF.get(dominant, dominant) if interp == 1
-                     else dominant,
+        "roofline": {"bound": "mfma", "kernel": recorded.get(dominant, (dominant, None))[0],
                      "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(dominant) if interp == 1 else None,
-                     "traffic_unit": "bytes per launch"},
+                     "traffic": recorded[dominant][1] if fresh and dominant in recorded else None,
+                     "traffic_unit": "bytes per launch",
+                     "traffic_source": "profiles/conv_fwd_bwd_headline_hbm_traffic.txt"
+                                       if fresh and dominant in recorded else
+                                       "none: no counter run of this kernel source is recorded"},
         "kernel_ms": {k: round(v, 4) for k, v in kernel_ms.items()},
     }
     if not args.no_cpu_baseline:

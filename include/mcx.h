@@ -277,9 +277,16 @@ int mcx_tconv_backward_planned(const void *gy, const void *map, const void *iw, 
  * ref [B,D,R], query [B,D,Q] (points are columns) -> idx int64 [B,k,Q]
  * (1-based reference index, row j = j-th nearest, ties keep the lower index),
  * dist [B,k,Q] (Euclidean).  k <= 64; F32 and F64.  The R x Q distance matrix
- * of the reference is never formed. */
-int mcx_knn(const void *ref, const void *query, int64_t *idx, void *dist, int64_t B, int64_t D,
-            int64_t R, int64_t Q, int64_t k, int dtype, void *stream);
+ * of the reference is never formed.
+ * workspace (optional): mcx_knn_workspace(B, D, R, dtype) bytes, nonzero for points of one to
+ * three dimensions and at least 512 reference points.  With it the reference points are
+ * binned into a uniform grid and every query only visits the cells around it; the result is
+ * the same bit for bit (same distance arithmetic, same order among equal distances).
+ * Without it (NULL) every query walks every reference point. */
+size_t mcx_knn_workspace(int64_t B, int64_t D, int64_t R, int dtype);
+int mcx_knn(const void *ref, const void *query, int64_t *idx, void *dist, void *workspace,
+            size_t workspace_bytes, int64_t B, int64_t D, int64_t R, int64_t Q, int64_t k,
+            int dtype, void *stream);
 
 /* ---- sample-map builders and cube-map resampling ----------------------------- */
 

@@ -662,9 +662,14 @@ def knn_forward(ref, query, k):
     Q, k = query.shape[2], int(k)
     idx = torch.empty((B, k, Q), dtype=torch.int64, device=ref.device)
     dist = torch.empty((B, k, Q), dtype=ref.dtype, device=ref.device)
+    lib = _lib.load()
     with torch.cuda.device(ref.device):
-        rc = _lib.load().mcx_knn(_ptr(ref), _ptr(query), _ptr(idx), _ptr(dist), B, D, R, Q, k, dt,
-                                 _stream(ref))
+        # (the grid search's bins; 0 bytes where it does not apply and every point is walked)
+        ws_bytes = lib.mcx_knn_workspace(B, D, R, dt)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=ref.device) if ws_bytes else None
+        rc = lib.mcx_knn(_ptr(ref), _ptr(query), _ptr(idx), _ptr(dist),
+                         _ptr(ws) if ws is not None else None, ws_bytes, B, D, R, Q, k, dt,
+                         _stream(ref))
     _lib.check(rc, "knn_forward")
     return [idx, dist]
 

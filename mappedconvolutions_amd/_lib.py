@@ -49,7 +49,8 @@ SIGNATURES = {
     "mcx_resample_to_map_planned": (_i, [_p] * 2 + [_sz, _p] + [_i64] * 7 + [_i, _i, _p]),
     "mcx_avg_unpool_planned": (_i, [_p] * 2 + [_sz, _p] + [_i64] * 8 + [_i, _i, _p]),
     "mcx_max_unpool_planned": (_i, [_p] * 3 + [_sz, _p] + [_i64] * 8 + [_i, _i, _p]),
-    "mcx_knn": (_i, [_p] * 4 + [_i64] * 5 + [_i, _p]),
+    "mcx_knn_workspace": (_sz, [_i64] * 3 + [_i]),
+    "mcx_knn": (_i, [_p] * 5 + [_sz] + [_i64] * 5 + [_i, _p]),
     "mcx_projection_map": (_i, [_p] + [_i64] * 4 + [_i] + [_i64] * 2 + [_p]),
     "mcx_cube_projection_map": (_i, [_p] + [_i64] * 4 + [_p]),
     "mcx_cube2rect": (_i, [_p] * 2 + [_i64] * 4 + [_i, _i, _p]),

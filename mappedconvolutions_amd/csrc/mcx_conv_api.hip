@@ -588,7 +588,7 @@ extern "C" int mcx_tconv_backward(const void *gy, const void *map, const void *i
                                                 workspace_bytes, d, interp, s));
 }
 
-extern "C" int mcx_abi_version(void) { return 9; }
+extern "C" int mcx_abi_version(void) { return 10; }
 
 extern "C" int mcx_profile_dominant_kernel(void *start_event, void *stop_event) {
   mcx::set_profile_events(start_event, stop_event);

@@ -44,7 +44,7 @@ def test_rejected_arguments_return_codes_without_a_gpu():
     assert lib.mcx_conv_forward_workspace(1, 64, 64, 8, 8, 8, 8, 9, 0, 1) == 0  # fp64: scalar kernels
     assert lib.mcx_resample_from_map(1, 1, None, 1, 0, 1, 4, 4, 4, 4, 0, 1, 0, None) == -2
     assert lib.mcx_resample_from_map(1, 1, None, 1, 1, 1, 4, 4, 4, 4, 0, 1, 7, None) == -1
-    assert lib.mcx_knn(1, 1, 1, 1, 1, 3, 10, 10, 65, 0, None) == -2
+    assert lib.mcx_knn(1, 1, 1, 1, None, 0, 1, 3, 10, 10, 65, 0, None) == -2
     # map builders: NULL output, a spherical grid of one row (divides by H - 1), unknown projection
     assert lib.mcx_projection_map(None, 8, 16, 3, 3, 1, 1, 1, None) == -3
     assert lib.mcx_projection_map(1, 1, 16, 3, 3, 1, 1, 1, None) == -2
