@@ -93,6 +93,18 @@ __device__ inline float buf_load(plane_buf_t r, unsigned byte_off, float) {
 __device__ inline double buf_load(plane_buf_t r, unsigned byte_off, double) {
   return __builtin_bit_cast(double, __builtin_amdgcn_raw_buffer_load_b64(r, (int)byte_off, 0, 0));
 }
+// Stores through a buffer resource: one whose byte offset lies beyond the size is dropped, so
+// a lane with nothing to store passes kOobOffset instead of branching around the store.
+typedef unsigned buf_u32x2 __attribute__((ext_vector_type(2)));
+__device__ inline void buf_store(plane_buf_t r, unsigned byte_off, float v) {
+  __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, (int)byte_off, 0, 0);
+}
+__device__ inline void buf_store(plane_buf_t r, unsigned byte_off, double v) {
+  __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(buf_u32x2, v), r, (int)byte_off, 0, 0);
+}
+__device__ inline void buf_store(plane_buf_t r, unsigned byte_off, int64_t v) {
+  __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(buf_u32x2, v), r, (int)byte_off, 0, 0);
+}
 // Two neighbouring elements with one load (the address need only be element-aligned).
 struct float_pair { float x, y; };
 struct double_pair { double x, y; };
@@ -145,6 +157,7 @@ struct Tap<T, kInterpNearest> {
   }
   static constexpr int kCorners = 1;
   __device__ inline int corner_off(int) const { return off; }
+  __device__ inline void set_corner_off(int, int v) { off = v; }
   __device__ inline T corner_wt(int) const { return T(1); }
 };
 
@@ -245,6 +258,7 @@ struct Tap {
   }
   static constexpr int kCorners = 4;
   __device__ inline int corner_off(int i) const { return off[i]; }
+  __device__ inline void set_corner_off(int i, int v) { off[i] = v; }
   __device__ inline T corner_wt(int i) const { return wt[i]; }
 };
 

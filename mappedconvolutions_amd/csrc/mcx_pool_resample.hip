@@ -4,6 +4,8 @@
 // channels: the tap (offsets + weights) is resolved once and applied to each of
 // the thread's channel planes, so map decoding is amortised and neighbouring lanes
 // read neighbouring pixels.
+#include <type_traits>
+
 #include "mcx_device.h"
 
 namespace mcx {
@@ -192,11 +194,304 @@ __device__ inline void direct_gather(const T *__restrict__ in, const T *__restri
   }
 }
 
+// ---------------------------------------------------------------------------------
+// Pooling through LDS windows.  The texture path resolves four lanes' addresses per clock
+// whatever the width of the load, so a gather of single elements (nine taps of two corners
+// per output and channel) is bound by it long before memory.  Where the taps of a wave's 64
+// neighbouring outputs read a few source rows over short spans - the distortion-aware kernels
+// of equirectangular images do: every tap of a row segment stays in one source row and moves
+// with the pixel - those spans are copied to LDS with 16-byte loads, one lane per four
+// elements, and the taps read LDS.  Every wave works alone (its own windows, no workgroup
+// barrier) and finds its spans from the map itself:
+//   * per (tap, corner row): the source row must be the same for every lane that uses it,
+//     and the columns must lie within a short distance (cyclic in the width, so a seam
+//     inside the segment is no obstacle) after the first lane's;
+//   * entries of one source row that lie close together share a row window; lane s of the
+//     wave keeps row window s while they are merged;
+//   * if anything does not fit, the wave takes the register path above.
+// The arithmetic per output is that of the register path (Tap::combine on the same values).
+// ---------------------------------------------------------------------------------
+constexpr int kWinChunks = 128;   // 16-byte chunks per window, followed by one of zeros
+constexpr int kWinRows = 6;
+constexpr int kWinSpanCap = 400;  // elements between the first and the last column of a span
+constexpr int kWinTaps = 9;
+constexpr int kWinDepth = 4;      // channels whose loads are in flight
+
+template <typename T, int MODE>
+struct WinShape {
+  static constexpr int kRowsPerTap = Tap<T, MODE>::kCorners == 4 ? 2 : 1;
+  static constexpr int kColsPerRow = Tap<T, MODE>::kCorners == 4 ? 2 : 1;
+  static constexpr int kEntries = kWinTaps * kRowsPerTap;
+};
+
+__device__ inline int cyc(int v, int w) { return v < 0 ? v + w : v; }  // v in (-w, w)
+
+// Largest value of the wave (all 64 lanes active), by data-parallel-primitive moves inside the
+// vector unit: shifts within rows of 16 lanes, then the rows' last lanes passed on; lanes a
+// step does not reach keep the identity.  (Shuffles go through LDS, a round trip per step.)
+__device__ inline int wave_max(int v) {
+  constexpr int kId = -0x7fffffff - 1;
+  v = max(v, __builtin_amdgcn_update_dpp(kId, v, 0x111, 0xf, 0xf, false));  // row_shr:1
+  v = max(v, __builtin_amdgcn_update_dpp(kId, v, 0x112, 0xf, 0xf, false));  // row_shr:2
+  v = max(v, __builtin_amdgcn_update_dpp(kId, v, 0x114, 0xf, 0xe, false));  // row_shr:4
+  v = max(v, __builtin_amdgcn_update_dpp(kId, v, 0x118, 0xf, 0xc, false));  // row_shr:8
+  v = max(v, __builtin_amdgcn_update_dpp(kId, v, 0x142, 0xa, 0xf, false));  // row_bcast:15
+  v = max(v, __builtin_amdgcn_update_dpp(kId, v, 0x143, 0xc, 0xf, false));  // row_bcast:31
+  return __builtin_amdgcn_readlane(v, 63);
+}
+
+// Returns false (wave-uniform) when the wave's taps do not fit windows; nothing is written then.
 template <typename T, int MODE, int OP>
-__global__ __launch_bounds__(kThreads) void gather_kernel(
+__device__ inline bool window_pool(const T *__restrict__ in, const T *__restrict__ map,
+                                   T *__restrict__ out, int64_t *__restrict__ idx, int C, int IH,
+                                   int IW, int N, int K, int n, bool live, int c0, int b,
+                                   int cpt) {
+  using Shape = WinShape<T, MODE>;
+  constexpr int kRPT = Shape::kRowsPerTap, kCPR = Shape::kColsPerRow, kEnt = Shape::kEntries;
+  constexpr int kCorners = Tap<T, MODE>::kCorners;
+  constexpr int kPer = 16 / (int)sizeof(T);  // elements per chunk
+  constexpr unsigned kZeroOff = kWinChunks * 16;
+  __shared__ uint4 win[kThreads / 64][2][kWinChunks + 1];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
+  // this thread's taps, and for every tap the row / (cyclic) column of its first corner
+  Tap<T, MODE> taps[kWinTaps];
+  int ty[kWinTaps], tx[kWinTaps];
+#pragma unroll
+  for (int k = 0; k < kWinTaps; k++) {
+    const int64_t e = (int64_t)(live ? n : 0) * K + min(k, K - 1);
+    const T x = map[e * 2], y = map[e * 2 + 1];
+    taps[k].set(x, y, IH, IW);
+    if (MODE == kInterpNearest) {
+      tx[k] = to_int(round_half_away(x));
+      ty[k] = to_int(round_half_away(y));
+    } else {
+      tx[k] = to_int(mcx_floor(x));
+      ty[k] = to_int(mcx_floor(y));
+    }
+    tx[k] = wrap_index(tx[k], IW);
+  }
+  // Entries: (tap, corner row) pairs in use.  Everything about them is wave-uniform.
+  bool fits = true;
+  unsigned rows_used = 0;  // bit (k * kRPT + r)
+  int e_row[kEnt], e_col[kEnt], e_len[kEnt];
+#pragma unroll
+  for (int k = 0; k < kWinTaps; k++) {
+#pragma unroll
+    for (int r = 0; r < kRPT; r++) {
+      const int e = k * kRPT + r;
+      const bool use = live && k < K && taps[k].row_in_use(r);
+      const unsigned long long bu = __builtin_amdgcn_ballot_w64(use);
+      e_row[e] = e_col[e] = e_len[e] = 0;
+      if (bu) {
+        const int first = __builtin_ctzll(bu);
+        const int row = ty[k] + r;
+        e_row[e] = __builtin_amdgcn_readlane(row, first);
+        e_col[e] = __builtin_amdgcn_readlane(tx[k], first);
+        const int far = wave_max(use ? cyc(tx[k] - e_col[e], IW) : 0);
+        if (__builtin_amdgcn_ballot_w64(use && row != e_row[e]) != 0 || far > kWinSpanCap)
+          fits = false;
+        e_len[e] = far + kCPR;
+        rows_used |= 1u << e;
+      }
+    }
+  }
+  // Second corner rows in use (row coordinates that are not integral): four offsets and
+  // weights per tap plus the loads in flight do not fit the register budget of four waves per
+  // SIMD, and spilling inside the channel loop costs more than the texture path does.
+  constexpr unsigned kSecondRows = kRPT == 2 ? 0x2aaaau : 0u;  // bits k * 2 + 1
+  if (!fits || !rows_used || (rows_used & kSecondRows)) return false;
+  // Row windows: lane s keeps window s (source row, first column, length in elements).
+  int r_row = 0, r_start = 0, r_len = 0, nrows = 0;
+  int e_slot[kEnt];
+#pragma unroll
+  for (int e = 0; e < kEnt; e++) {
+    e_slot[e] = 0;
+    if ((rows_used >> e) & 1u) {
+      const int d = cyc(e_col[e] - r_start, IW), d2 = cyc(r_start - e_col[e], IW);
+      const bool mine = lane < nrows && r_row == e_row[e] && min(d, d2) <= kWinSpanCap;
+      const unsigned long long bm = __builtin_amdgcn_ballot_w64(mine);
+      if (bm) {
+        e_slot[e] = __builtin_ctzll(bm);
+        if (lane == e_slot[e]) {
+          if (d <= d2) {  // starts inside or after the window
+            r_len = max(r_len, d + e_len[e]);
+          } else {  // starts before it
+            r_len = max(e_len[e], d2 + r_len);
+            r_start = e_col[e];
+          }
+        }
+      } else {
+        e_slot[e] = nrows;
+        if (lane == nrows) {
+          r_row = e_row[e];
+          r_start = e_col[e];
+          r_len = e_len[e];
+        }
+        nrows++;
+      }
+    }
+  }
+  // windows start on a chunk boundary; one that reaches all the way round is the whole row
+  int r_first = r_start & ~(kPer - 1);
+  r_len += r_start - r_first;
+  if (r_len >= IW) {
+    r_len = IW;
+    r_first = 0;
+  }
+  const int r_chunks = lane < nrows ? (r_len + kPer - 1) / kPer : 0;
+  int r_chunk0 = 0, chunks = 0;
+#pragma unroll
+  for (int s2 = 0; s2 < kWinRows; s2++) {
+    if (lane == s2) r_chunk0 = chunks;
+    chunks += __builtin_amdgcn_readlane(r_chunks, s2);
+  }
+  if (nrows > kWinRows || chunks > kWinChunks) return false;
+
+  // LDS byte offset of every corner (the zero chunk for corners outside the plane or of
+  // weight zero), kept where the register path keeps the element offsets
+#pragma unroll
+  for (int k = 0; k < kWinTaps; k++) {
+#pragma unroll
+    for (int r = 0; r < kRPT; r++) {
+      const int e = k * kRPT + r;
+      const bool used = (rows_used >> e) & 1u;
+      const int first = __builtin_amdgcn_readlane(r_first, e_slot[e]);
+      const int base = __builtin_amdgcn_readlane(r_chunk0, e_slot[e]) * kPer;
+      const int col = cyc(tx[k] - first, IW);
+#pragma unroll
+      for (int i = 0; i < kCPR; i++) {
+        int cc = col + i;
+        cc = cc >= IW ? cc - IW : cc;
+        const bool valid = live && used && taps[k].corner_off(r * kCPR + i) >= 0;
+        taps[k].set_corner_off(r * kCPR + i,
+                               valid ? (int)((unsigned)(base + cc) * (unsigned)sizeof(T))
+                                     : (int)kZeroOff);
+      }
+    }
+  }
+  // the chunks this lane copies per channel: byte offset in the plane, or out of range
+  unsigned goff[2];
+#pragma unroll
+  for (int j = 0; j < 2; j++) {
+    const int q = lane + j * 64;
+    goff[j] = kOobOffset;
+#pragma unroll
+    for (int s2 = 0; s2 < kWinRows; s2++) {
+      const int c_0 = __builtin_amdgcn_readlane(r_chunk0, s2);
+      const int c_n = __builtin_amdgcn_readlane(r_chunks, s2);
+      const int c_y = __builtin_amdgcn_readlane(r_row, s2);
+      const int c_x = __builtin_amdgcn_readlane(r_first, s2);
+      int x = c_x + (q - c_0) * kPer;
+      x = x >= IW ? x - IW : x;
+      if (q >= c_0 && q < c_0 + c_n) goff[j] = (unsigned)(c_y * IW + x) * (unsigned)sizeof(T);
+    }
+  }
+
+  const int64_t plane = (int64_t)IH * IW;
+  const unsigned plane_bytes = (unsigned)(plane * (int64_t)sizeof(T));
+  const T *src = in + ((int64_t)b * C + c0) * plane;
+  const int nc = min(cpt, C - c0);
+  const int64_t o_plane = ((int64_t)b * C + c0) * N;
+  const int64_t idx_base = (int64_t)n * K * 2;
+  // Per channel: its window's chunks travel memory -> registers -> LDS.  The loads of
+  // kWinDepth channels are in flight (one channel's arithmetic is far shorter than a load's
+  // latency); LDS holds two windows, the one being read and the one being filled.  A wave's
+  // LDS accesses execute in order, so the wave needs no barrier between filling a window
+  // and reading it; wave_barrier() only keeps the compiler from moving them.
+  uint4 pre[kWinDepth][2];
+  auto fetch = [&](int c, int slot) {
+    const plane_buf_t pl = plane_buf(src + c * plane, plane_bytes);
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+      pre[slot][j] =
+          __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(pl, (int)goff[j], 0, 0));
+  };
+  auto stash = [&](int slot, int buf) {
+    win[wave][buf][lane] = pre[slot][0];
+    win[wave][buf][lane + 64] = pre[slot][1];
+    __builtin_amdgcn_wave_barrier();
+  };
+  if (lane < 2) win[wave][lane][kWinChunks] = make_uint4(0u, 0u, 0u, 0u);
+  // FULL (all kWinTaps taps exist) is settled once per wave rather than per tap and channel,
+  // with one copy of the channel loop for each answer.  Only the first corner row of a tap is
+  // read: the products of the second are zeros here, so the sum differs from the register
+  // path's at most in the sign of a zero.
+  auto run = [&](auto full_tag) {
+    constexpr bool FULL = decltype(full_tag)::value;
+    constexpr int kRead = kCPR;
+    auto compute = [&](int c, int buf) {
+      const char *wb = reinterpret_cast<const char *>(&win[wave][buf][0]);
+      // every read is unconditional (a corner that is not in use reads the zero chunk), so
+      // all of a channel's reads are in flight together
+      T d[kWinTaps][kCorners];
+#pragma unroll
+      for (int k = 0; k < kWinTaps; k++)
+#pragma unroll
+        for (int i = 0; i < kRead; i++)
+          d[k][i] = *reinterpret_cast<const T *>(wb + (unsigned)taps[k].corner_off(i));
+      __builtin_amdgcn_sched_barrier(0);
+      T val[kWinTaps];
+#pragma unroll
+      for (int k = 0; k < kWinTaps; k++) {
+        if (kRead == kCorners)
+          val[k] = taps[k].combine(d[k]);
+        else
+          val[k] = taps[k].corner_wt(0) * d[k][0] + taps[k].corner_wt(1) * d[k][1];
+      }
+      T a = OP == OP_MAX ? T(-3.402823466e+38F) : T(0);
+      int bk = -1;
+#pragma unroll
+      for (int k = 0; k < kWinTaps; k++) {
+        if (OP == OP_MAX) {
+          const bool better = (FULL || k < K) && val[k] > a;
+          a = better ? val[k] : a;
+          bk = better ? k : bk;
+        } else {
+          a = (FULL || k < K) ? a + val[k] : a;
+        }
+      }
+      // (stores without a branch: lanes past the row's end and channels past the last one
+      // store out of range, which drops the store)
+      const int cc = min(c, nc - 1);
+      const bool keep = live && c < nc;
+      buf_store(plane_buf(out + o_plane + (int64_t)cc * N, (unsigned)N * (unsigned)sizeof(T)),
+                keep ? (unsigned)n * (unsigned)sizeof(T) : kOobOffset,
+                OP == OP_AVG ? a / (T)K : a);
+      if (OP == OP_MAX)
+        buf_store(plane_buf(idx + o_plane + (int64_t)cc * N, (unsigned)N * 8u),
+                  keep ? (unsigned)n * 8u : kOobOffset,
+                  bk < 0 ? (int64_t)-1 : idx_base + 2 * bk);
+      __builtin_amdgcn_wave_barrier();
+    };
+    // (the loop runs over a whole number of rings and re-reads the last channel past the end:
+    // with the same loads and stores on every path the compiler can count how many may still
+    // be in flight at each wait; a load behind a test makes every wait a full one)
+#pragma unroll
+    for (int u = 0; u < kWinDepth; u++) fetch(min(u, nc - 1), u);
+    stash(0, 0);
+    for (int cb = 0; cb < nc; cb += kWinDepth) {
+#pragma unroll
+      for (int u = 0; u < kWinDepth; u++) {
+        const int c = cb + u;
+        fetch(min(c + kWinDepth, nc - 1), u);  // slot u went to LDS in the previous step
+        compute(c, u & 1);
+        stash((u + 1) % kWinDepth, (u + 1) & 1);
+      }
+    }
+  };
+  if (K == kWinTaps)
+    run(std::true_type());
+  else
+    run(std::false_type());
+  return true;
+}
+
+template <typename T, int MODE, int OP>
+__global__ __launch_bounds__(kThreads, 4) void gather_kernel(
     const T *__restrict__ in, const T *__restrict__ map, const T *__restrict__ iw,
     T *__restrict__ out, int64_t *__restrict__ idx, int C, int IH, int IW, int N, int MW, int K,
-    int P, int cpt) {
+    int P, int cpt, int windows) {
   constexpr int kTileW = Patch<OP>::kW, kTileH = Patch<OP>::kH;
   const int tiles_x = (MW + kTileW - 1) / kTileW;
   // (pooling only: a resampling map's rows need not read neighbouring source rows, and the
@@ -205,7 +500,14 @@ __global__ __launch_bounds__(kThreads) void gather_kernel(
   const int tx = (tile % tiles_x) * kTileW + threadIdx.x % kTileW;
   const int ty = (tile / tiles_x) * kTileH + threadIdx.x / kTileW;
   const int n = ty * MW + tx;
-  if (tx >= MW || n >= N) return;
+  const bool live = tx < MW && n < N;
+  if constexpr (OP != OP_RESAMPLE) {
+    // `windows`: unweighted, at most kWinTaps taps, rows a whole number of 16-byte chunks
+    if (windows && window_pool<T, MODE, OP>(in, map, out, idx, C, IH, IW, N, K, n, live,
+                                            blockIdx.y * cpt, blockIdx.z, cpt))
+      return;
+  }
+  if (!live) return;
   direct_gather<T, MODE, OP>(in, map, iw, out, idx, C, IH, IW, N, K, P, n, blockIdx.y * cpt,
                              blockIdx.z, cpt);
 }
@@ -632,12 +934,30 @@ int launch_gather(const void *in, const void *map, const void *iw, void *out, in
                   int64_t P, int interp, hipStream_t s) {
   const int64_t N = MH * MW;
   // (the same test as in direct_gather: unweighted pooling with at most 9 taps)
-  const int cpt = (OP != OP_RESAMPLE && P == 0 && K <= 9) ? kPoolCH : kCH;
+  const bool tap_registers = OP != OP_RESAMPLE && P == 0 && K <= 9;
+  int cpt = tap_registers ? kPoolCH : kCH;
+  if (tap_registers && B * C <= 0x7fffffffLL) {
+    // Images and channels are one run of planes to these kernels, and resolving a thread's
+    // taps costs as much as sampling some fifty planes: every thread takes as many planes
+    // as still leaves about eight waves for each of the 1024 SIMDs.
+    C *= B;
+    B = 1;
+    const int64_t waves = (int64_t)div_up(MW, Patch<OP>::kW) * div_up(MH, Patch<OP>::kH) *
+                          (kThreads / 64);
+    while (cpt < 1024 && cpt * 2 <= C && waves * div_up(C, cpt * 2) >= 8192) cpt *= 2;
+  }
   dim3 grid(div_up(MW, Patch<OP>::kW) * div_up(MH, Patch<OP>::kH), div_up(C, cpt), (unsigned)B);
+  // (the LDS-window path copies 16-byte chunks of source rows)
+  const int windows = tap_registers && N * 8 < (int64_t)kOobOffset &&
+                              IW % (16 / (int)sizeof(T)) == 0 &&
+                              (reinterpret_cast<uintptr_t>(in) & 15) == 0
+                          ? 1
+                          : 0;
   MCX_DISPATCH_MODE(interp, hipLaunchKernelGGL((gather_kernel<T, MODE, OP>), grid, dim3(kThreads),
                                                0, s, (const T *)in, (const T *)map,
                                                (const T *)iw, (T *)out, idx, (int)C, (int)IH,
-                                               (int)IW, (int)N, (int)MW, (int)K, (int)P, cpt));
+                                               (int)IW, (int)N, (int)MW, (int)K, (int)P, cpt,
+                                               windows));
   MCX_HIP_CHECK_LAUNCH();
   return 0;
 }
