@@ -912,7 +912,7 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
           }
           // The products of a unit issue back to back: at the default priority the other
           // waves of the SIMD slip their vector work in between and the matrix pipe idles.
-          __builtin_amdgcn_s_setprio(1);
+          if constexpr (!kBf16) __builtin_amdgcn_s_setprio(1);
           if constexpr (kBf16) {
 #pragma unroll
             for (int s = 0; s < 4; s++) {
@@ -933,7 +933,7 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
               acc[k][cb][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[4 * s4 + 3], bq.w, acc[k][cb][0], 0, 0, 0);
             }
           }
-          __builtin_amdgcn_s_setprio(0);
+          if constexpr (!kBf16) __builtin_amdgcn_s_setprio(0);
         }
       }
     }
