@@ -805,22 +805,202 @@ __global__ __launch_bounds__(kThreads) void sort_entries_kernel(
 template <int OP>
 constexpr int planes_per_thread() { return OP == UN_RESAMPLE ? 8 : 64; }
 
-// One thread per destination pixel and kTCH planes.  UN_MAX keeps a contribution
-// only where the recorded winner of that source element is this tap.
+// Smallest value of the wave (all 64 lanes active); see wave_max.
+__device__ inline uint32_t wave_min_u32(uint32_t v) {
+  constexpr int kId = -1;  // 0xffffffff
+  int x = (int)v;
+  auto mn = [](int a, int b) { return (int)min((uint32_t)a, (uint32_t)b); };
+  x = mn(x, __builtin_amdgcn_update_dpp(kId, x, 0x111, 0xf, 0xf, false));  // row_shr:1
+  x = mn(x, __builtin_amdgcn_update_dpp(kId, x, 0x112, 0xf, 0xf, false));  // row_shr:2
+  x = mn(x, __builtin_amdgcn_update_dpp(kId, x, 0x114, 0xf, 0xe, false));  // row_shr:4
+  x = mn(x, __builtin_amdgcn_update_dpp(kId, x, 0x118, 0xf, 0xc, false));  // row_shr:8
+  x = mn(x, __builtin_amdgcn_update_dpp(kId, x, 0x142, 0xa, 0xf, false));  // row_bcast:15
+  x = mn(x, __builtin_amdgcn_update_dpp(kId, x, 0x143, 0xc, 0xf, false));  // row_bcast:31
+  return (uint32_t)__builtin_amdgcn_readlane(x, 63);
+}
+
+// The unpoolings through LDS windows (fp32; see window_pool for why).  A wave's 64 destination
+// pixels read, through their lists, a few short runs of source elements - one per source row
+// under a pooling map.  The runs are found greedily on the list entries themselves, as
+// intervals of the linear source index (so neither the width of the source nor a seam
+// matters): the smallest entry not yet covered starts an interval of kUnIvLen elements, up to
+// kUnIntervals of them.  Per plane the intervals are copied to LDS with 16-byte loads and the
+// list entries read LDS; for max unpooling the recorded winners travel the same way, their low
+// words only (the caller guarantees that every tap code fits 32 bits, and the indices are
+// those mapped_max_pool wrote: a tap code or -1).  The sum keeps the order of the list.
+// Returns false (wave-uniform) when the wave's lists do not fit; nothing is written then.
+constexpr int kUnList = 16;      // entries per lane
+constexpr int kUnIntervals = 4;
+constexpr int kUnIvLen = 128;    // elements
+constexpr int kUnChunks = kUnIntervals * kUnIvLen / 4;  // 16-byte chunks of a window
+
 template <typename T, int OP>
-__global__ __launch_bounds__(kThreads) void transposed_gather_kernel(
+__device__ inline bool window_unpool(const T *__restrict__ src, const int64_t *__restrict__ idx,
+                                     T *__restrict__ dst, const uint32_t *__restrict__ e_src,
+                                     const T *__restrict__ e_wt, uint32_t start, uint32_t len,
+                                     bool live, int p, int64_t plane0, int nc, int nsrc, int ndst,
+                                     int K, int idx_scale) {
+  if constexpr (sizeof(T) != 4) {
+    return false;
+  } else {
+    constexpr int kDepth = OP == UN_MAX ? 2 : 4;  // planes whose loads are in flight
+    constexpr unsigned kZeroOff = kUnChunks * 16;
+    __shared__ uint4 win[kThreads / 64][2][kUnChunks + 1];
+    __shared__ uint4 iwin[OP == UN_MAX ? kThreads / 64 : 1][2][OP == UN_MAX ? kUnChunks + 1 : 1];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (__builtin_amdgcn_ballot_w64(len > (uint32_t)kUnList) != 0) return false;
+    uint32_t longest = (uint32_t)wave_max((int)len);
+    if (longest == 0) return false;
+
+    uint32_t loc[kUnList], want[kUnList];
+    T w[kUnList];
+#pragma unroll
+    for (int u = 0; u < kUnList; u++) {
+      const bool in = (uint32_t)u < len;
+      const uint32_t cd = e_src[in ? start + u : (len ? start : 0u)];
+      w[u] = in ? e_wt[start + u] : T(0);
+      loc[u] = in ? (OP == UN_MAX ? cd / (uint32_t)K : cd) : 0xffffffffu;
+      want[u] = in ? cd * (uint32_t)idx_scale : 0xffffffffu;  // (no recorded winner reads so)
+    }
+    // intervals: the smallest entry not yet covered starts the next one
+    uint32_t iv[kUnIntervals];
+    uint32_t bound = 0;
+    int nint = 0;
+#pragma unroll
+    for (int s2 = 0; s2 < kUnIntervals; s2++) {
+      uint32_t m = 0xffffffffu;
+#pragma unroll
+      for (int u = 0; u < kUnList; u++) m = min(m, loc[u] >= bound ? loc[u] : 0xffffffffu);
+      const uint32_t first = wave_min_u32(m);
+      iv[s2] = 0xffffffffu;
+      if (first != 0xffffffffu) {  // wave-uniform
+        iv[s2] = first & ~3u;
+        bound = iv[s2] + kUnIvLen;
+        nint = s2 + 1;
+      } else {
+        bound = 0xffffffffu;
+      }
+    }
+    {  // anything left beyond the last interval?
+      bool more = false;
+#pragma unroll
+      for (int u = 0; u < kUnList; u++) more = more || (loc[u] != 0xffffffffu && loc[u] >= bound);
+      if (bound != 0xffffffffu && __builtin_amdgcn_ballot_w64(more) != 0) return false;
+    }
+    // LDS byte offset of every entry (the zero chunk for the padding of a shorter list)
+    unsigned off[kUnList];
+#pragma unroll
+    for (int u = 0; u < kUnList; u++) {
+      unsigned sel = 0;
+      uint32_t base = iv[0];
+#pragma unroll
+      for (int s2 = 1; s2 < kUnIntervals; s2++) {
+        const bool ge = loc[u] >= iv[s2];  // (unused intervals start at 0xffffffff)
+        sel = ge ? (unsigned)s2 : sel;
+        base = ge ? iv[s2] : base;
+      }
+      off[u] = loc[u] == 0xffffffffu ? kZeroOff : (sel * kUnIvLen + (loc[u] - base)) * 4u;
+    }
+    // the chunks this lane copies per plane: first element, or none
+    unsigned goff[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const int q = lane + j * 64, s2 = q >> 5;
+      uint32_t first = iv[0];
+#pragma unroll
+      for (int t = 1; t < kUnIntervals; t++) first = s2 == t ? iv[t] : first;
+      const uint32_t elem = first + (uint32_t)(q & 31) * 4u;
+      goff[j] = (s2 < nint && elem < (uint32_t)nsrc) ? elem * 4u : kOobOffset;
+    }
+    if (lane < 2) {
+      win[wave][lane][kUnChunks] = make_uint4(0u, 0u, 0u, 0u);
+      if (OP == UN_MAX) iwin[wave][lane][kUnChunks] = make_uint4(0u, 0u, 0u, 0u);
+    }
+
+    const unsigned src_bytes = (unsigned)nsrc * 4u;
+    uint4 pre[kDepth][2];
+    uint4 ipre[OP == UN_MAX ? kDepth : 1][OP == UN_MAX ? 2 : 1][2];
+    auto fetch = [&](int c, int slot) {
+      const plane_buf_t pl = plane_buf(src + (plane0 + c) * nsrc, src_bytes);
+#pragma unroll
+      for (int j = 0; j < 2; j++)
+        pre[slot][j] = __builtin_bit_cast(
+            uint4, __builtin_amdgcn_raw_buffer_load_b128(pl, (int)goff[j], 0, 0));
+      if constexpr (OP == UN_MAX) {
+        // (an index plane of 8-byte elements: the same chunk is two 16-byte loads; offsets
+        // beyond 4 GiB are ruled out by the caller)
+        const plane_buf_t ipl = plane_buf(idx + (plane0 + c) * nsrc, (unsigned)nsrc * 8u);
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+          const unsigned o = goff[j] == kOobOffset ? kOobOffset : goff[j] * 2u;
+          ipre[slot][j][0] = __builtin_bit_cast(
+              uint4, __builtin_amdgcn_raw_buffer_load_b128(ipl, (int)o, 0, 0));
+          ipre[slot][j][1] = __builtin_bit_cast(
+              uint4, __builtin_amdgcn_raw_buffer_load_b128(ipl, (int)(o == kOobOffset ? o : o + 16u),
+                                                           0, 0));
+        }
+      }
+    };
+    auto stash = [&](int slot, int buf) {
+      win[wave][buf][lane] = pre[slot][0];
+      win[wave][buf][lane + 64] = pre[slot][1];
+      if constexpr (OP == UN_MAX) {
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+          iwin[wave][buf][lane + 64 * j] = make_uint4(ipre[slot][j][0].x, ipre[slot][j][0].z,
+                                                      ipre[slot][j][1].x, ipre[slot][j][1].z);
+      }
+      __builtin_amdgcn_wave_barrier();
+    };
+    auto compute = [&](int c, int buf) {
+      const char *wb = reinterpret_cast<const char *>(&win[wave][buf][0]);
+      const char *ib = reinterpret_cast<const char *>(&iwin[OP == UN_MAX ? wave : 0][buf][0]);
+      T v[kUnList];
+      uint32_t won[kUnList];
+#pragma unroll
+      for (int u = 0; u < kUnList; u++) {
+        v[u] = *reinterpret_cast<const T *>(wb + off[u]);
+        if (OP == UN_MAX) won[u] = *reinterpret_cast<const uint32_t *>(ib + off[u]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      T a = T(0);
+#pragma unroll
+      for (int u = 0; u < kUnList; u++) {
+        // (padding: weight zero times the zero chunk; max unpooling: its `want` matches nothing)
+        if (OP == UN_MAX)
+          a = won[u] == want[u] ? mcx_fma(w[u], v[u], a) : a;
+        else
+          a = mcx_fma(w[u], v[u], a);
+      }
+      const int cc = min(c, nc - 1);
+      buf_store(plane_buf(dst + (plane0 + cc) * ndst, (unsigned)ndst * 4u),
+                (live && c < nc) ? (unsigned)p * 4u : kOobOffset, OP == UN_AVG ? a / (T)K : a);
+      __builtin_amdgcn_wave_barrier();
+    };
+#pragma unroll
+    for (int u = 0; u < kDepth; u++) fetch(min(u, nc - 1), u);
+    stash(0, 0);
+    for (int cb = 0; cb < nc; cb += kDepth) {
+#pragma unroll
+      for (int u = 0; u < kDepth; u++) {
+        const int c = cb + u;
+        fetch(min(c + kDepth, nc - 1), u);
+        compute(c, u & 1);
+        stash((u + 1) % kDepth, (u + 1) & 1);
+      }
+    }
+    return true;
+  }
+}
+
+// Planes [plane0, plane0 + nc) of destination pixel p through its list [start, end).  UN_MAX
+// keeps a contribution only where the recorded winner of that source element is this tap.
+template <typename T, int OP>
+__device__ inline void transposed_gather_planes(
     const T *__restrict__ src, const int64_t *__restrict__ idx, T *__restrict__ dst,
-    const uint32_t *__restrict__ local, const uint32_t *__restrict__ bsum,
-    const uint32_t *__restrict__ e_src, const T *__restrict__ e_wt, int64_t planes, int nsrc,
-    int ndst, int K, int idx_scale, int groups) {
+    const uint32_t *__restrict__ e_src, const T *__restrict__ e_wt, uint32_t start, uint32_t end,
+    int p, int64_t plane0, int nc, int nsrc, int ndst, int K, int idx_scale) {
   constexpr int kTCH = planes_per_thread<OP>();
-  const int pg = blockIdx.x % groups;
-  const int p = (blockIdx.x / groups) * kThreads + threadIdx.x;
-  if (p >= ndst) return;
-  const int64_t plane0 = (int64_t)pg * kTCH;
-  const int nc = (int)min((int64_t)kTCH, planes - plane0);
-  const uint32_t start = local[p] + bsum[p / kScanBlock];
-  const uint32_t end = local[p + 1] + bsum[(p + 1) / kScanBlock];
   const T *s0 = src + plane0 * nsrc;
   const int64_t *i0 = OP == UN_MAX ? idx + plane0 * nsrc : nullptr;
   // Short lists (every lane of the wave has at most kListRegs entries: pooling maps): the
@@ -911,6 +1091,34 @@ __global__ __launch_bounds__(kThreads) void transposed_gather_kernel(
 #pragma unroll
   for (int c = 0; c < kTCH; c++)
     if (c < nc) d0[(int64_t)c * ndst] = OP == UN_AVG ? acc[c] / (T)K : acc[c];
+}
+
+// One workgroup: 256 destination pixels x `reps` groups of kTCH planes.
+template <typename T, int OP>
+__global__ __launch_bounds__(kThreads, OP == UN_AVG ? 4 : OP == UN_MAX ? 3 : 1) void transposed_gather_kernel(
+    const T *__restrict__ src, const int64_t *__restrict__ idx, T *__restrict__ dst,
+    const uint32_t *__restrict__ local, const uint32_t *__restrict__ bsum,
+    const uint32_t *__restrict__ e_src, const T *__restrict__ e_wt, int64_t planes, int nsrc,
+    int ndst, int K, int idx_scale, int groups, int reps, int windows) {
+  constexpr int kTCH = planes_per_thread<OP>();
+  const int pg = blockIdx.x % groups;
+  const int p = (blockIdx.x / groups) * kThreads + threadIdx.x;
+  const bool live = p < ndst;
+  const int pc = live ? p : 0;
+  const uint32_t start = local[pc] + bsum[pc / kScanBlock];
+  const uint32_t end = local[pc + 1] + bsum[(pc + 1) / kScanBlock];
+  const int64_t first_plane = (int64_t)pg * reps * kTCH;
+  const int np = (int)min((int64_t)reps * kTCH, planes - first_plane);
+  if constexpr (OP != UN_RESAMPLE) {
+    if (windows && window_unpool<T, OP>(src, idx, dst, e_src, e_wt, start, live ? end - start : 0u,
+                                        live, p, first_plane, np, nsrc, ndst, K, idx_scale))
+      return;
+  }
+  if (!live) return;
+  for (int done = 0; done < np; done += kTCH)
+    transposed_gather_planes<T, OP>(src, idx, dst, e_src, e_wt, start, end, p,
+                                    first_plane + done, min(kTCH, np - done), nsrc, ndst, K,
+                                    idx_scale);
 }
 
 bool bad_dims(std::initializer_list<int64_t> dims) {
@@ -1046,15 +1254,29 @@ int gather_transposed(const void *src, const int64_t *idx, void *dst, const void
   const TransposedLayout l = transposed_layout(ndst, samples, corners_of(interp), sizeof(T));
   if (!ws || !l.ok || ws_bytes < l.total || nsrc * K > 0xffffffffLL) return kNotApplicable;
   constexpr int kTCH = planes_per_thread<OP>();
-  const int64_t groups = (planes + kTCH - 1) / kTCH;
-  const int64_t blocks = groups * ((ndst + kThreads - 1) / kThreads);
+  // The LDS-window path copies 16-byte chunks of source planes (fp32; for max unpooling the
+  // recorded winners too, compared by their low words: every tap code must fit 32 bits).
+  const bool windows = OP != UN_RESAMPLE && sizeof(T) == 4 && nsrc % 4 == 0 &&
+                       (reinterpret_cast<uintptr_t>(src) & 15) == 0 &&
+                       nsrc * 8 < (int64_t)kOobOffset && ndst * 4 < (int64_t)kOobOffset &&
+                       (OP != UN_MAX || ((reinterpret_cast<uintptr_t>(idx) & 15) == 0 &&
+                                         nsrc * K * pm * 2 < 0xffffffffLL));
+  // A workgroup takes `reps` groups of kTCH planes (a wave's window set-up is spread over
+  // them) while about eight waves per SIMD remain.
+  int reps = 1;
+  const int64_t tiles = (ndst + kThreads - 1) / kThreads;
+  while (windows && reps < 4 && (int64_t)reps * 2 * kTCH <= planes &&
+         tiles * (kThreads / 64) * ((planes + reps * 2 * kTCH - 1) / (reps * 2 * kTCH)) >= 8192)
+    reps *= 2;
+  const int64_t groups = (planes + reps * kTCH - 1) / (reps * kTCH);
+  const int64_t blocks = groups * tiles;
   if (blocks > 0x7fffffffLL) return kNotApplicable;
   const char *base = (const char *)ws;
   hipLaunchKernelGGL((transposed_gather_kernel<T, OP>), dim3((unsigned)blocks), dim3(kThreads), 0,
                      s, (const T *)src, idx, (T *)dst, (const uint32_t *)(base + l.local),
                      (const uint32_t *)(base + l.bsum), (const uint32_t *)(base + l.e_src),
                      (const T *)(base + l.e_wt), planes, (int)nsrc, (int)ndst, (int)K,
-                     (int)(pm * 2), (int)groups);
+                     (int)(pm * 2), (int)groups, reps, windows ? 1 : 0);
   MCX_HIP_CHECK_LAUNCH();
   return 0;
 }

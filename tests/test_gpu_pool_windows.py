@@ -110,3 +110,71 @@ def test_maps_that_do_not_fit_windows(interp, device):
     _check(x, wide, 9, interp)
     xo = torch.randn(1, 2, 7, 202, generator=g)
     _check(xo, synthetic.latitude_map(7, 202, 1), 9, interp)
+
+
+# ------------------------------------------------------------------ unpoolings
+def _rel(a, b):
+    return float((a.cpu().double() - b.double()).abs().max() / b.double().abs().max().clamp_min(1e-30))
+
+
+def _check_unpool(gy, smap, H, W, K, interp, plan=False):
+    """avg and max unpooling of gy (the size of the map) onto H x W, against the oracle; the
+    argmax comes from the oracle's pooling of a random image."""
+    g = torch.Generator().manual_seed(99)
+    x = torch.randn(gy.shape[0], gy.shape[1], H, W, generator=g, dtype=gy.dtype)
+    _, mi = O.mapped_max_pool(x, smap, K, interp)
+    want_avg = O.mapped_avg_unpool(gy, smap, H, W, K, interp)
+    want_max = O.mapped_max_unpool(gy, mi, smap, H, W, K, interp)
+    kw = {}
+    if plan:
+        kw_avg = {"plan": _C.scatter_map_plan(smap.cuda(), None, H, W, interp, kernel=True)}
+        kw_max = {"plan": _C.scatter_map_plan(smap.cuda(), None, H, W, interp, for_max_unpool=True,
+                                              kernel=True)}
+    else:
+        kw_avg = kw_max = kw
+    got_avg = _C.mapped_avg_unpool(gy.cuda(), smap.cuda(), H, W, K, interp, **kw_avg)
+    got_max = _C.mapped_max_unpool(gy.cuda(), mi.cuda(), smap.cuda(), H, W, K, interp, **kw_max)
+    assert _rel(got_avg, want_avg) < 1e-5     # tolerance of the atomic-accumulated paths
+    assert _rel(got_max, want_max) < 1e-5
+
+
+@pytest.mark.parametrize("interp", [0, 1, 2])
+@pytest.mark.parametrize("shape", [(24, 192), (9, 200), (6, 64), (5, 1024), (7, 202)])
+def test_unpoolings_over_latitude_kernels(shape, interp, device):
+    """The unpoolings gather through per-pixel lists; where a wave's lists read a few short runs
+    of the pooled image they are staged in LDS.  Widths of one to sixteen waves, one whose
+    destination rows end inside a wave, one whose planes are not whole 16-byte chunks (no
+    windows); with and without a plan."""
+    H, W = shape
+    g = torch.Generator().manual_seed(H + W + interp)
+    gy = torch.randn(2, 70, H, W, generator=g)      # 140 planes: groups of 64, the last ragged
+    lmap = synthetic.latitude_map(H, W, 1)
+    _check_unpool(gy, lmap, H, W, 9, interp)
+    _check_unpool(gy[:, :3].contiguous(), lmap, H, W, 9, interp, plan=True)
+
+
+@pytest.mark.parametrize("interp", [0, 1])
+def test_unpoolings_whose_lists_do_not_fit_windows(interp, device):
+    """Lists longer than a lane keeps (row coordinates that are not integral: up to 36 entries),
+    scattered taps, a pooled image smaller than the unpooled one (stride 2), and a mixture."""
+    H, W = 12, 256
+    g = torch.Generator().manual_seed(31 + interp)
+    gy = torch.randn(1, 5, H, W, generator=g)
+    lat = synthetic.latitude_map(H, W, 1)
+    frac = lat.clone()
+    frac[..., 1] += 0.25
+    _check_unpool(gy, frac, H, W, 9, interp)
+    rnd = torch.stack([torch.rand(H, W, 9, generator=g) * (W + 4) - 2,
+                       torch.rand(H, W, 9, generator=g) * (H + 4) - 2], -1)
+    _check_unpool(gy, rnd, H, W, 9, interp)
+    mixed = lat.clone()
+    mixed[:, 100:, :, :] = rnd[:, 100:, :, :]
+    _check_unpool(gy, mixed, H, W, 9, interp)
+    OH, OW = H // 2, W // 2
+    i = np.arange(OH, dtype=np.float64)[:, None, None]
+    j = np.arange(OW, dtype=np.float64)[None, :, None]
+    offs = np.arange(-1, 2, dtype=np.float64)
+    dy, dx = [a.reshape(1, 1, -1) for a in np.meshgrid(offs, offs, indexing="ij")]
+    smap = torch.from_numpy(np.ascontiguousarray(
+        np.stack([2 * j + dx + 0 * i, 2 * i + dy + 0 * j], -1))).float()
+    _check_unpool(gy[:, :, :OH, :OW].contiguous(), smap, H, W, 9, interp)
