@@ -799,11 +799,12 @@ __global__ __launch_bounds__(kThreads) void sort_entries_kernel(
   }
 }
 
-// Planes per thread of the transposed gather.  The unpoolings read their list of about 15
-// entries once per thread: more planes per thread spread that over more work (8 -> 64 planes
-// took a third off the kernel); resampling lists are short and 8 planes measured best.
+// Planes per thread of the transposed gather's register paths.  The unpoolings read their list
+// of about 15 entries once per thread: more planes per thread spread that over more work (8 ->
+// 64 planes took a third off the kernel); resampling lists are short: 16 planes measured best
+// (0.70 ms against 0.75 with 8 and 0.74 with 32).
 template <int OP>
-constexpr int planes_per_thread() { return OP == UN_RESAMPLE ? 8 : 64; }
+constexpr int planes_per_thread() { return OP == UN_RESAMPLE ? 16 : 64; }
 
 // Smallest value of the wave (all 64 lanes active); see wave_max.
 __device__ inline uint32_t wave_min_u32(uint32_t v) {
@@ -1052,6 +1053,91 @@ __device__ inline void transposed_gather_planes(
       d0[(int64_t)c * ndst] = OP == UN_AVG ? a / (T)K : a;
     }
     return;
+  }
+  if constexpr (OP == UN_RESAMPLE) {
+    // Resampling lists are short (three entries on average under a cube map, up to fourteen)
+    // and differ in length from lane to lane.  Every lane walks the wave's longest list
+    // without a branch: an entry past the end of a lane's list loads out of range (a zero, no
+    // memory traffic) with weight zero, so that all loads of a step are in flight together.
+    // (With the loads behind the per-lane test every load was followed by a full wait: 0.93 ms
+    // at 4 x 64 planes of 512 x 1024, against 0.70 ms.  What remains is the texture path, busy
+    // 80 % of the time: the padded entries cost it as much as real ones, and the longest list
+    // of a wave is 4.9 entries where the average is 3.0.)
+    if ((int64_t)nsrc * (int64_t)sizeof(T) < (int64_t)kOobOffset) {
+      constexpr int kPair = 2;
+      plane_buf_t pl[kTCH];
+#pragma unroll
+      for (int c = 0; c < kTCH; c++)
+        pl[c] = plane_buf(s0 + (int64_t)min(c, nc - 1) * nsrc, (unsigned)nsrc * (unsigned)sizeof(T));
+      T acc[kTCH];
+#pragma unroll
+      for (int c = 0; c < kTCH; c++) acc[c] = T(0);
+      const uint32_t len = end - start;
+      // (lanes past the last pixel have left: the ballot-free reduction below needs all 64)
+      uint32_t longest = len;
+      for (int d = 32; d > 0; d >>= 1) longest = max(longest, (uint32_t)__shfl_xor((int)longest, d));
+      longest = __builtin_amdgcn_readfirstlane(longest);
+      constexpr int kRegs = 8, kStep = 4;
+      if (longest <= (uint32_t)kRegs) {
+        // the whole list first (one round trip), then the samples, four entries at a time
+        unsigned off[kRegs];
+        T w[kRegs];
+#pragma unroll
+        for (int u = 0; u < kRegs; u++) {
+          const bool in = (uint32_t)u < len;
+          const uint32_t ee = in ? start + u : 0u;
+          const uint32_t code = e_src[ee];
+          const T wt = e_wt[ee];
+          off[u] = in ? code * (unsigned)sizeof(T) : kOobOffset;
+          w[u] = in ? wt : T(0);
+        }
+#pragma unroll
+        for (int g = 0; g < kRegs / kStep; g++) {
+          if ((uint32_t)(g * kStep) < longest) {  // wave-uniform
+            T v[kStep][kTCH];
+#pragma unroll
+            for (int u = 0; u < kStep; u++)
+#pragma unroll
+              for (int c = 0; c < kTCH; c++) v[u][c] = buf_load(pl[c], off[g * kStep + u], T());
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < kStep; u++)
+#pragma unroll
+              for (int c = 0; c < kTCH; c++)
+                acc[c] = mcx_fma(w[g * kStep + u], v[u][c], acc[c]);
+          }
+        }
+      } else {
+        for (uint32_t t = 0; t < longest; t += kPair) {
+          unsigned off[kPair];
+          T w[kPair];
+#pragma unroll
+          for (int u = 0; u < kPair; u++) {
+            const bool in = t + u < len;
+            const uint32_t ee = in ? start + t + u : 0u;
+            const uint32_t code = e_src[ee];
+            const T wt = e_wt[ee];
+            off[u] = in ? code * (unsigned)sizeof(T) : kOobOffset;
+            w[u] = in ? wt : T(0);
+          }
+          T v[kPair][kTCH];
+#pragma unroll
+          for (int u = 0; u < kPair; u++)
+#pragma unroll
+            for (int c = 0; c < kTCH; c++) v[u][c] = buf_load(pl[c], off[u], T());
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int u = 0; u < kPair; u++)
+#pragma unroll
+            for (int c = 0; c < kTCH; c++) acc[c] = mcx_fma(w[u], v[u][c], acc[c]);
+        }
+      }
+      T *d0 = dst + plane0 * ndst + p;
+#pragma unroll
+      for (int c = 0; c < kTCH; c++)
+        if (c < nc) d0[(int64_t)c * ndst] = acc[c];
+      return;
+    }
   }
   T acc[kTCH];
 #pragma unroll
