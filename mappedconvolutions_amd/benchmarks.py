@@ -24,10 +24,23 @@ FP32_VALU_TFLOPS = 157.3  # vector fp32 FMA peak (packed); KNN is bound by it
 
 
 def _time(fn, iters=10, warmup=2):
+    """ms per call: `warmup` calls, untimed loops of `iters` for at least 80 ms (after a change
+    of workload the GPU runs at a lower clock for some tens of milliseconds: up to 10 % slower),
+    then the timed loop."""
+    import time
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    while True:
+        start.record()
+        for _ in range(iters):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        if time.perf_counter() - t0 >= 0.08:
+            break
     start.record()
     for _ in range(iters):
         fn()
@@ -205,8 +218,6 @@ def plans(dev):
     smap = synthetic.latitude_map(H, W, 1).to(dev)
     cplan = _C.conv_map_plan(smap, None, H, W, 1)
     flop = 2.0 * B * H * W * C * C * K
-    # (the first timed loop after a change of workload runs at a lower clock: one untimed)
-    _time(lambda: _C.mapped_conv_forward(x, smap, w, b, K, 1), iters=20)
     _line("planned headline conv forward fp32",
           _time(lambda: _C.mapped_conv_forward(x, smap, w, b, K, 1, plan=cplan)), flops=flop)
     _line("unplanned headline conv forward fp32",
