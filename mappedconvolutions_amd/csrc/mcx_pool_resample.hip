@@ -1195,8 +1195,11 @@ __global__ __launch_bounds__(kThreads, OP == UN_AVG ? 4 : OP == UN_MAX ? 3 : 1) 
     const uint32_t *__restrict__ e_src, const T *__restrict__ e_wt, int64_t planes, int nsrc,
     int ndst, int K, int idx_scale, int groups, int reps, int windows) {
   constexpr int kTCH = planes_per_thread<OP>();
-  const int pg = blockIdx.x % groups;
-  const int p = (blockIdx.x / groups) * kThreads + threadIdx.x;
+  // (the unpoolings: every XCD takes one contiguous run of the destination, so that the source
+  // rows neighbouring destination rows share are read into one L2 only)
+  const int wg = OP == UN_RESAMPLE ? (int)blockIdx.x : xcd_contiguous(blockIdx.x, gridDim.x);
+  const int pg = wg % groups;
+  const int p = (wg / groups) * kThreads + threadIdx.x;
   const bool live = p < ndst;
   const int pc = live ? p : 0;
   const uint32_t start = local[pc] + bsum[pc / kScanBlock];
