@@ -178,3 +178,30 @@ def test_unpoolings_whose_lists_do_not_fit_windows(interp, device):
     smap = torch.from_numpy(np.ascontiguousarray(
         np.stack([2 * j + dx + 0 * i, 2 * i + dy + 0 * j], -1))).float()
     _check_unpool(gy[:, :, :OH, :OW].contiguous(), smap, H, W, 9, interp)
+
+
+@pytest.mark.parametrize("interp", [0, 1])
+def test_weighted_unpoolings_through_windows(interp, device):
+    """Weighted taps (two points per tap, the second one column to the right): lists of up to
+    twelve (nearest) entries go through the windows, longer ones (bilinear) through the register
+    path; the recorded winners of the weighted max pooling count points, not taps."""
+    H, W, K, P = 10, 192, 3, 2
+    g = torch.Generator().manual_seed(41 + interp)
+    i = np.arange(H, dtype=np.float64)[:, None, None, None]
+    j = np.arange(W, dtype=np.float64)[None, :, None, None]
+    dx = np.array([-1.0, 0.0, 1.0]).reshape(1, 1, K, 1)
+    pt = np.array([0.0, 1.0]).reshape(1, 1, 1, P)
+    x = np.mod(j + dx * 1.5 + pt + 0 * i, W)
+    y = i + 0 * j + 0 * dx + 0 * pt
+    smap = torch.from_numpy(np.ascontiguousarray(np.stack([x, y], -1))).float()
+    wts = torch.rand(H, W, K, P, generator=g) + 0.1
+    gy = torch.randn(2, 6, H, W, generator=g)
+    src = torch.randn(2, 6, H, W, generator=g)
+    _, mi = O.weighted_mapped_max_pool(src, smap, wts, K, interp)
+    want_avg = O.weighted_mapped_avg_unpool(gy, smap, wts, H, W, K, interp)
+    want_max = O.weighted_mapped_max_unpool(gy, mi, smap, wts, H, W, K, interp)
+    got_avg = _C.weighted_mapped_avg_unpool(gy.cuda(), smap.cuda(), wts.cuda(), H, W, K, interp)
+    got_max = _C.weighted_mapped_max_unpool(gy.cuda(), mi.cuda(), smap.cuda(), wts.cuda(), H, W,
+                                            K, interp)
+    assert _rel(got_avg, want_avg) < 1e-5
+    assert _rel(got_max, want_max) < 1e-5
