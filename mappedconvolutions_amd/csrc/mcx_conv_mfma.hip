@@ -1055,23 +1055,6 @@ constexpr int kScPx = 32;        // pixels per wave
 constexpr int kScEntries = 40;   // cached (tap, point, corner) entries per pixel
 constexpr int kScThreads = 64;
 
-// Repack W[s][d][k] -> Wq[k][dc][s][16]: per (tap, 16-channel block) a contiguous
-// [Spad x 16] slice; s padded to 64, d padded to 16, zeros in the padding.
-template <typename TD>
-__global__ void pack_scatter_weights_kernel(const TD *__restrict__ w, float *__restrict__ wq,
-                                            int S, int D, int K, int Spad, int dchunks) {
-  const int64_t total = (int64_t)K * dchunks * Spad * kScDC;
-  for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total;
-       e += (int64_t)gridDim.x * blockDim.x) {
-    const int dl = (int)(e % kScDC);
-    const int s = (int)((e / kScDC) % Spad);
-    const int dc = (int)((e / ((int64_t)kScDC * Spad)) % dchunks);
-    const int k = (int)(e / ((int64_t)kScDC * Spad * dchunks));
-    const int d = dc * kScDC + dl;
-    wq[e] = (s < S && d < D) ? to_f32(w[((int64_t)s * D + d) * K + k]) : 0.f;
-  }
-}
-
 __device__ inline int wave_min(int v) {
 #pragma unroll
   for (int m = 32; m > 0; m >>= 1) v = min(v, __shfl_xor(v, m, 64));
@@ -1891,15 +1874,30 @@ __global__ void after_transposed_map_kernel(const int *__restrict__ cnt, int64_t
     img[i] = 0.f;
 }
 
-// dst[b,c,:] = bias[c] (or 0); runs only when the gate agrees (see above).
+// What the scatter form needs before it runs, in one launch (a launch costs about 4 us even
+// when every workgroup leaves at once, as here on maps the gather form handles):
+// dst[b,c,:] = bias[c] (or 0), and the weights repacked W[s][d][k] -> Wq[k][dc][s][16]: per
+// (tap, 16-channel block) a contiguous [Spad x 16] slice; s padded to 64, d padded to 16, zeros
+// in the padding.  Runs only when the gate agrees (see above).
 template <typename TD>
-__global__ void init_planes_kernel(float *__restrict__ dst, const TD *__restrict__ bias, int C,
-                                   int64_t plane, int64_t total, const int *__restrict__ gate,
-                                   int run_if_zero) {
+__global__ void init_scatter_kernel(float *__restrict__ dst, const TD *__restrict__ bias, int C,
+                                    int64_t plane, int64_t total, const TD *__restrict__ w,
+                                    float *__restrict__ wq, int S, int K, int Spad, int dchunks,
+                                    const int *__restrict__ gate, int run_if_zero) {
   if (gate && ((*gate == 0) != (run_if_zero != 0))) return;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
        i += (int64_t)gridDim.x * blockDim.x)
     dst[i] = bias ? to_f32(bias[(i / plane) % C]) : 0.f;
+  const int64_t packed = (int64_t)K * dchunks * Spad * kScDC;
+  for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < packed;
+       e += (int64_t)gridDim.x * blockDim.x) {
+    const int dl = (int)(e % kScDC);
+    const int sl = (int)((e / kScDC) % Spad);
+    const int dc = (int)((e / ((int64_t)kScDC * Spad)) % dchunks);
+    const int k = (int)(e / ((int64_t)kScDC * Spad * dchunks));
+    const int d = dc * kScDC + dl;
+    wq[e] = (sl < S && d < C) ? to_f32(w[((int64_t)sl * C + d) * K + k]) : 0.f;
+  }
 }
 
 template <typename TD>
@@ -2164,13 +2162,8 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
   const int64_t total_dst = B * D * DH * DW;
   float *acc = sizeof(TD) == 4 ? (float *)dst : (float *)(base + sc.acc32);
   const unsigned fill_blocks = (unsigned)std::min<int64_t>((total_dst + 1023) / 1024, 8192);
-  hipLaunchKernelGGL(init_planes_kernel<TD>, dim3(fill_blocks), dim3(256), 0, s, acc, bias, (int)D,
-                     DH * DW, total_dst, gate, 0);
-  MCX_HIP_CHECK_LAUNCH();
-  const int64_t packed = (int64_t)K * dchunks * Spad * kScDC;
-  hipLaunchKernelGGL(pack_scatter_weights_kernel<TD>,
-                     dim3((unsigned)std::min<int64_t>((packed + 255) / 256, 4096)), dim3(256), 0, s,
-                     w, wq, (int)S, (int)D, (int)K, Spad, dchunks);
+  hipLaunchKernelGGL(init_scatter_kernel<TD>, dim3(fill_blocks), dim3(256), 0, s, acc, bias, (int)D,
+                     DH * DW, total_dst, w, wq, (int)S, (int)K, Spad, dchunks, gate, 0);
   MCX_HIP_CHECK_LAUNCH();
   const int tiles_x = (int)((MW + kScPx - 1) / kScPx);
   const int64_t tiles_per_img = (int64_t)tiles_x * MH;
