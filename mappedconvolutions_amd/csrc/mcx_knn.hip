@@ -1,4 +1,6 @@
-// Brute-force k nearest neighbours with a streaming top-k.  The reference
+// k nearest neighbours: a walk over all reference points with a streaming top-k, and (second
+// half of the file) a search over a uniform grid for points of one to three dimensions that
+// gives the same result bit for bit.  The reference
 // (include/util/cuda/knn.cuh:43-275) materialises the R x Q matrix of squared
 // distances and insertion-sorts each column with one thread; here one thread owns
 // one query, walks the reference points once and keeps its k best in registers,

@@ -3,7 +3,10 @@
 // plain and weighted.  One thread owns one map location and a chunk of CH
 // channels: the tap (offsets + weights) is resolved once and applied to each of
 // the thread's channel planes, so map decoding is amortised and neighbouring lanes
-// read neighbouring pixels.
+// read neighbouring pixels.  Pooling and unpooling have a second form, chosen per
+// wave on the device: where the taps (or the transposed lists) of a wave's 64
+// locations read a few short runs of the source, those runs are staged in LDS with
+// 16-byte loads and the taps read LDS (window_pool, window_unpool).
 #include <type_traits>
 
 #include "mcx_device.h"
