@@ -171,7 +171,7 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
     int O, int Opad, int Gpad, int SH, int SW, int OH, int OW, int K, int weighted, int wrap,
     int tiles_x, int tiles_per_img, int tw_shift, const int *__restrict__ gate, int run_if_zero,
     const float *__restrict__ addend, const int *__restrict__ pair_mask, int run_if_leading,
-    int packed_map, int accumulate, int cl_blocked) {
+    int packed_map, int accumulate, int cl_blocked, const int *__restrict__ row_mask) {
   constexpr int NE = NP * NCORN;         // (offset, weight) pairs per pixel and tap
   static_assert(NA >= 1 && NA <= NE, "NA counts leading pairs");
   constexpr bool kMasked = NA == NE;
@@ -189,7 +189,6 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
   // accumulated.
   __shared__ unsigned TapMask[TG][2][2];
   if (gate && ((*gate == 0) != (run_if_zero != 0))) return;  // device-side path selection
-  if (pair_mask && (((unsigned)*pair_mask < (1u << 2)) != (run_if_leading != 0))) return;
   // a pass that adds onto y (the second level of a transposed map) has nothing to do when
   // no pair of its map is in use
   if (accumulate && pair_mask && *pair_mask == 0) return;
@@ -201,6 +200,19 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
   const int tile_y = t_in / tiles_x, tile_x = t_in - tile_y * tiles_x;
   const int tw_mask = (1 << tw_shift) - 1;
   const int th = kTilePx >> tw_shift;
+  if (pair_mask) {
+    // The two-pair form serves the whole map when no tap anywhere uses a later pair; with
+    // `row_mask` (one word per row of output pixels, nonzero iff a tap of the row does) it
+    // serves every tile whose rows are clear, and the general form the others: a few border
+    // rows that hold more must not put the whole image on the slower form.
+    bool leading = (unsigned)*pair_mask < (1u << 2);
+    if (!leading && row_mask) {
+      int any = 0;
+      for (int r = tile_y * th; r < min(tile_y * th + th, OH); r++) any |= row_mask[r];
+      leading = any == 0;
+    }
+    if (leading != (run_if_leading != 0)) return;
+  }
   const int o0 = blockIdx.y * (kOT * OG);
   const int N = OH * OW;
   const int64_t plane = (int64_t)SH * SW;
@@ -1445,7 +1457,7 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
                           int interp, const int *gate, int run_if_zero, hipStream_t s,
                           const float *addend = nullptr, bool staged = false,
                           const int *pair_mask = nullptr, bool packed_map = false,
-                          bool accumulate = false) {
+                          bool accumulate = false, const int *row_mask = nullptr) {
   const int Opad = (int)round_up(O, kOT), Gpad = (int)round_up(G, kGC);
   const bool blocked = stage != nullptr && use_channel_blocks(SH, interp, sizeof(TD)) &&
                        SH * SW * 8 * (int64_t)sizeof(TD) <= 0xffffffffLL;
@@ -1477,7 +1489,7 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
                      dim3(kThreads), 0, s, src, map, iw, wp, bias, y, (int)G, (int)O, Opad,      \
                      Gpad, (int)SH, (int)SW, (int)OH, (int)OW, (int)K, m.weighted, m.wrap,       \
                      t.tiles_x, t.tiles_per_img, t.tw_shift, gate, run_if_zero, addend, MASK,    \
-                     LEAD, packed_map ? 1 : 0, accumulate ? 1 : 0, blocked ? 1 : 0)
+                     LEAD, packed_map ? 1 : 0, accumulate ? 1 : 0, blocked ? 1 : 0, row_mask)
 #define MCX_LAUNCH_CL(NCORN, NP, OG, CL)                                      \
   if constexpr (NCORN * NP == 4) {                                            \
     if (pair_mask) {                                                          \
@@ -1843,21 +1855,28 @@ __global__ __launch_bounds__(64) void overflow_scatter_kernel(
 }
 
 // Two jobs that follow the building of a transposed map, in one launch.  (1) mask[0] >= 4
-// iff some cell holds more than two entries (bits [0, min(cnt, kTransSlots))); with a
-// second level, mask[1] holds the bits of the second-level slots in use (0: none).  (2) Clear
+// iff some cell holds more than two entries (bits [0, min(cnt, kTransSlots))), and row_mask
+// says in which rows of the destination; with a second level, mask[1] holds the bits of the
+// second-level slots in use (0: none).  (2) Clear
 // the fp32 image the overflow list is accumulated into, only when the list is in use and
 // not empty.
 __global__ void after_transposed_map_kernel(const int *__restrict__ cnt, int64_t cells,
                                             int *__restrict__ mask, int two_level,
                                             float *__restrict__ img, int64_t total,
-                                            const int *__restrict__ overflow) {
+                                            const int *__restrict__ overflow,
+                                            int *__restrict__ row_mask, int row_cells) {
   __shared__ unsigned block_mask;
   if (threadIdx.x == 0) block_mask = 0;
   __syncthreads();
   unsigned m = 0;
   for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < cells;
-       e += (int64_t)gridDim.x * blockDim.x)
-    m |= (1u << min(cnt[e], 2 * kTransSlots)) - 1u;
+       e += (int64_t)gridDim.x * blockDim.x) {
+    const int c = cnt[e];
+    m |= (1u << min(c, 2 * kTransSlots)) - 1u;
+    // row_mask[y] != 0 iff a cell of destination row y holds more than two entries (cells are
+    // [pixel][tap], row_cells of them per row; every writer stores the same value)
+    if (c > 2) row_mask[e / row_cells] = 1;
+  }
   for (int d = 32; d > 0; d >>= 1) m |= __shfl_xor(m, d);
   if ((threadIdx.x & 63) == 0 && m) atomicOr(&block_mask, m);
   __syncthreads();
@@ -1981,7 +2000,7 @@ ScatterScratch scatter_scratch(int64_t B, int64_t S, int64_t D, int64_t K, int64
     sc.wpt = off;
     off += align256((size_t)(K * round_up(S, kGC) * round_up(D, kOT)) * 4);
     sc.cnt = off;  // counters, the overflow flag and list length; cleared with tmap
-    off += align256((size_t)(cells + 8) * 4);
+    off += align256((size_t)(cells + 8 + DH) * 4);  // (and a word per destination row)
     sc.tmap = off;  // [tap][slot][pixel] (source pixel index as bits, weight)
     off += align256((size_t)cells * kTransSlots * 2 * 4);
     sc.tmap2 = off;
@@ -2032,7 +2051,7 @@ int build_transposed_map(const ScatterScratch &sc, const float *map, const float
 
 // ---- plan: the transposed map of one sample map, kept by the caller across calls ----------
 // Layout: the scratch region [cnt, stage) of mfma_product_scatter (counters, eight flag words,
-// slots, second-level slots, overflow list); flag word 4 holds the pair mask of the map itself,
+// a word per destination row, slots, second-level slots, overflow list); flag word 4 holds the pair mask of the map itself,
 // for the weight gradient.  Depends on the map, its interpolation and the two image sizes only.
 // (followed, for maps of at most four points per tap, by the gather part: MH * MW * K cells of
 // four resolved entries)
@@ -2065,7 +2084,7 @@ int mfma_scatter_plan_build(const float *map, const float *iw, void *plan, int64
   hipLaunchKernelGGL(after_transposed_map_kernel,
                      dim3((unsigned)std::min<int64_t>((cells + 255) / 256, 4096)), dim3(256), 0, s,
                      cnt, cells, flag + 2, sc.two_level ? 1 : 0, (float *)nullptr, (int64_t)0,
-                     flag);
+                     flag, flag + 8, (int)(K * DW));
   MCX_HIP_CHECK_LAUNCH();
   if (m.np * (m.mode == kInterpNearest ? 1 : 4) == 4)
     if (int rc = launch_pair_mask(map, iw, flag + 4, m, DH, DW, MH * MW * K, s, true)) return rc;
@@ -2133,7 +2152,7 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
                        dim3((unsigned)std::min<int64_t>(
                            std::max((total_img + 1023) / 1024, (cells + 255) / 256), 4096)),
                        dim3(256), 0, s, cnt, plan ? (int64_t)0 : cells, flag + 2,
-                       sc.two_level ? 1 : 0, img, total_img, flag);
+                       sc.two_level ? 1 : 0, img, total_img, flag, flag + 8, (int)(K * DW));
     MCX_HIP_CHECK_LAUNCH();
     if (cl) {  // the overflow pass reads the channel-last copy before the gather would make it
       dim3 tg((unsigned)((MH * MW + 63) / 64), (unsigned)((Spad16 + 63) / 64), (unsigned)B);
@@ -2148,7 +2167,8 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
     MCX_HIP_CHECK_LAUNCH();
     if (int rc = launch_gather_product<TD>(src, (const float *)tmap, nullptr, wpt, bias, dst,
                                            stage, B, S, D, MH, MW, DH, DW, K, kTransSlots,
-                                           kInterpNearest, gate, 1, s, img, cl, flag + 2, true))
+                                           kInterpNearest, gate, 1, s, img, cl, flag + 2, true,
+                                           false, flag + 8))
       return rc;
     if (sc.two_level)  // entries five to eight of every cell, added onto dst
       if (int rc = launch_gather_product<TD>(src, (const float *)tmap2, nullptr, wpt,

@@ -152,6 +152,10 @@ struct Tap<T, kInterpNearest> {
   __device__ inline void load_rows(plane_buf_t plane, T *d, bool, bool, bool) const {
     load(plane, d);
   }
+  template <bool PAIRS>
+  __device__ inline void load_flat(plane_buf_t plane, T *d) const {
+    load(plane, d);
+  }
   __device__ inline void scatter(T *plane, T v) const {
     if (off >= 0) atomic_add(plane + off, v);
   }
@@ -244,6 +248,23 @@ struct Tap {
           d[i] = buf_load(plane, off[i] < 0 ? kOobOffset : (unsigned)off[i] * (unsigned)sizeof(T),
                           T());
       }
+    }
+  }
+  // load_rows() without its switches: both rows, as two two-element loads (PAIRS; every
+  // lane's tap must be pairable) or four single ones.  No branch, so a caller can keep the
+  // loads of several planes in flight and the compiler can count them.
+  template <bool PAIRS>
+  __device__ inline void load_flat(plane_buf_t plane, T *d) const {
+    if constexpr (PAIRS) {
+#pragma unroll
+      for (int r = 0; r < 2; r++) {
+        const auto v = buf_load_pair(
+            plane, off[2 * r] < 0 ? kOobOffset : (unsigned)off[2 * r] * (unsigned)sizeof(T), T());
+        d[2 * r] = v.x;
+        d[2 * r + 1] = v.y;
+      }
+    } else {
+      load(plane, d);
     }
   }
   __device__ inline T gather(plane_buf_t plane) const {

@@ -205,6 +205,34 @@ def test_conv_and_tconv_fp32_many_points_or_one_tap(k, p, interp, device):
         assert rel_err(a, r) < 1e-5, "transposed " + nm
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("with_plan", [False, True])
+def test_input_gradient_with_border_rows_beyond_two_entries(with_plan, dtype, device):
+    """5x5 latitude map: the clamped rows at the top and the bottom put three and more
+    contributions into cells of the first and the last input row, every other row holds at most
+    two per cell.  The input gradient then runs its two-entry form on the tiles whose rows are
+    clear and the general form on the others, several tiles per row and per image here."""
+    B, Ci, Co, H, W, K = 2, 24, 40, 24, 288, 25
+    g = torch.Generator().manual_seed(77)
+    cast = lambda t: t.to(dtype)
+    x, gy = cast(torch.randn(B, Ci, H, W, generator=g)), cast(torch.randn(B, Co, H, W, generator=g))
+    w = cast(torch.randn(Co, Ci, K, generator=g) / (Ci * K) ** 0.5)
+    b = cast(torch.randn(Co, generator=g))
+    smap = synthetic.latitude_map(H, W, 2)
+    # the premise: cells of the border rows receive more than two contributions, no others do
+    cnt = torch.bincount(helpers.map_contributions(smap, None, H, W, 1), minlength=H * W * K)
+    rows = (cnt.view(H, W * K) > 2).any(1)
+    assert rows[0] and rows[-1] and not rows[2:-2].any()
+    g_o = O.mapped_conv_backward(gy.float(), smap, x.float(), w.float(), b.float(), K, 1)
+    xd, sd, wd_, bd, gyd = dev(x, smap, w, b, gy)
+    plan = _C.conv_map_plan(sd, None, H, W, 1, dtype) if with_plan else None
+    for _ in range(2):
+        gr = _C.mapped_conv_backward(gyd, sd, xd, wd_, bd, K, 1, plan=plan)
+        for a, r, nm in zip(gr, g_o, ("grad_input", "grad_weight", "grad_bias")):
+            assert rel_err(a.float().cpu(), r) < TOL[dtype], nm
+        assert_close_elementwise(gr[0].float().cpu(), g_o[0], TOL[dtype])
+
+
 def test_bf16_with_more_than_four_points_is_rejected(device):
     """bf16 storage exists on the matrix-core kernels only, which take at most four points."""
     g = torch.Generator().manual_seed(5)
