@@ -42,7 +42,7 @@ int mfma_gather_product(const TD *src, const float *map, const float *iw, const 
                         int64_t SH, int64_t SW, int64_t OH, int64_t OW, int64_t K, int64_t P,
                         int interp, hipStream_t s, const void *plan = nullptr);
 size_t mfma_weight_grad_bytes(int64_t B, int64_t A, int64_t G, int64_t MH, int64_t MW, int64_t K,
-                              int64_t GH, int64_t GW);
+                              int64_t GH, int64_t GW, size_t elem);
 template <typename TD>
 int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const float *iw, TD *gw,
                      void *scratch, int64_t B, int64_t A, int64_t G, int64_t GH, int64_t GW,

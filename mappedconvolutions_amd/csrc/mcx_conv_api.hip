@@ -103,7 +103,7 @@ size_t gather_product_ws(int dtype, int64_t G, int64_t O, int64_t K, int64_t P, 
 }
 size_t weight_grad_ws(int dtype, int64_t B, int64_t A, int64_t G, int64_t MH, int64_t MW,
                       int64_t K, int64_t P, int64_t GH, int64_t GW) {
-  return use_mfma(dtype, P) ? mfma_weight_grad_bytes(B, A, G, MH, MW, K, GH, GW) : 0;
+  return use_mfma(dtype, P) ? mfma_weight_grad_bytes(B, A, G, MH, MW, K, GH, GW, elem_size(dtype)) : 0;
 }
 size_t product_scatter_ws(int dtype, int64_t B, int64_t S, int64_t D, int64_t K, int64_t P,
                           int64_t DH, int64_t DW, int64_t MH, int64_t MW) {
@@ -234,7 +234,7 @@ int weight_grad<float>(bool mfma, const void *plain, const void *gath, const voi
     return generic_weight_grad<float>((const float *)plain, (const float *)gath,
                                       (const float *)map, (const float *)iw, (float *)gw, B, A, G,
                                       GH, GW, MH * MW, K, P, interp, s);
-  if (!ws || ws_bytes < mfma_weight_grad_bytes(B, A, G, MH, MW, K, GH, GW))
+  if (!ws || ws_bytes < mfma_weight_grad_bytes(B, A, G, MH, MW, K, GH, GW, 4))
     return MCX_E_WORKSPACE;
   return mfma_weight_grad<float>((const float *)plain, (const float *)gath, (const float *)map,
                                  (const float *)iw, (float *)gw, ws, B, A, G, GH, GW, MH, MW, K, P,
@@ -284,7 +284,7 @@ int weight_grad<bf16_t>(bool mfma, const void *plain, const void *gath, const vo
                         int64_t P, int interp, hipStream_t s, void *plain_sum,
                         const void *plan) {
   if (!mfma) return MCX_E_DTYPE;
-  if (!ws || ws_bytes < mfma_weight_grad_bytes(B, A, G, MH, MW, K, GH, GW))
+  if (!ws || ws_bytes < mfma_weight_grad_bytes(B, A, G, MH, MW, K, GH, GW, 2))
     return MCX_E_WORKSPACE;
   return mfma_weight_grad<bf16_t>((const bf16_t *)plain, (const bf16_t *)gath, (const float *)map,
                                   (const float *)iw, (bf16_t *)gw, ws, B, A, G, GH, GW, MH, MW, K,

@@ -124,7 +124,10 @@ __global__ __launch_bounds__(256) void to_channel_last_kernel(const TD *__restri
 template <typename TD>
 __global__ __launch_bounds__(256) void to_channel_blocks_kernel(const TD *__restrict__ x,
                                                                 TD *__restrict__ xt, int G,
-                                                                int64_t plane) {
+                                                                int64_t plane,
+                                                                const int *__restrict__ pair_mask) {
+  // (with a pair mask: the copy is for a kernel that only runs while the mask is below 4)
+  if (pair_mask && (unsigned)*pair_mask >= (1u << 2)) return;
   const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int g8 = blockIdx.y, b = blockIdx.z;
   if (n >= plane) return;
@@ -1035,6 +1038,312 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(
 }
 
 // ---------------------------------------------------------------------------------
+// Weight gradient, bf16 storage, bilinear taps whose two lower corners weigh nothing anywhere
+// in the map (integral row coordinates), gathered operand in blocks of 8 channels per pixel
+// ([B][Gpad/8][GH*GW][8], to_channel_blocks_kernel).  With bf16 MFMA the products are short
+// and the kernel lives or dies by its gather, so this form is built around it:
+//   * a thread gathers two neighbouring pixels x 8 channels of a unit (one tap, 32 gathered
+//     channels): four 16-byte loads instead of 32 two-byte ones (the texture path resolves
+//     four lanes per clock whatever the width), and a channel's two pixels leave as one
+//     32-bit LDS store, consecutive lanes to consecutive banks;
+//   * the loads of kRgDepth units are in flight, across tile boundaries: the taps of the next
+//     tile are resolved (into the other half of a double-buffered tap cache) and the next
+//     plain tile is fetched into registers while this tile's units are multiplied, so that in
+//     the steady state no wave waits for memory at a tile's start;
+//   * every load and store is unconditional (past the range's last tile the last one is
+//     fetched again, padded taps weigh zero), so the compiler's waits count exactly;
+//   * five taps per pass keep the accumulators at 80 registers, which leaves room for the
+//     rings at two workgroups per CU.
+// Partial sums leave in the layout of weight_grad_mfma_kernel.
+constexpr int kRgKT = 5;      // taps per pass
+constexpr int kRgG = 32;      // gathered channels per workgroup
+constexpr int kRgA = 128;     // plain channels per workgroup
+constexpr int kRgDepth = 2;   // units whose gathers are in flight
+constexpr int kRgLd = kTilePx + 8;  // bf16 elements per LDS row
+
+inline int ring_weight_grad_ranges(int64_t total_tiles, int64_t A, int64_t G, int64_t K) {
+  const int64_t per_range = ((G + kRgG - 1) / kRgG) * ((A + kRgA - 1) / kRgA) *
+                            ((K + kRgKT - 1) / kRgKT);
+  int64_t r = std::max<int64_t>(8, (1024 / per_range) / 8 * 8);  // about four workgroups per CU
+  r = std::min<int64_t>(r, std::max<int64_t>(total_tiles / 8 * 8, 8));
+  return (int)r;
+}
+
+__global__ __launch_bounds__(kThreads, 2) void weight_grad_bf16_ring_kernel(
+    const bf16_t *__restrict__ plain, const bf16_t *__restrict__ gath,
+    const float *__restrict__ map, float *__restrict__ part, int A, int G, int Gpad, int GH,
+    int GW, int MH, int MW, int K, int wrap, int tiles_x, int tiles_per_img, int tw_shift,
+    int total_tiles, int ranges, int cgroups, int passes, float *__restrict__ plain_sum_part,
+    const int *__restrict__ pair_mask) {
+  if (pair_mask && (unsigned)*pair_mask >= (1u << 2)) return;  // the general form runs instead
+  constexpr int MB = kRgA / 64, NB = kRgG / 16;
+  __shared__ __attribute__((aligned(16))) uint16_t PtB[kRgA][kRgLd];
+  __shared__ __attribute__((aligned(16))) uint16_t SB[2][kRgG][kRgLd];
+  __shared__ __attribute__((aligned(16))) unsigned TapOff[2][kRgKT][kTilePx][2];
+  __shared__ __attribute__((aligned(16))) float TapWt[2][kRgKT][kTilePx][2];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l15 = lane & 15, lq = lane >> 4;
+  // the workgroups of one pixel range (channel groups x tap passes) share an XCD and its L2
+  const int combos = cgroups * passes;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int combo = slot % combos;
+  const int range = xcd * (ranges >> 3) + slot / combos;
+  const int cg = combo % cgroups, pass = combo / cgroups;
+  const int a0 = blockIdx.y * kRgA;
+  const int k_base = pass * kRgKT;
+  const int tpr = (total_tiles + ranges - 1) / ranges;
+  const int t_begin = range * tpr, t_end = min(total_tiles, t_begin + tpr);
+  const int tw_mask = (1 << tw_shift) - 1, th = kTilePx >> tw_shift;
+  const int N = MH * MW;
+  const int64_t gplane = (int64_t)GH * GW;
+  const int g_first = cg * kRgG;
+
+  // roles.  Tap resolution: pixel p, taps half, half + 2, ...  Gather: pixel pair pp, the
+  // wave's 8 channels.  Plain tile: 16 lanes per row of 128 pixels, 16 rows per step.
+  const int p = tid & (kTilePx - 1), half = tid >> 7;
+  const int pp = lane;
+  const int64_t group = min(g_first / 8 + wave, Gpad / 8 - 1);  // (past Gpad: not stored)
+  constexpr int kTapsPerThread = (kRgKT + 1) / 2;
+  constexpr int kRowsPerStep = kThreads / 16, kSteps = kRgA / kRowsPerStep;
+  const int px0 = (tid & 15) * 8;
+
+  floatx4 acc[kRgKT][NB][MB];
+#pragma unroll
+  for (int k = 0; k < kRgKT; k++)
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+      for (int mb = 0; mb < MB; mb++) acc[k][nb][mb] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const bool sum_plain = plain_sum_part != nullptr && combo == 0;
+  float plain_sum[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; mb++) plain_sum[mb] = 0.f;
+
+  uint4 raw[kSteps];
+  float2 mxy[kTapsPerThread];
+  uint4 q[kRgDepth][4];
+
+  // (tiles past the range's end, which pad it to a whole number of ring periods, are fetched
+  // as zeros and weigh zero; their addresses are those of the last tile)
+  auto tile_origin = [&](int tile, int &b, int &i0, int &j0) __attribute__((always_inline)) {
+    tile = min(tile, t_end - 1);
+    b = tile / tiles_per_img;
+    const int t_in = tile - b * tiles_per_img;
+    const int tile_y = t_in / tiles_x, tile_x = t_in - tile_y * tiles_x;
+    i0 = tile_y * th;
+    j0 = tile_x << tw_shift;
+  };
+  // (the plain operand of an image as a buffer: rows past the last channel lie beyond its end
+  // and read as zeros, like the pieces outside the image, which get an offset out of range;
+  // a piece of 8 pixels never straddles the image's edge because MW is a multiple of 8)
+  const unsigned plain_rows = (unsigned)min(A - a0, kRgA);
+  auto fetch_plain = [&](int tile) __attribute__((always_inline)) {
+    int b, i0, j0;
+    tile_origin(tile, b, i0, j0);
+    const int si = i0 + (px0 >> tw_shift), sj = j0 + (px0 & tw_mask);
+    const auto rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<bf16_t *>(plain + ((int64_t)b * A + a0) * N), (short)0,
+        (int)(plain_rows * (unsigned)N * 2u), 0x00020000);
+    const unsigned off = (si < MH && sj < MW && tile < t_end)
+                             ? ((unsigned)(tid >> 4) * (unsigned)N + (unsigned)(si * MW + sj)) * 2u
+                             : 0xffffff00u;
+#pragma unroll
+    for (int r = 0; r < kSteps; r++)
+      raw[r] = __builtin_bit_cast(
+          uint4, __builtin_amdgcn_raw_buffer_load_b128(
+                     rsrc, (int)off, (int)((unsigned)(r * kRowsPerStep) * (unsigned)N * 2u), 0));
+  };
+  auto fetch_coords = [&](int tile) __attribute__((always_inline)) {
+    int b, i0, j0;
+    tile_origin(tile, b, i0, j0);
+    const int gi = min(i0 + (p >> tw_shift), MH - 1), gj = min(j0 + (p & tw_mask), MW - 1);
+    const int64_t n_g = (int64_t)gi * MW + gj;
+#pragma unroll
+    for (int t = 0; t < kTapsPerThread; t++) {
+      const int k = min(k_base + half + 2 * t, K - 1);
+      mxy[t] = *reinterpret_cast<const float2 *>(map + (n_g * K + k) * 2);
+    }
+  };
+  // taps of `tile`, from the coordinates fetch_coords(tile) brought, into half `par` of the
+  // tap cache: byte offsets into a channel block (16 bytes per pixel) and weights; pixels
+  // outside the image and taps past the last one weigh zero
+  auto resolve_taps = [&](int tile, int par) __attribute__((always_inline)) {
+    int b, i0, j0;
+    tile_origin(tile, b, i0, j0);
+    const bool live = i0 + (p >> tw_shift) < MH && j0 + (p & tw_mask) < MW && tile < t_end;
+#pragma unroll
+    for (int t = 0; t < kTapsPerThread; t++) {
+      const int k = half + 2 * t;
+      if (k < kRgKT) {
+        PairTap<4> tp;
+        resolve_pairs<4, 16>(mxy[t].x, mxy[t].y, GH, GW, wrap != 0,
+                             (live && k_base + k < K) ? 1.f : 0.f, tp);
+        *reinterpret_cast<uint2 *>(&TapOff[par][k][p][0]) = make_uint2(tp.off[0], tp.off[1]);
+        *reinterpret_cast<float2 *>(&TapWt[par][k][p][0]) = make_float2(tp.wt[0], tp.wt[1]);
+      }
+    }
+  };
+  // (the wave's block of 8 channels of an image as a buffer; tap offsets are bytes inside it)
+  auto gather_base = [&](int tile) __attribute__((always_inline)) {
+    const int b = min(tile, t_end - 1) / tiles_per_img;
+    return __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char *>(reinterpret_cast<const char *>(gath) +
+                           (((int64_t)b * (Gpad / 8) + group) * gplane) * 16),
+        (short)0, (int)((unsigned)gplane * 16u), 0x00020000);
+  };
+  // (SLOT is a constant once the unit loops are unrolled: the ring stays in registers)
+  auto issue = [&](__amdgpu_buffer_rsrc_t base, int par, int k, const int SLOT)
+                   __attribute__((always_inline)) {
+    const uint4 o = *reinterpret_cast<const uint4 *>(&TapOff[par][k][2 * pp][0]);
+    q[SLOT][0] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(base, (int)o.x, 0, 0));
+    q[SLOT][1] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(base, (int)o.y, 0, 0));
+    q[SLOT][2] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(base, (int)o.z, 0, 0));
+    q[SLOT][3] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(base, (int)o.w, 0, 0));
+  };
+  auto stage = [&](int par, int k, const int SLOT, int buf) __attribute__((always_inline)) {
+    const float4 w = *reinterpret_cast<const float4 *>(&TapWt[par][k][2 * pp][0]);
+    const unsigned x0[4] = {q[SLOT][0].x, q[SLOT][0].y, q[SLOT][0].z, q[SLOT][0].w};
+    const unsigned x1[4] = {q[SLOT][1].x, q[SLOT][1].y, q[SLOT][1].z, q[SLOT][1].w};
+    const unsigned y0[4] = {q[SLOT][2].x, q[SLOT][2].y, q[SLOT][2].z, q[SLOT][2].w};
+    const unsigned y1[4] = {q[SLOT][3].x, q[SLOT][3].y, q[SLOT][3].z, q[SLOT][3].w};
+    auto lo = [](unsigned v) { return __builtin_bit_cast(float, v << 16); };
+    auto hi = [](unsigned v) { return __builtin_bit_cast(float, v & 0xffff0000u); };
+#pragma unroll
+    for (int j = 0; j < 4; j++) {  // channels 2j and 2j + 1 of the wave's eight
+      const float e0 = __builtin_fmaf(w.y, lo(x1[j]), __builtin_fmaf(w.x, lo(x0[j]), 0.f));
+      const float e1 = __builtin_fmaf(w.w, lo(y1[j]), __builtin_fmaf(w.z, lo(y0[j]), 0.f));
+      const float o0 = __builtin_fmaf(w.y, hi(x1[j]), __builtin_fmaf(w.x, hi(x0[j]), 0.f));
+      const float o1 = __builtin_fmaf(w.w, hi(y1[j]), __builtin_fmaf(w.z, hi(y0[j]), 0.f));
+      // (hardware round-to-nearest-even, the two pixels of a channel in one word)
+      *reinterpret_cast<unsigned *>(&SB[buf][wave * 8 + 2 * j][2 * pp]) =
+          __builtin_bit_cast(unsigned, __builtin_convertvector(floatx2{e0, e1}, bf16x2));
+      *reinterpret_cast<unsigned *>(&SB[buf][wave * 8 + 2 * j + 1][2 * pp]) =
+          __builtin_bit_cast(unsigned, __builtin_convertvector(floatx2{o0, o1}, bf16x2));
+    }
+  };
+
+  int buf = 0;
+  // One tile.  The ring's period is kRgDepth units and a tile has kRgKT of them, so the slot
+  // of a unit depends on the tile's place (PHASE) among kRgDepth consecutive ones: unit k of
+  // the tile sits in slot (PHASE * kRgKT + k) % kRgDepth, and the unit issued in its place,
+  // kRgDepth units further on, takes the same slot.
+  auto run_tile = [&](auto phase_tag, int tile) __attribute__((always_inline)) {
+    constexpr int PHASE = decltype(phase_tag)::value;
+    const int par = (tile - t_begin) & 1;
+    __syncthreads();  // the previous tile's plain operand and the other half of the tap cache are free
+#pragma unroll
+    for (int r = 0; r < kSteps; r++)
+      *reinterpret_cast<uint4 *>(&PtB[(tid >> 4) + r * kRowsPerStep][px0]) = raw[r];
+    resolve_taps(tile + 1, par ^ 1);
+    __syncthreads();
+    bf16x8 aregb[MB][4];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+      for (int s4 = 0; s4 < 4; s4++)
+        aregb[mb][s4] = __builtin_bit_cast(
+            bf16x8, *reinterpret_cast<const uint4 *>(
+                        &PtB[(wave * MB + mb) * 16 + l15][32 * s4 + 8 * lq]));
+    if (sum_plain) {  // thread (row tid/4 of each 64, quarter tid%4) adds 32 pixels of its row
+#pragma unroll
+      for (int mb = 0; mb < MB; mb++) {
+        const uint4 *row =
+            reinterpret_cast<const uint4 *>(&PtB[64 * mb + (tid >> 2)][(tid & 3) * 32]);
+        float t = 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const uint4 v = row[r];
+          const unsigned w4[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+          for (int j = 0; j < 4; j++)
+            t += __builtin_bit_cast(float, w4[j] << 16) +
+                 __builtin_bit_cast(float, w4[j] & 0xffff0000u);
+        }
+        plain_sum[mb] += t;
+      }
+    }
+    fetch_plain(tile + 1);
+    fetch_coords(tile + 2);
+    const auto base = gather_base(tile), base_next = gather_base(tile + 1);
+#pragma unroll
+    for (int k = 0; k < kRgKT; k++) {
+      const int slot_k = (PHASE * kRgKT + k) % kRgDepth;
+      buf ^= 1;
+      stage(par, k, slot_k, buf);
+      __syncthreads();
+      if (k + kRgDepth < kRgKT)
+        issue(base, par, k + kRgDepth, slot_k);
+      else
+        issue(base_next, par ^ 1, k + kRgDepth - kRgKT, slot_k);
+#pragma unroll
+      for (int s4 = 0; s4 < 4; s4++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+          const bf16x8 bq = __builtin_bit_cast(
+              bf16x8,
+              *reinterpret_cast<const uint4 *>(&SB[buf][nb * 16 + l15][32 * s4 + 8 * lq]));
+#pragma unroll
+          for (int mb = 0; mb < MB; mb++)
+            acc[k][nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aregb[mb][s4], bq,
+                                                                     acc[k][nb][mb], 0, 0, 0);
+        }
+    }
+  };
+
+  // prologue: taps of the first tile, its plain operand, coordinates of the second, and the
+  // gathers of the first kRgDepth units (a range without tiles stores its zeros)
+  static_assert(kRgDepth == 2 || kRgDepth == 3, "run_tile is instantiated per phase below");
+  if (t_begin < t_end) {
+    fetch_coords(t_begin);
+    resolve_taps(t_begin, 0);
+    fetch_plain(t_begin);
+    fetch_coords(t_begin + 1);
+    __syncthreads();
+    {
+      const auto base0 = gather_base(t_begin);
+#pragma unroll
+      for (int u = 0; u < kRgDepth; u++) issue(base0, 0, u, u);
+    }
+    for (int tile = t_begin; tile < t_end; tile += kRgDepth) {
+      run_tile(std::integral_constant<int, 0>(), tile);
+      run_tile(std::integral_constant<int, 1>(), tile + 1);
+      if constexpr (kRgDepth == 3) run_tile(std::integral_constant<int, 2>(), tile + 2);
+    }
+  }
+
+  if (sum_plain) {  // the four quarters of a row sit in neighbouring lanes
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) {
+      float t = plain_sum[mb];
+      t += __shfl_xor(t, 1);
+      t += __shfl_xor(t, 2);
+      const int a = a0 + 64 * mb + (tid >> 2);
+      if ((tid & 3) == 0 && a < A) plain_sum_part[(int64_t)range * A + a] = t;
+    }
+  }
+  const int A4 = (A + 3) & ~3;
+  float *pr = part + (int64_t)range * A4 * G * K;
+#pragma unroll
+  for (int k = 0; k < kRgKT; k++) {
+    if (k_base + k < K) {
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++) {
+        const int g = g_first + nb * 16 + l15;
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) {
+          const int a = a0 + (wave * MB + mb) * 16 + lq * 4;
+          if (a < A && g < G)
+            *reinterpret_cast<floatx4 *>(&pr[((int64_t)(k_base + k) * G + g) * A4 + a]) =
+                acc[k][nb][mb];
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------
 // product_scatter: dst[b,d] += splat(sum_s W[s,d,k] * src[b,s,n], map[n,k])
 // (convolution backward-input: s = Co, d = Ci; transposed forward: s = Ci, d = Co).
 // One wavefront (= one workgroup) owns a row segment of 32 map pixels.  It keeps
@@ -1440,10 +1749,11 @@ inline bool use_channel_blocks(int64_t SH, int interp, size_t elem) {
 }
 template <typename TD>
 int launch_channel_blocks(const TD *src, TD *stage, int64_t B, int64_t G, int64_t plane,
-                          hipStream_t s) {
+                          hipStream_t s, const int *pair_mask = nullptr) {
   const int64_t Gpad = round_up(G, kGC);
   dim3 tg((unsigned)((plane + 255) / 256), (unsigned)(Gpad / 8), (unsigned)B);
-  hipLaunchKernelGGL(to_channel_blocks_kernel<TD>, tg, dim3(256), 0, s, src, stage, (int)G, plane);
+  hipLaunchKernelGGL(to_channel_blocks_kernel<TD>, tg, dim3(256), 0, s, src, stage, (int)G, plane,
+                     pair_mask);
   MCX_HIP_CHECK_LAUNCH();
   return 0;
 }
@@ -1643,15 +1953,23 @@ int mfma_gather_product(const TD *src, const float *map, const float *iw, const 
 // Per-range partial sums of gW, per-range partial sums of the plain operand, then
 // (single-row gathered operands) their channel-last copy.
 size_t mfma_weight_grad_bytes(int64_t B, int64_t A, int64_t G, int64_t MH, int64_t MW, int64_t K,
-                              int64_t GH, int64_t GW) {
-  // (sized for either storage type: the tiling and the number of ranges depend on it)
-  const size_t ranges =
+                              int64_t GH, int64_t GW, size_t elem) {
+  // (the tiling and the number of ranges depend on the storage type and on the kernel)
+  size_t ranges =
       (size_t)std::max(weight_grad_ranges<float>(make_tiling(B, MH, MW, 4).total, A, G, K),
                        weight_grad_ranges<bf16_t>(make_tiling(B, MH, MW, 2).total, A, G, K));
+  if (elem == 2)
+    ranges = std::max(
+        ranges, (size_t)ring_weight_grad_ranges(make_tiling(B, MH, MW, 2).total, A, G, K));
   size_t n = align256(ranges * (size_t)(round_up(A, 4) * G * K) * sizeof(float));
   n += align256(ranges * (size_t)A * sizeof(float));
   n += 256;  // the map's pair mask
-  if (GH == 1) n += align256((size_t)(B * GH * GW * round_up(G, kGC)) * sizeof(float));
+  // a copy of the gathered operand: channel-last for single-row sources, in blocks of 8
+  // channels for bf16 images
+  if (GH == 1)
+    n += align256((size_t)(B * GH * GW * round_up(G, kGC)) * sizeof(float));
+  else if (elem == 2)
+    n += align256((size_t)(B * GH * GW * round_up(G, kGC)) * elem);
   return n;
 }
 
@@ -1667,14 +1985,25 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
   if (t.total > 0x7fffffffLL) return MCX_E_SHAPE;
   if (GH * GW * (int64_t)sizeof(TD) > 0xffffffffLL) return MCX_E_SHAPE;  // 32-bit tap offsets
   constexpr int kWgA = wg_plain_channels<TD>(), kWgCB = wg_gathered_blocks<TD>();
-  const int ranges = weight_grad_ranges<TD>(t.total, A, G, K);
+  const ModeArgs m = mode_args(interp, P);
   const int cgroups = (int)((G + kWgCB * kGC - 1) / (kWgCB * kGC));
   const int64_t Gpad = round_up(G, kGC);
   const bool cl = use_channel_last(GH, interp) &&
                   GH * GW * Gpad * (int64_t)sizeof(TD) <= 0xffffffffLL;
+  // bf16 images under unweighted bilinear taps: the ring kernel takes the maps whose lower
+  // corners weigh nothing (the pair mask tells), the general form the others
+  // (its 16-byte pieces of the plain operand want rows that are a multiple of 8 pixels, and
+  // an image of either operand is addressed as a buffer of less than 4 GiB)
+  const bool ring = sizeof(TD) == 2 && !cl && m.np == 1 && m.mode != kInterpNearest &&
+                    GH * GW * 16 < 0xffffff00LL && MW % 8 == 0 &&
+                    (reinterpret_cast<uintptr_t>(plain) & 15) == 0 &&
+                    (int64_t)kRgA * MH * MW * 2 < 0xffffff00LL;
+  const int ranges = ring ? ring_weight_grad_ranges(t.total, A, G, K)
+                          : weight_grad_ranges<TD>(t.total, A, G, K);
   float *sum_part = reinterpret_cast<float *>(
       (char *)scratch + align256((size_t)ranges * (size_t)(round_up(A, 4) * G * K) * 4));
   int *pair_mask = reinterpret_cast<int *>((char *)sum_part + align256((size_t)ranges * A * 4));
+  int *const pair_mask_ws = pair_mask;  // (a plan may supply the mask; the copy's room follows this one)
   if (cl) {
     TD *stage = reinterpret_cast<TD *>((char *)pair_mask + 256);
     dim3 tg((unsigned)((GH * GW + 63) / 64), (unsigned)((Gpad + 63) / 64), (unsigned)B);
@@ -1685,7 +2014,6 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
   }
   dim3 grid((unsigned)(ranges * cgroups), (unsigned)((A + kWgA - 1) / kWgA),
             (unsigned)((K + kWgKT - 1) / kWgKT));
-  const ModeArgs m = mode_args(interp, P);
   // Four pairs per tap: it pays to find out (on the device) whether only the first two pairs
   // are ever in use (bilinear maps with integral rows, two of four points weighted) and to
   // launch both variants, of which one returns at once.
@@ -1704,7 +2032,7 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
                      plain_sum ? sum_part : (float *)nullptr, MASK, LEAD)
 #define MCX_LAUNCH_CL(NCORN, NP, CL)                                          \
   if constexpr (NCORN * NP == 4) {                                            \
-    MCX_LAUNCH_NA(NCORN, NP, CL, 2, pair_mask, 1);                            \
+    if (!ring) MCX_LAUNCH_NA(NCORN, NP, CL, 2, pair_mask, 1);                 \
     MCX_LAUNCH_NA(NCORN, NP, CL, NCORN * NP, pair_mask, 0);                   \
   } else {                                                                    \
     MCX_LAUNCH_NA(NCORN, NP, CL, NCORN * NP, (const int *)nullptr, 0);        \
@@ -1719,7 +2047,27 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
   } else {                                 \
     MCX_LAUNCH_CL(NCORN, NP, false);       \
   }
+  if constexpr (sizeof(TD) == 2) {
+    if (ring) {
+      TD *stage = reinterpret_cast<TD *>((char *)pair_mask_ws + 256);
+      if (int rc = launch_channel_blocks<TD>(gath, stage, B, G, GH * GW, s, pair_mask)) return rc;
+    }
+  }
   profile_begin(s);
+  if constexpr (sizeof(TD) == 2) {
+    if (ring) {
+      const int rg_groups = (int)((G + kRgG - 1) / kRgG), rg_passes = (int)((K + kRgKT - 1) / kRgKT);
+      hipLaunchKernelGGL(weight_grad_bf16_ring_kernel,
+                         dim3((unsigned)(ranges * rg_groups * rg_passes),
+                              (unsigned)((A + kRgA - 1) / kRgA)),
+                         dim3(kThreads), 0, s, plain,
+                         reinterpret_cast<const TD *>((char *)pair_mask_ws + 256), map, part,
+                         (int)A, (int)G, (int)Gpad, (int)GH, (int)GW, (int)MH, (int)MW, (int)K,
+                         m.wrap, t.tiles_x, t.tiles_per_img, t.tw_shift, (int)t.total, ranges,
+                         rg_groups, rg_passes, plain_sum ? sum_part : (float *)nullptr, pair_mask);
+      MCX_HIP_CHECK_LAUNCH();
+    }
+  }
   MCX_DISPATCH_TAPS(m, MCX_LAUNCH)
   profile_end(s);
 #undef MCX_LAUNCH
