@@ -1064,7 +1064,10 @@ constexpr int kRgLd = kTilePx + 8;  // bf16 elements per LDS row
 inline int ring_weight_grad_ranges(int64_t total_tiles, int64_t A, int64_t G, int64_t K) {
   const int64_t per_range = ((G + kRgG - 1) / kRgG) * ((A + kRgA - 1) / kRgA) *
                             ((K + kRgKT - 1) / kRgKT);
-  int64_t r = std::max<int64_t>(8, (1024 / per_range) / 8 * 8);  // about four workgroups per CU
+  // about twenty workgroups per CU, two of them resident at a time: they drift apart, and
+  // short ones even out the end of the launch (config 5: 27.8 / 26.3 / 25.6 / 25.6 ms per
+  // backward call with 1024 / 2560 / 5120 / 10240 workgroups)
+  int64_t r = std::max<int64_t>(8, (5120 / per_range) / 8 * 8);
   r = std::min<int64_t>(r, std::max<int64_t>(total_tiles / 8 * 8, 8));
   return (int)r;
 }
