@@ -233,6 +233,35 @@ def test_input_gradient_with_border_rows_beyond_two_entries(with_plan, dtype, de
         assert_close_elementwise(gr[0].float().cpu(), g_o[0], TOL[dtype])
 
 
+@pytest.mark.parametrize("interp", [1, 2])
+@pytest.mark.parametrize("shape", [(4, 130, 96, 40, 392, 2), (2, 72, 200, 33, 264, 1),
+                                   (3, 128, 128, 16, 1024, 2)])
+def test_bf16_weight_gradient_over_many_tiles_per_workgroup(shape, interp, device):
+    """bf16 storage under a latitude map (integral rows): the weight gradient's workgroups walk
+    runs of several row tiles with their gathers in flight across tile boundaries, runs that are
+    padded to a whole number of ring periods, ragged channel counts on both sides, rows that end
+    inside a tile, 9 and 25 taps (passes of 5 + 4 and 5 x 5).  Checked against the fp32 kernels on
+    the same bf16-valued inputs (themselves checked against the oracle), which differ by the
+    rounding of the samples to bf16 only; the oracle itself runs on the small cases elsewhere in
+    this file and on sampled positions at full size."""
+    B, Co, Ci, H, W, radius = shape
+    K = (2 * radius + 1) ** 2
+    g = torch.Generator().manual_seed(91)
+    x = torch.randn(B, Ci, H, W, generator=g).bfloat16().cuda()
+    gy = torch.randn(B, Co, H, W, generator=g).bfloat16().cuda()
+    w = (torch.randn(Co, Ci, K, generator=g) / (Ci * K) ** 0.5).bfloat16().cuda()
+    b = torch.randn(Co, generator=g).bfloat16().cuda()
+    smap = synthetic.latitude_map(H, W, radius).cuda()
+    got = _C.mapped_conv_backward(gy, smap, x, w, b, K, interp)
+    ref = _C.mapped_conv_backward(gy.float(), smap, x.float(), w.float(), b.float(), K, interp)
+    for a, r, nm in zip(got, ref, ("grad_input", "grad_weight", "grad_bias")):
+        assert rel_err(a.float(), r) < 2e-2, nm
+    assert_close_elementwise(got[1].float(), ref[1], 2e-2, "grad_weight")
+    # the same bits on every call (fixed summation order)
+    again = _C.mapped_conv_backward(gy, smap, x, w, b, K, interp)
+    assert torch.equal(got[1], again[1]) and torch.equal(got[2], again[2])
+
+
 def test_bf16_with_more_than_four_points_is_rejected(device):
     """bf16 storage exists on the matrix-core kernels only, which take at most four points."""
     g = torch.Generator().manual_seed(5)
