@@ -76,49 +76,61 @@ __device__ inline void direct_gather(const T *__restrict__ in, const T *__restri
     // other closely and hit in cache (with the taps outside, a line was gone before the
     // next tap came back to it: every sampled byte came from memory).
     constexpr int kTaps = 9;
-    if (P == 0 && K <= kTaps) {
-      Tap<T, MODE> taps[kTaps];
-#pragma unroll
-      for (int k = 0; k < kTaps; k++) {
-        const int64_t e = (int64_t)n * K + min(k, K - 1);
-        taps[k].set(map[e * 2], map[e * 2 + 1], IH, IW);
-      }
-      // wave-uniform: bit k set when some lane uses row 0 / row 1 of tap k, and when every
-      // lane's tap k can fetch a row's two corners with one load
-      unsigned rows0 = 0, rows1 = 0, pairs = 0;
-#pragma unroll
-      for (int k = 0; k < kTaps; k++) {
-        rows0 |= __builtin_amdgcn_ballot_w64(taps[k].row_in_use(0)) ? 1u << k : 0u;
-        rows1 |= __builtin_amdgcn_ballot_w64(taps[k].row_in_use(1)) ? 1u << k : 0u;
-        pairs |= __builtin_amdgcn_ballot_w64(!taps[k].pairable()) ? 0u : 1u << k;
-      }
-      for (int c = 0; c < nc; c++) {
-        const plane_buf_t pl = plane_buf(src + c * plane, plane_bytes);
-        // every load of the channel is issued before the first one is used (left to itself
-        // the compiler interleaves loads and waits to save registers, one load in flight)
-        T d[kTaps][Tap<T, MODE>::kCorners];
-#pragma unroll
-        for (int k = 0; k < kTaps; k++)
-          taps[k].load_rows(pl, d[k], (rows0 >> k) & 1u, (rows1 >> k) & 1u, (pairs >> k) & 1u);
-        __builtin_amdgcn_sched_barrier(0);
-        T val[kTaps];
-#pragma unroll
-        for (int k = 0; k < kTaps; k++) val[k] = taps[k].combine(d[k]);
-        T a = OP == OP_MAX ? T(-3.402823466e+38F) : T(0);
-        int bk = -1;
+    if (P == 0) {
+      // More than kTaps taps: groups of kTaps, each a pass over the planes that continues
+      // from the value (and winner) the pass before left in the output, so the additions and
+      // the comparisons keep the order of the taps.
+      for (int k0 = 0; k0 < K; k0 += kTaps) {
+        const int kn = min(kTaps, K - k0);
+        const bool first = k0 == 0, last = k0 + kTaps >= K;
+        Tap<T, MODE> taps[kTaps];
 #pragma unroll
         for (int k = 0; k < kTaps; k++) {
-          if (OP == OP_MAX) {
-            const bool better = k < K && val[k] > a;
-            a = better ? val[k] : a;
-            bk = better ? k : bk;
-          } else {
-            a = k < K ? a + val[k] : a;
-          }
+          const int64_t e = (int64_t)n * K + min(k0 + k, K - 1);
+          taps[k].set(map[e * 2], map[e * 2 + 1], IH, IW);
         }
-        out[o + (int64_t)c * N] = OP == OP_AVG ? a / (T)K : a;
-        if (OP == OP_MAX)
-          idx[o + (int64_t)c * N] = bk < 0 ? (int64_t)-1 : ((int64_t)n * K + bk) * 2;
+        // wave-uniform: bit k set when some lane uses row 0 / row 1 of tap k, and when every
+        // lane's tap k can fetch a row's two corners with one load
+        unsigned rows0 = 0, rows1 = 0, pairs = 0;
+#pragma unroll
+        for (int k = 0; k < kTaps; k++) {
+          rows0 |= __builtin_amdgcn_ballot_w64(taps[k].row_in_use(0)) ? 1u << k : 0u;
+          rows1 |= __builtin_amdgcn_ballot_w64(taps[k].row_in_use(1)) ? 1u << k : 0u;
+          pairs |= __builtin_amdgcn_ballot_w64(!taps[k].pairable()) ? 0u : 1u << k;
+        }
+        for (int c = 0; c < nc; c++) {
+          const plane_buf_t pl = plane_buf(src + c * plane, plane_bytes);
+          // every load of the channel is issued before the first one is used (left to itself
+          // the compiler interleaves loads and waits to save registers, one load in flight)
+          T a = OP == OP_MAX ? T(-3.402823466e+38F) : T(0);
+          int64_t best = -1;
+          if (!first) {  // (uniform over the launch)
+            a = out[o + (int64_t)c * N];
+            if (OP == OP_MAX) best = idx[o + (int64_t)c * N];
+          }
+          T d[kTaps][Tap<T, MODE>::kCorners];
+#pragma unroll
+          for (int k = 0; k < kTaps; k++)
+            taps[k].load_rows(pl, d[k], (rows0 >> k) & 1u, (rows1 >> k) & 1u, (pairs >> k) & 1u);
+          __builtin_amdgcn_sched_barrier(0);
+          T val[kTaps];
+#pragma unroll
+          for (int k = 0; k < kTaps; k++) val[k] = taps[k].combine(d[k]);
+          int bk = -1;
+#pragma unroll
+          for (int k = 0; k < kTaps; k++) {
+            if (OP == OP_MAX) {
+              const bool better = k < kn && val[k] > a;
+              a = better ? val[k] : a;
+              bk = better ? k : bk;
+            } else {
+              a = k < kn ? a + val[k] : a;
+            }
+          }
+          out[o + (int64_t)c * N] = (OP == OP_AVG && last) ? a / (T)K : a;
+          if (OP == OP_MAX)
+            idx[o + (int64_t)c * N] = bk < 0 ? best : ((int64_t)n * K + k0 + bk) * 2;
+        }
       }
       return;
     }
@@ -834,6 +846,40 @@ __global__ __launch_bounds__(kThreads) void sort_entries_kernel(
     }
     return;
   }
+  // Lists of 33 to 64 entries somewhere in the wave (5 x 5 pooling maps: about fifty): the
+  // wave sorts its lists one after the other, a lane per entry, by rank - the number of
+  // entries that come before it (by source, then weight, then position) - which is where the
+  // entry goes.  Same order as the insertion sort below, which took 5.4 ms for the 524 288
+  // lists of a 5 x 5 map on 512 x 1024 against 0.1 ms here.
+  {
+    const uint32_t len = live ? end - start : 0u;
+    const uint32_t longest = (uint32_t)wave_max((int)min(len, 0x7fffffffu));
+    if (longest > (uint32_t)kNetN && longest <= 64u) {
+      const uint32_t lane = threadIdx.x & 63;
+      for (int q = 0; q < 64; q++) {
+        const uint32_t s = (uint32_t)__builtin_amdgcn_readlane((int)start, q);
+        const uint32_t n = (uint32_t)__builtin_amdgcn_readlane((int)len, q);
+        if (n < 2u) continue;  // wave-uniform
+        const bool mine = lane < n;
+        const uint32_t code = e_src[s + (mine ? lane : 0u)];
+        const T w = e_wt[s + (mine ? lane : 0u)];
+        uint32_t rank = 0;
+        for (uint32_t j = 0; j < n; j++) {
+          const uint32_t cj = e_src[s + j];
+          const T wj = e_wt[s + j];
+          const bool tie = !(wj < w) && !(w < wj);
+          rank += (cj < code || (cj == code && (wj < w || (tie && j < lane)))) ? 1u : 0u;
+        }
+        // (every lane has read the whole list before the first one writes: the stores depend
+        // on all of the wave's loads)
+        if (mine) {
+          e_src[s + rank] = code;
+          e_wt[s + rank] = w;
+        }
+      }
+      return;
+    }
+  }
   if (!live) return;
   if (end - start > kSortMax) return;
   for (uint32_t i = start + 1; i < end; i++) {
@@ -1055,7 +1101,7 @@ template <typename T, int OP>
 __device__ inline void transposed_gather_planes(
     const T *__restrict__ src, const int64_t *__restrict__ idx, T *__restrict__ dst,
     const uint32_t *__restrict__ e_src, const T *__restrict__ e_wt, uint32_t start, uint32_t end,
-    int p, int64_t plane0, int nc, int nsrc, int ndst, int K, int idx_scale) {
+    int p, int64_t plane0, int nc, int nsrc, int ndst, int K, int idx_scale, uint32_t longest) {
   constexpr int kTCH = planes_per_thread<OP>();
   const T *s0 = src + plane0 * nsrc;
   const int64_t *i0 = OP == UN_MAX ? idx + plane0 * nsrc : nullptr;
@@ -1065,48 +1111,57 @@ __device__ inline void transposed_gather_planes(
   // every sampled byte came from memory.  The additions keep the order of the list.
   constexpr int kListRegs = 24, kGroup = 6;
   const uint32_t len = end - start;
-  if (OP != UN_RESAMPLE && __builtin_amdgcn_ballot_w64(len > (uint32_t)kListRegs) == 0) {
-    uint32_t code[kListRegs];
-    T w[kListRegs];
-    uint32_t longest = len;
-    for (int d = 32; d > 0; d >>= 1) longest = max(longest, (uint32_t)__shfl_xor((int)longest, d));
-    longest = __builtin_amdgcn_readfirstlane(longest);
-#pragma unroll
-    for (int u = 0; u < kListRegs; u++) {
-      const bool in = (uint32_t)u < len;
-      code[u] = e_src[in ? start + u : (len ? start : 0u)];
-      w[u] = in ? e_wt[start + u] : T(0);
-    }
+  if (OP != UN_RESAMPLE) {
+    // (`longest`: the longest list of the wave, taken by the caller while all 64 lanes were
+    // still there)
     T *d0 = dst + plane0 * ndst + p;
-    for (int c = 0; c < nc; c++) {
-      const T *sc = s0 + (int64_t)c * nsrc;
-      const int64_t *ic = OP == UN_MAX ? i0 + (int64_t)c * nsrc : nullptr;
-      T a = T(0);
+    // Lists longer than kListRegs (5 x 5 pooling maps: about fifty entries) take several
+    // passes of kListRegs entries over the planes; a pass continues from the sum the pass
+    // before left in the destination, so the order of the additions stays that of the list.
+    uint32_t base = 0;
+    do {
+      const uint32_t part = len > base ? len - base : 0u;  // this lane's entries in the pass
+      const uint32_t wave_part = longest - base;
+      const bool first = base == 0, last = base + kListRegs >= longest;
+      uint32_t code[kListRegs];
+      T w[kListRegs];
 #pragma unroll
-      for (int g = 0; g < kListRegs / kGroup; g++) {
-        if ((uint32_t)(g * kGroup) < longest) {  // wave-uniform, once per six entries
-          T v[kGroup];
-          bool keep[kGroup];
-#pragma unroll
-          for (int j = 0; j < kGroup; j++) {
-            const uint32_t cd = code[g * kGroup + j];
-            const uint32_t n = OP == UN_MAX ? cd / (uint32_t)K : cd;
-            v[j] = sc[n];
-            // Entries past the end of a lane's list are dropped by a test, not by their zero
-            // weight (an Inf or NaN in an unrelated source element must not reach the
-            // destination).  Max unpooling keeps the recorded-winner test alone: its padded
-            // entries repeat the lane's own first entry with weight zero, and the extra test
-            // cost it a third of its speed.
-            keep[j] = OP == UN_MAX ? ic[n] == (int64_t)cd * idx_scale
-                                   : (uint32_t)(g * kGroup + j) < len;
-          }
-#pragma unroll
-          for (int j = 0; j < kGroup; j++)
-            if (keep[j]) a = mcx_fma(w[g * kGroup + j], v[j], a);
-        }
+      for (int u = 0; u < kListRegs; u++) {
+        const bool in = (uint32_t)u < part;
+        code[u] = e_src[in ? start + base + u : (len ? start : 0u)];
+        w[u] = in ? e_wt[start + base + u] : T(0);
       }
-      d0[(int64_t)c * ndst] = OP == UN_AVG ? a / (T)K : a;
-    }
+      for (int c = 0; c < nc; c++) {
+        const T *sc = s0 + (int64_t)c * nsrc;
+        const int64_t *ic = OP == UN_MAX ? i0 + (int64_t)c * nsrc : nullptr;
+        T a = first ? T(0) : d0[(int64_t)c * ndst];
+#pragma unroll
+        for (int g = 0; g < kListRegs / kGroup; g++) {
+          if ((uint32_t)(g * kGroup) < wave_part) {  // wave-uniform, once per six entries
+            T v[kGroup];
+            bool keep[kGroup];
+#pragma unroll
+            for (int j = 0; j < kGroup; j++) {
+              const uint32_t cd = code[g * kGroup + j];
+              const uint32_t n = OP == UN_MAX ? cd / (uint32_t)K : cd;
+              v[j] = sc[n];
+              // Entries past the end of a lane's list are dropped by a test, not by their zero
+              // weight (an Inf or NaN in an unrelated source element must not reach the
+              // destination).  Max unpooling keeps the recorded-winner test alone: its padded
+              // entries repeat the lane's own first entry with weight zero, and the extra test
+              // cost it a third of its speed.
+              keep[j] = OP == UN_MAX ? ic[n] == (int64_t)cd * idx_scale
+                                     : (uint32_t)(g * kGroup + j) < part;
+            }
+#pragma unroll
+            for (int j = 0; j < kGroup; j++)
+              if (keep[j]) a = mcx_fma(w[g * kGroup + j], v[j], a);
+          }
+        }
+        d0[(int64_t)c * ndst] = (OP == UN_AVG && last) ? a / (T)K : a;
+      }
+      base += kListRegs;
+    } while (base < longest);
     return;
   }
   if constexpr (OP == UN_RESAMPLE) {
@@ -1128,10 +1183,6 @@ __device__ inline void transposed_gather_planes(
 #pragma unroll
       for (int c = 0; c < kTCH; c++) acc[c] = T(0);
       const uint32_t len = end - start;
-      // (lanes past the last pixel have left: the ballot-free reduction below needs all 64)
-      uint32_t longest = len;
-      for (int d = 32; d > 0; d >>= 1) longest = max(longest, (uint32_t)__shfl_xor((int)longest, d));
-      longest = __builtin_amdgcn_readfirstlane(longest);
       constexpr int kRegs = 8, kStep = 4;
       if (longest <= (uint32_t)kRegs) {
         // the whole list first (one round trip), then the samples, four entries at a time
@@ -1258,11 +1309,12 @@ __global__ __launch_bounds__(kThreads, OP == UN_AVG ? 4 : OP == UN_MAX ? 3 : 1) 
                                         live, p, first_plane, np, nsrc, ndst, K, idx_scale))
       return;
   }
+  const uint32_t longest = (uint32_t)wave_max(live ? (int)(end - start) : 0);
   if (!live) return;
   for (int done = 0; done < np; done += kTCH)
     transposed_gather_planes<T, OP>(src, idx, dst, e_src, e_wt, start, end, p,
                                     first_plane + done, min(kTCH, np - done), nsrc, ndst, K,
-                                    idx_scale);
+                                    idx_scale, longest);
 }
 
 bool bad_dims(std::initializer_list<int64_t> dims) {
@@ -1286,7 +1338,7 @@ int launch_gather(const void *in, const void *map, const void *iw, void *out, in
                   int64_t P, int interp, hipStream_t s) {
   const int64_t N = MH * MW;
   // (the same test as in direct_gather: unweighted pooling with at most 9 taps)
-  const bool tap_registers = OP != OP_RESAMPLE && P == 0 && K <= 9;
+  const bool tap_registers = OP != OP_RESAMPLE && P == 0;
   int cpt = tap_registers ? kPoolCH : kCH;
   if (tap_registers && B * C <= 0x7fffffffLL) {
     // Images and channels are one run of planes to these kernels, and resolving a thread's
@@ -1310,7 +1362,7 @@ int launch_gather(const void *in, const void *map, const void *iw, void *out, in
   }
   dim3 grid(div_up(MW, Patch<OP>::kW) * div_up(MH, Patch<OP>::kH), div_up(C, cpt), (unsigned)B);
   // (the LDS-window path copies 16-byte chunks of source rows)
-  const int windows = plane_ring || (tap_registers && N * 8 < (int64_t)kOobOffset &&
+  const int windows = plane_ring || (tap_registers && K <= 9 && N * 8 < (int64_t)kOobOffset &&
                                      IW % (16 / (int)sizeof(T)) == 0 &&
                                      (reinterpret_cast<uintptr_t>(in) & 15) == 0)
                           ? 1

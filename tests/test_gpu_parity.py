@@ -582,7 +582,8 @@ def test_pools_with_more_channels_than_one_thread_takes(interp, device):
 def test_unpool_list_lengths_for_both_sorting_networks(radius, interp, device):
     """Unpooling through latitude maps whose per-pixel contribution lists are 9 to 16 entries
     long (3x3 bilinear: the 16-key sorting network) and 17 to 32 (5x5 nearest: 25 entries,
-    the 32-key network) or longer (5x5 bilinear: 50, insertion sort): same values as the
+    the 32-key network) or longer (5x5 bilinear: 50 - sorted by rank, a lane per entry, and
+    gathered in passes of 24 entries that continue from the destination): same values as the
     oracle, and the same bits on every call."""
     B, C, H, W = 2, 3, 24, 128
     K = (2 * radius + 1) ** 2
