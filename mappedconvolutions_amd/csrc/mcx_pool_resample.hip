@@ -850,7 +850,7 @@ __global__ __launch_bounds__(kThreads) void sort_entries_kernel(
   // wave sorts its lists one after the other, a lane per entry, by rank - the number of
   // entries that come before it (by source, then weight, then position) - which is where the
   // entry goes.  Same order as the insertion sort below, which took 5.4 ms for the 524 288
-  // lists of a 5 x 5 map on 512 x 1024 against 0.1 ms here.
+  // lists of a 5 x 5 map on 512 x 1024.
   {
     const uint32_t len = live ? end - start : 0u;
     const uint32_t longest = (uint32_t)wave_max((int)min(len, 0x7fffffffu));
@@ -864,9 +864,17 @@ __global__ __launch_bounds__(kThreads) void sort_entries_kernel(
         const uint32_t code = e_src[s + (mine ? lane : 0u)];
         const T w = e_wt[s + (mine ? lane : 0u)];
         uint32_t rank = 0;
-        for (uint32_t j = 0; j < n; j++) {
-          const uint32_t cj = e_src[s + j];
-          const T wj = e_wt[s + j];
+        for (uint32_t j = 0; j < n; j++) {  // (entry j sits in lane j)
+          const uint32_t cj = (uint32_t)__builtin_amdgcn_readlane((int)code, (int)j);
+          T wj;
+          if constexpr (sizeof(T) == 4) {
+            wj = __builtin_bit_cast(T, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w), (int)j));
+          } else {
+            const long long wb = __builtin_bit_cast(long long, w);
+            const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)wb, (int)j);
+            const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(wb >> 32), (int)j);
+            wj = __builtin_bit_cast(T, (long long)(((unsigned long long)hi << 32) | lo));
+          }
           const bool tie = !(wj < w) && !(w < wj);
           rank += (cj < code || (cj == code && (wj < w || (tie && j < lane)))) ? 1u : 0u;
         }
