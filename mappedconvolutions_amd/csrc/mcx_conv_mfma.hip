@@ -192,6 +192,8 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
   // accumulated.
   __shared__ unsigned TapMask[TG][2][2];
   if (gate && ((*gate == 0) != (run_if_zero != 0))) return;  // device-side path selection
+  if (pair_mask && !row_mask && (((unsigned)*pair_mask < (1u << 2)) != (run_if_leading != 0)))
+    return;
   // a pass that adds onto y (the second level of a transposed map) has nothing to do when
   // no pair of its map is in use
   if (accumulate && pair_mask && *pair_mask == 0) return;
@@ -203,7 +205,7 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
   const int tile_y = t_in / tiles_x, tile_x = t_in - tile_y * tiles_x;
   const int tw_mask = (1 << tw_shift) - 1;
   const int th = kTilePx >> tw_shift;
-  if (pair_mask) {
+  if (pair_mask && row_mask) {
     // The two-pair form serves the whole map when no tap anywhere uses a later pair; with
     // `row_mask` (one word per row of output pixels, nonzero iff a tap of the row does) it
     // serves every tile whose rows are clear, and the general form the others: a few border
