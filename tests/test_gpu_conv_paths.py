@@ -262,6 +262,32 @@ def test_bf16_weight_gradient_over_many_tiles_per_workgroup(shape, interp, devic
     assert torch.equal(got[1], again[1]) and torch.equal(got[2], again[2])
 
 
+@pytest.mark.parametrize("interp", [1, 2])
+@pytest.mark.parametrize("with_plan", [False, True])
+def test_bf16_transposed_conv_under_a_map_with_integral_rows(with_plan, interp, device):
+    """Transposed convolution, bf16 storage, latitude map: its weight gradient (plain operand the
+    input, gathered operand grad_output) takes the same bf16 kernel as the convolution's, and
+    its input gradient the two-pair gather-product."""
+    B, Ci, Co, H, W, K = 2, 20, 36, 12, 136, 9
+    g = torch.Generator().manual_seed(123 + interp)
+    bf = lambda t: t.to(torch.bfloat16)
+    x, gy = bf(torch.randn(B, Ci, H, W, generator=g)), bf(torch.randn(B, Co, H, W, generator=g))
+    w = bf(torch.randn(Ci, Co, K, generator=g) / (Ci * K) ** 0.5)
+    b = bf(torch.randn(Co, generator=g))
+    smap = synthetic.latitude_map(H, W, 1)
+    y_o = O.mapped_transposed_conv_forward(x.float(), smap, w.float(), b.float(), H, W, K, interp)
+    g_o = O.mapped_transposed_conv_backward(gy.float(), smap, x.float(), w.float(), b.float(), K,
+                                            interp)
+    xd, sd, wd_, bd, gyd = dev(x, smap, w, b, gy)
+    plan = _C.conv_map_plan(sd, None, H, W, interp, torch.bfloat16) if with_plan else None
+    y = _C.mapped_transposed_conv_forward(xd, sd, wd_, bd, H, W, K, interp, plan=plan)
+    gr = _C.mapped_transposed_conv_backward(gyd, sd, xd, wd_, bd, K, interp, plan=plan)
+    assert rel_err(y.float(), y_o) < 2e-2
+    for a, r, nm in zip(gr, g_o, ("grad_input", "grad_weight", "grad_bias")):
+        assert rel_err(a.float(), r) < 2e-2, nm
+    assert_close_elementwise(gr[1].float(), g_o[1], 2e-2, "grad_weight")
+
+
 def test_bf16_with_more_than_four_points_is_rejected(device):
     """bf16 storage exists on the matrix-core kernels only, which take at most four points."""
     g = torch.Generator().manual_seed(5)
