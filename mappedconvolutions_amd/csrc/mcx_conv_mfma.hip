@@ -1040,18 +1040,22 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(
 }
 
 // ---------------------------------------------------------------------------------
-// Weight gradient, bf16 storage, bilinear taps whose two lower corners weigh nothing anywhere
-// in the map (integral row coordinates), gathered operand in blocks of 8 channels per pixel
-// ([B][Gpad/8][GH*GW][8], to_channel_blocks_kernel).  With bf16 MFMA the products are short
+// Weight gradient, bf16 storage, unweighted bilinear taps, gathered operand in blocks of 8
+// channels per pixel ([B][Gpad/8][GH*GW][8], to_channel_blocks_kernel).  NA == 2: maps whose
+// two lower corners weigh nothing anywhere (integral row coordinates); NA == 4: all others (the
+// pair mask of the map lets one of the two launches run).  With bf16 MFMA the products are short
 // and the kernel lives or dies by its gather, so this form is built around it:
 //   * a thread gathers two neighbouring pixels x 8 channels of a unit (one tap, 32 gathered
 //     channels): four 16-byte loads instead of 32 two-byte ones (the texture path resolves
 //     four lanes per clock whatever the width), and a channel's two pixels leave as one
 //     32-bit LDS store, consecutive lanes to consecutive banks;
-//   * the loads of kRgDepth units are in flight, across tile boundaries: the taps of the next
-//     tile are resolved (into the other half of a double-buffered tap cache) and the next
-//     plain tile is fetched into registers while this tile's units are multiplied, so that in
-//     the steady state no wave waits for memory at a tile's start;
+//   * NA == 2: the loads of kRgDepth units are in flight, across tile boundaries: the taps of
+//     the next tile are resolved (into the other half of a double-buffered tap cache) and the
+//     next plain tile is fetched into registers while this tile's units are multiplied, so
+//     that in the steady state no wave waits for memory at a tile's start.  NA == 4 has twice
+//     the loads per unit and the same registers: one unit in flight (the next unit's loads are
+//     issued before this unit's products), a single tap cache, the first unit of a tile waited
+//     for;
 //   * every load and store is unconditional (past the range's last tile the last one is
 //     fetched again, padded taps weigh zero), so the compiler's waits count exactly;
 //   * five taps per pass keep the accumulators at 80 registers, which leaves room for the
@@ -1074,18 +1078,24 @@ inline int ring_weight_grad_ranges(int64_t total_tiles, int64_t A, int64_t G, in
   return (int)r;
 }
 
+template <int NA>
 __global__ __launch_bounds__(kThreads, 2) void weight_grad_bf16_ring_kernel(
     const bf16_t *__restrict__ plain, const bf16_t *__restrict__ gath,
     const float *__restrict__ map, float *__restrict__ part, int A, int G, int Gpad, int GH,
     int GW, int MH, int MW, int K, int wrap, int tiles_x, int tiles_per_img, int tw_shift,
     int total_tiles, int ranges, int cgroups, int passes, float *__restrict__ plain_sum_part,
     const int *__restrict__ pair_mask) {
-  if (pair_mask && (unsigned)*pair_mask >= (1u << 2)) return;  // the general form runs instead
+  // NA == 2 runs while no tap of the map uses a pair beyond its first two, NA == 4 otherwise
+  if (pair_mask && (((unsigned)*pair_mask < (1u << 2)) != (NA == 2))) return;
+  static_assert(NA == 2 || NA == 4, "two or four pairs per tap");
+  constexpr bool kCross = NA == 2;               // gathers in flight across tile boundaries
+  constexpr int kDepth = kCross ? kRgDepth : 1;  // units in flight
+  constexpr int kTapBufs = kCross ? 2 : 1;
   constexpr int MB = kRgA / 64, NB = kRgG / 16;
   __shared__ __attribute__((aligned(16))) uint16_t PtB[kRgA][kRgLd];
   __shared__ __attribute__((aligned(16))) uint16_t SB[2][kRgG][kRgLd];
-  __shared__ __attribute__((aligned(16))) unsigned TapOff[2][kRgKT][kTilePx][2];
-  __shared__ __attribute__((aligned(16))) float TapWt[2][kRgKT][kTilePx][2];
+  __shared__ __attribute__((aligned(16))) unsigned TapOff[kTapBufs][kRgKT][kTilePx][NA];
+  __shared__ __attribute__((aligned(16))) float TapWt[kTapBufs][kRgKT][kTilePx][NA];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1128,7 +1138,7 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_bf16_ring_kernel(
 
   uint4 raw[kSteps];
   float2 mxy[kTapsPerThread];
-  uint4 q[kRgDepth][4];
+  uint4 q[kDepth][2 * NA];  // [unit in flight][pixel of the pair * NA + pair of the tap]
 
   // (tiles past the range's end, which pad it to a whole number of ring periods, are fetched
   // as zeros and weigh zero; their addresses are those of the last tile)
@@ -1185,8 +1195,15 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_bf16_ring_kernel(
         PairTap<4> tp;
         resolve_pairs<4, 16>(mxy[t].x, mxy[t].y, GH, GW, wrap != 0,
                              (live && k_base + k < K) ? 1.f : 0.f, tp);
-        *reinterpret_cast<uint2 *>(&TapOff[par][k][p][0]) = make_uint2(tp.off[0], tp.off[1]);
-        *reinterpret_cast<float2 *>(&TapWt[par][k][p][0]) = make_float2(tp.wt[0], tp.wt[1]);
+        if constexpr (NA == 2) {
+          *reinterpret_cast<uint2 *>(&TapOff[par][k][p][0]) = make_uint2(tp.off[0], tp.off[1]);
+          *reinterpret_cast<float2 *>(&TapWt[par][k][p][0]) = make_float2(tp.wt[0], tp.wt[1]);
+        } else {
+          *reinterpret_cast<uint4 *>(&TapOff[par][k][p][0]) =
+              make_uint4(tp.off[0], tp.off[1], tp.off[2], tp.off[3]);
+          *reinterpret_cast<float4 *>(&TapWt[par][k][p][0]) =
+              make_float4(tp.wt[0], tp.wt[1], tp.wt[2], tp.wt[3]);
+        }
       }
     }
   };
@@ -1201,31 +1218,48 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_bf16_ring_kernel(
   // (SLOT is a constant once the unit loops are unrolled: the ring stays in registers)
   auto issue = [&](__amdgpu_buffer_rsrc_t base, int par, int k, const int SLOT)
                    __attribute__((always_inline)) {
-    const uint4 o = *reinterpret_cast<const uint4 *>(&TapOff[par][k][2 * pp][0]);
-    q[SLOT][0] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(base, (int)o.x, 0, 0));
-    q[SLOT][1] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(base, (int)o.y, 0, 0));
-    q[SLOT][2] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(base, (int)o.z, 0, 0));
-    q[SLOT][3] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(base, (int)o.w, 0, 0));
+    // (the 2 * NA offsets of the pixel pair are consecutive words)
+    const uint4 *op = reinterpret_cast<const uint4 *>(&TapOff[par][k][2 * pp][0]);
+#pragma unroll
+    for (int h = 0; h < NA / 2; h++) {
+      const uint4 o = op[h];
+      const unsigned ov[4] = {o.x, o.y, o.z, o.w};
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+        q[SLOT][4 * h + i] = __builtin_bit_cast(
+            uint4, __builtin_amdgcn_raw_buffer_load_b128(base, (int)ov[i], 0, 0));
+    }
   };
   auto stage = [&](int par, int k, const int SLOT, int buf) __attribute__((always_inline)) {
-    const float4 w = *reinterpret_cast<const float4 *>(&TapWt[par][k][2 * pp][0]);
-    const unsigned x0[4] = {q[SLOT][0].x, q[SLOT][0].y, q[SLOT][0].z, q[SLOT][0].w};
-    const unsigned x1[4] = {q[SLOT][1].x, q[SLOT][1].y, q[SLOT][1].z, q[SLOT][1].w};
-    const unsigned y0[4] = {q[SLOT][2].x, q[SLOT][2].y, q[SLOT][2].z, q[SLOT][2].w};
-    const unsigned y1[4] = {q[SLOT][3].x, q[SLOT][3].y, q[SLOT][3].z, q[SLOT][3].w};
+    // weights of the pixel pair: NA for the first pixel, then NA for the second
+    float wv[2 * NA];
+    {
+      const float4 *wp4 = reinterpret_cast<const float4 *>(&TapWt[par][k][2 * pp][0]);
+#pragma unroll
+      for (int h = 0; h < NA / 2; h++) {
+        const float4 t = wp4[h];
+        wv[4 * h] = t.x; wv[4 * h + 1] = t.y; wv[4 * h + 2] = t.z; wv[4 * h + 3] = t.w;
+      }
+    }
     auto lo = [](unsigned v) { return __builtin_bit_cast(float, v << 16); };
     auto hi = [](unsigned v) { return __builtin_bit_cast(float, v & 0xffff0000u); };
 #pragma unroll
     for (int j = 0; j < 4; j++) {  // channels 2j and 2j + 1 of the wave's eight
-      const float e0 = __builtin_fmaf(w.y, lo(x1[j]), __builtin_fmaf(w.x, lo(x0[j]), 0.f));
-      const float e1 = __builtin_fmaf(w.w, lo(y1[j]), __builtin_fmaf(w.z, lo(y0[j]), 0.f));
-      const float o0 = __builtin_fmaf(w.y, hi(x1[j]), __builtin_fmaf(w.x, hi(x0[j]), 0.f));
-      const float o1 = __builtin_fmaf(w.w, hi(y1[j]), __builtin_fmaf(w.z, hi(y0[j]), 0.f));
+      float e[2] = {0.f, 0.f}, o[2] = {0.f, 0.f};  // [pixel of the pair]
+#pragma unroll
+      for (int px = 0; px < 2; px++)
+#pragma unroll
+        for (int i = 0; i < NA; i++) {  // in the order of the pairs, like every other kernel
+          const uint4 t = q[SLOT][px * NA + i];
+          const unsigned word = j == 0 ? t.x : j == 1 ? t.y : j == 2 ? t.z : t.w;
+          e[px] = __builtin_fmaf(wv[px * NA + i], lo(word), e[px]);
+          o[px] = __builtin_fmaf(wv[px * NA + i], hi(word), o[px]);
+        }
       // (hardware round-to-nearest-even, the two pixels of a channel in one word)
       *reinterpret_cast<unsigned *>(&SB[buf][wave * 8 + 2 * j][2 * pp]) =
-          __builtin_bit_cast(unsigned, __builtin_convertvector(floatx2{e0, e1}, bf16x2));
+          __builtin_bit_cast(unsigned, __builtin_convertvector(floatx2{e[0], e[1]}, bf16x2));
       *reinterpret_cast<unsigned *>(&SB[buf][wave * 8 + 2 * j + 1][2 * pp]) =
-          __builtin_bit_cast(unsigned, __builtin_convertvector(floatx2{o0, o1}, bf16x2));
+          __builtin_bit_cast(unsigned, __builtin_convertvector(floatx2{o[0], o[1]}, bf16x2));
     }
   };
 
@@ -1236,12 +1270,17 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_bf16_ring_kernel(
   // kRgDepth units further on, takes the same slot.
   auto run_tile = [&](auto phase_tag, int tile) __attribute__((always_inline)) {
     constexpr int PHASE = decltype(phase_tag)::value;
-    const int par = (tile - t_begin) & 1;
-    __syncthreads();  // the previous tile's plain operand and the other half of the tap cache are free
+    // (kCross: `mxy` holds the coordinates of the next tile, whose taps go to the other half
+    // of the cache; else those of this tile, resolved now)
+    const int par = kCross ? (tile - t_begin) & 1 : 0;
+    __syncthreads();  // the previous tile's plain operand and the tap cache to be written are free
 #pragma unroll
     for (int r = 0; r < kSteps; r++)
       *reinterpret_cast<uint4 *>(&PtB[(tid >> 4) + r * kRowsPerStep][px0]) = raw[r];
-    resolve_taps(tile + 1, par ^ 1);
+    if constexpr (kCross)
+      resolve_taps(tile + 1, par ^ 1);
+    else
+      resolve_taps(tile, 0);
     __syncthreads();
     bf16x8 aregb[MB][4];
 #pragma unroll
@@ -1269,19 +1308,20 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_bf16_ring_kernel(
         plain_sum[mb] += t;
       }
     }
-    fetch_plain(tile + 1);
-    fetch_coords(tile + 2);
     const auto base = gather_base(tile), base_next = gather_base(tile + 1);
+    if constexpr (!kCross) issue(base, 0, 0, 0);  // (before the prefetches: it is waited for first)
+    fetch_plain(tile + 1);
+    fetch_coords(kCross ? tile + 2 : tile + 1);
 #pragma unroll
     for (int k = 0; k < kRgKT; k++) {
-      const int slot_k = (PHASE * kRgKT + k) % kRgDepth;
+      const int slot_k = (PHASE * kRgKT + k) % kDepth;
       buf ^= 1;
       stage(par, k, slot_k, buf);
       __syncthreads();
-      if (k + kRgDepth < kRgKT)
-        issue(base, par, k + kRgDepth, slot_k);
-      else
-        issue(base_next, par ^ 1, k + kRgDepth - kRgKT, slot_k);
+      if (k + kDepth < kRgKT)
+        issue(base, par, k + kDepth, slot_k);
+      else if constexpr (kCross)
+        issue(base_next, par ^ 1, k + kDepth - kRgKT, slot_k);
 #pragma unroll
       for (int s4 = 0; s4 < 4; s4++)
 #pragma unroll
@@ -1302,19 +1342,23 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_bf16_ring_kernel(
   static_assert(kRgDepth == 2 || kRgDepth == 3, "run_tile is instantiated per phase below");
   if (t_begin < t_end) {
     fetch_coords(t_begin);
-    resolve_taps(t_begin, 0);
-    fetch_plain(t_begin);
-    fetch_coords(t_begin + 1);
-    __syncthreads();
-    {
+    if constexpr (kCross) {
+      resolve_taps(t_begin, 0);
+      fetch_plain(t_begin);
+      fetch_coords(t_begin + 1);
+      __syncthreads();
       const auto base0 = gather_base(t_begin);
 #pragma unroll
-      for (int u = 0; u < kRgDepth; u++) issue(base0, 0, u, u);
-    }
-    for (int tile = t_begin; tile < t_end; tile += kRgDepth) {
-      run_tile(std::integral_constant<int, 0>(), tile);
-      run_tile(std::integral_constant<int, 1>(), tile + 1);
-      if constexpr (kRgDepth == 3) run_tile(std::integral_constant<int, 2>(), tile + 2);
+      for (int u = 0; u < kDepth; u++) issue(base0, 0, u, u);
+      for (int tile = t_begin; tile < t_end; tile += kDepth) {
+        run_tile(std::integral_constant<int, 0>(), tile);
+        run_tile(std::integral_constant<int, 1>(), tile + 1);
+        if constexpr (kDepth == 3) run_tile(std::integral_constant<int, 2>(), tile + 2);
+      }
+    } else {
+      fetch_plain(t_begin);
+      for (int tile = t_begin; tile < t_end; ++tile)
+        run_tile(std::integral_constant<int, 0>(), tile);
     }
   }
 
@@ -1995,8 +2039,9 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
   const int64_t Gpad = round_up(G, kGC);
   const bool cl = use_channel_last(GH, interp) &&
                   GH * GW * Gpad * (int64_t)sizeof(TD) <= 0xffffffffLL;
-  // bf16 images under unweighted bilinear taps: the ring kernel takes the maps whose lower
-  // corners weigh nothing (the pair mask tells), the general form the others
+  // bf16 images under unweighted bilinear taps: the ring kernel, in its two-pair form for maps
+  // whose lower corners weigh nothing and its four-pair form for the others (the pair mask
+  // lets one of the two launches run)
   // (its 16-byte pieces of the plain operand want rows that are a multiple of 8 pixels, and
   // an image of either operand is addressed as a buffer of less than 4 GiB)
   const bool ring = sizeof(TD) == 2 && !cl && m.np == 1 && m.mode != kInterpNearest &&
@@ -2037,8 +2082,10 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
                      plain_sum ? sum_part : (float *)nullptr, MASK, LEAD)
 #define MCX_LAUNCH_CL(NCORN, NP, CL)                                          \
   if constexpr (NCORN * NP == 4) {                                            \
-    if (!ring) MCX_LAUNCH_NA(NCORN, NP, CL, 2, pair_mask, 1);                 \
-    MCX_LAUNCH_NA(NCORN, NP, CL, NCORN * NP, pair_mask, 0);                   \
+    if (!ring) {                                                              \
+      MCX_LAUNCH_NA(NCORN, NP, CL, 2, pair_mask, 1);                          \
+      MCX_LAUNCH_NA(NCORN, NP, CL, NCORN * NP, pair_mask, 0);                 \
+    }                                                                         \
   } else {                                                                    \
     MCX_LAUNCH_NA(NCORN, NP, CL, NCORN * NP, (const int *)nullptr, 0);        \
   }
@@ -2055,21 +2102,25 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
   if constexpr (sizeof(TD) == 2) {
     if (ring) {
       TD *stage = reinterpret_cast<TD *>((char *)pair_mask_ws + 256);
-      if (int rc = launch_channel_blocks<TD>(gath, stage, B, G, GH * GW, s, pair_mask)) return rc;
+      if (int rc = launch_channel_blocks<TD>(gath, stage, B, G, GH * GW, s)) return rc;
     }
   }
   profile_begin(s);
   if constexpr (sizeof(TD) == 2) {
     if (ring) {
       const int rg_groups = (int)((G + kRgG - 1) / kRgG), rg_passes = (int)((K + kRgKT - 1) / kRgKT);
-      hipLaunchKernelGGL(weight_grad_bf16_ring_kernel,
-                         dim3((unsigned)(ranges * rg_groups * rg_passes),
-                              (unsigned)((A + kRgA - 1) / kRgA)),
-                         dim3(kThreads), 0, s, plain,
-                         reinterpret_cast<const TD *>((char *)pair_mask_ws + 256), map, part,
-                         (int)A, (int)G, (int)Gpad, (int)GH, (int)GW, (int)MH, (int)MW, (int)K,
-                         m.wrap, t.tiles_x, t.tiles_per_img, t.tw_shift, (int)t.total, ranges,
-                         rg_groups, rg_passes, plain_sum ? sum_part : (float *)nullptr, pair_mask);
+#define MCX_LAUNCH_RING(NA)                                                                       \
+  hipLaunchKernelGGL(weight_grad_bf16_ring_kernel<NA>,                                            \
+                     dim3((unsigned)(ranges * rg_groups * rg_passes),                             \
+                          (unsigned)((A + kRgA - 1) / kRgA)),                                     \
+                     dim3(kThreads), 0, s, plain,                                                 \
+                     reinterpret_cast<const TD *>((char *)pair_mask_ws + 256), map, part, (int)A, \
+                     (int)G, (int)Gpad, (int)GH, (int)GW, (int)MH, (int)MW, (int)K, m.wrap,       \
+                     t.tiles_x, t.tiles_per_img, t.tw_shift, (int)t.total, ranges, rg_groups,     \
+                     rg_passes, plain_sum ? sum_part : (float *)nullptr, pair_mask)
+      MCX_LAUNCH_RING(2);
+      MCX_LAUNCH_RING(4);
+#undef MCX_LAUNCH_RING
       MCX_HIP_CHECK_LAUNCH();
     }
   }

@@ -234,13 +234,15 @@ def test_input_gradient_with_border_rows_beyond_two_entries(with_plan, dtype, de
 
 
 @pytest.mark.parametrize("interp", [1, 2])
+@pytest.mark.parametrize("row_shift", [0.0, 0.37])
 @pytest.mark.parametrize("shape", [(4, 130, 96, 40, 392, 2), (2, 72, 200, 33, 264, 1),
                                    (3, 128, 128, 16, 1024, 2)])
-def test_bf16_weight_gradient_over_many_tiles_per_workgroup(shape, interp, device):
-    """bf16 storage under a latitude map (integral rows): the weight gradient's workgroups walk
-    runs of several row tiles with their gathers in flight across tile boundaries, runs that are
-    padded to a whole number of ring periods, ragged channel counts on both sides, rows that end
-    inside a tile, 9 and 25 taps (passes of 5 + 4 and 5 x 5).  Checked against the fp32 kernels on
+def test_bf16_weight_gradient_over_many_tiles_per_workgroup(shape, row_shift, interp, device):
+    """bf16 storage under a latitude map, with integral rows (two pairs per tap) and with the
+    rows shifted by a fraction (all four): the weight gradient's workgroups walk runs of several
+    row tiles (with two pairs: their gathers in flight across tile boundaries, runs padded to a
+    whole number of ring periods), ragged channel counts on both sides, rows that end inside a
+    tile, 9 and 25 taps (passes of 5 + 4 and 5 x 5).  Checked against the fp32 kernels on
     the same bf16-valued inputs (themselves checked against the oracle), which differ by the
     rounding of the samples to bf16 only; the oracle itself runs on the small cases elsewhere in
     this file and on sampled positions at full size."""
@@ -251,7 +253,9 @@ def test_bf16_weight_gradient_over_many_tiles_per_workgroup(shape, interp, devic
     gy = torch.randn(B, Co, H, W, generator=g).bfloat16().cuda()
     w = (torch.randn(Co, Ci, K, generator=g) / (Ci * K) ** 0.5).bfloat16().cuda()
     b = torch.randn(Co, generator=g).bfloat16().cuda()
-    smap = synthetic.latitude_map(H, W, radius).cuda()
+    smap = synthetic.latitude_map(H, W, radius)
+    smap[..., 1] = (smap[..., 1] + row_shift).clamp(0, H - 1)
+    smap = smap.cuda()
     got = _C.mapped_conv_backward(gy, smap, x, w, b, K, interp)
     ref = _C.mapped_conv_backward(gy.float(), smap, x.float(), w.float(), b.float(), K, interp)
     for a, r, nm in zip(got, ref, ("grad_input", "grad_weight", "grad_bias")):
@@ -283,6 +287,29 @@ def test_bf16_transposed_conv_under_a_map_with_integral_rows(with_plan, interp, 
     y = _C.mapped_transposed_conv_forward(xd, sd, wd_, bd, H, W, K, interp, plan=plan)
     gr = _C.mapped_transposed_conv_backward(gyd, sd, xd, wd_, bd, K, interp, plan=plan)
     assert rel_err(y.float(), y_o) < 2e-2
+    for a, r, nm in zip(gr, g_o, ("grad_input", "grad_weight", "grad_bias")):
+        assert rel_err(a.float(), r) < 2e-2, nm
+    assert_close_elementwise(gr[1].float(), g_o[1], 2e-2, "grad_weight")
+
+
+@pytest.mark.parametrize("interp", [1, 2])
+@pytest.mark.parametrize("radius", [1, 2])
+def test_bf16_backward_under_a_map_with_fractional_rows(radius, interp, device):
+    """bf16 storage, rows of the latitude map shifted by a fraction so that all four corners of
+    every tap weigh something, image rows a multiple of 8 pixels: the weight gradient's
+    four-pair form on the 8-channel block copy, against the oracle."""
+    B, Ci, Co, H, W = 2, 24, 40, 14, 136
+    K = (2 * radius + 1) ** 2
+    g = torch.Generator().manual_seed(321 + radius)
+    bf = lambda t: t.to(torch.bfloat16)
+    x, gy = bf(torch.randn(B, Ci, H, W, generator=g)), bf(torch.randn(B, Co, H, W, generator=g))
+    w = bf(torch.randn(Co, Ci, K, generator=g) / (Ci * K) ** 0.5)
+    b = bf(torch.randn(Co, generator=g))
+    smap = synthetic.latitude_map(H, W, radius)
+    smap[..., 1] = (smap[..., 1] + 0.37).clamp(0, H - 1)
+    g_o = O.mapped_conv_backward(gy.float(), smap, x.float(), w.float(), b.float(), K, interp)
+    xd, sd, wd_, bd, gyd = dev(x, smap, w, b, gy)
+    gr = _C.mapped_conv_backward(gyd, sd, xd, wd_, bd, K, interp)
     for a, r, nm in zip(gr, g_o, ("grad_input", "grad_weight", "grad_bias")):
         assert rel_err(a.float(), r) < 2e-2, nm
     assert_close_elementwise(gr[1].float(), g_o[1], 2e-2, "grad_weight")
