@@ -187,9 +187,13 @@ __global__ void cube_projection_map_kernel(float *__restrict__ out, int dim, int
 // pixel's face coordinates.
 constexpr int kCubeChannels = 16;
 
-template <typename T>
+// BILINEAR is a template parameter and every load unconditional (a corner outside the image
+// reads element 0 and is replaced by zero afterwards), four channels at a time: with the loads
+// behind per-lane tests and a run-time corner count each one was waited for on its own
+// (bilinear 0.158 ms for 64 channels onto 512 x 1024).
+template <typename T, bool BILINEAR>
 __global__ void cube2rect_kernel(const T *__restrict__ cube, T *__restrict__ rect, int C, int dim,
-                                 int RH, int RW, int bilinear) {
+                                 int RH, int RW) {
   const int64_t px = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (px >= (int64_t)RH * RW) return;
   const int xr = (int)(px % RW), yr = (int)(px / RW);
@@ -218,10 +222,10 @@ __global__ void cube2rect_kernel(const T *__restrict__ cube, T *__restrict__ rec
   const int width = 6 * dim;
   const int64_t plane = (int64_t)dim * width, start = (int64_t)face * dim;
   const int64_t limit = (int64_t)C * plane;  // elements in the whole cube map
-  int64_t off[4];
-  T wt[4];
-  int n;
-  if (bilinear) {
+  constexpr int NQ = BILINEAR ? 4 : 1;
+  int64_t off[NQ];
+  T wt[NQ];
+  if constexpr (BILINEAR) {
     const T x1f = mcx_floor(u), y1f = mcx_floor(v);
     const int x1 = to_int(x1f), y1 = to_int(y1f), x2 = x1 + 1, y2 = y1 + 1;
     const bool x1ok = x1 >= 0 && x1 <= width - 1, x2ok = x2 >= 0 && x2 <= width - 1;
@@ -232,27 +236,37 @@ __global__ void cube2rect_kernel(const T *__restrict__ cube, T *__restrict__ rec
     off[1] = x2ok && y1ok ? start + (int64_t)y1 * width + x2 : -1;
     off[2] = x1ok && y2ok ? start + (int64_t)y2 * width + x1 : -1;
     off[3] = x2ok && y2ok ? start + (int64_t)y2 * width + x2 : -1;
-    n = 4;
   } else {
     const int xi = to_int(round_half_away(u)), yi = to_int(round_half_away(v));
     const bool ok = xi >= 0 && xi <= width - 1 && yi >= 0 && yi <= dim - 1;
     wt[0] = T(1);
     off[0] = ok ? start + (int64_t)yi * width + xi : -1;
-    n = 1;
   }
   const int c0 = blockIdx.y * kCubeChannels, c1 = min(c0 + kCubeChannels, C);
-#pragma unroll 4
-  for (int c = c0; c < c1; c++) {
-    const int64_t base = (int64_t)c * plane;
-    T d[4];
-    for (int q = 0; q < n; q++)  // never read past the end of the buffer
-      d[q] = (off[q] >= 0 && base + off[q] < limit) ? cube[base + off[q]] : T(0);
-    T r;
-    if (bilinear)
-      r = wt[0] * d[0] + wt[1] * d[1] + wt[2] * d[2] + wt[3] * d[3];
-    else
-      r = d[0];
-    rect[(int64_t)c * RH * RW + px] = r;
+  constexpr int kStep = 4;
+  for (int cb = c0; cb < c1; cb += kStep) {
+    T d[kStep][NQ];
+    bool ok[kStep][NQ];
+#pragma unroll
+    for (int i = 0; i < kStep; i++) {
+      const int64_t base = (int64_t)min(cb + i, c1 - 1) * plane;
+#pragma unroll
+      for (int q = 0; q < NQ; q++) {  // never read past the end of the buffer
+        ok[i][q] = off[q] >= 0 && base + off[q] < limit;
+        d[i][q] = cube[ok[i][q] ? base + off[q] : 0];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kStep; i++) {
+#pragma unroll
+      for (int q = 0; q < NQ; q++) d[i][q] = ok[i][q] ? d[i][q] : T(0);
+      T r;
+      if constexpr (BILINEAR)
+        r = wt[0] * d[i][0] + wt[1] * d[i][1] + wt[2] * d[i][2] + wt[3] * d[i][3];
+      else
+        r = d[i][0];
+      if (cb + i < c1) rect[(int64_t)(cb + i) * RH * RW + px] = r;
+    }
   }
 }
 
@@ -307,15 +321,16 @@ int mcx_cube2rect(const void *cubemap, void *rect, int64_t C, int64_t cube_dim, 
     return MCX_E_SHAPE;
   if (C > 65535LL * kCubeChannels) return MCX_E_SHAPE;
   const dim3 grid(div_up(RH * RW, 256), div_up(C, kCubeChannels));
-  const int bilinear = interp == 1;  // cube2rect.cuh:49-61: everything else is nearest
-  if (dtype == MCX_F32)
-    hipLaunchKernelGGL(cube2rect_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream,
-                       (const float *)cubemap, (float *)rect, (int)C, (int)cube_dim, (int)RH,
-                       (int)RW, bilinear);
-  else
-    hipLaunchKernelGGL(cube2rect_kernel<double>, grid, dim3(256), 0, (hipStream_t)stream,
-                       (const double *)cubemap, (double *)rect, (int)C, (int)cube_dim, (int)RH,
-                       (int)RW, bilinear);
+  const bool bilinear = interp == 1;  // cube2rect.cuh:49-61: everything else is nearest
+#define MCX_LAUNCH_C2R(T, BIL)                                                                  \
+  hipLaunchKernelGGL((cube2rect_kernel<T, BIL>), grid, dim3(256), 0, (hipStream_t)stream,       \
+                     (const T *)cubemap, (T *)rect, (int)C, (int)cube_dim, (int)RH, (int)RW)
+  if (dtype == MCX_F32) {
+    if (bilinear) MCX_LAUNCH_C2R(float, true); else MCX_LAUNCH_C2R(float, false);
+  } else {
+    if (bilinear) MCX_LAUNCH_C2R(double, true); else MCX_LAUNCH_C2R(double, false);
+  }
+#undef MCX_LAUNCH_C2R
   MCX_HIP_CHECK_LAUNCH();
   return 0;
 }
