@@ -315,6 +315,31 @@ def test_bf16_backward_under_a_map_with_fractional_rows(radius, interp, device):
     assert_close_elementwise(gr[1].float(), g_o[1], 2e-2, "grad_weight")
 
 
+@pytest.mark.parametrize("row_shift", [0.0, 0.5])
+@pytest.mark.parametrize("shape", [(1, 3, 5, 6, 16), (2, 1, 2, 3, 8), (1, 9, 17, 5, 264)])
+def test_bf16_backward_with_very_few_channels(shape, row_shift, device):
+    """bf16 storage, rows a multiple of 8 pixels, fewer channels than one 8-channel block or one
+    MFMA tile on either side, images of a few rows: the block copy's padding channels and the
+    workgroups' idle channel groups must add nothing.  Against the oracle."""
+    B, Ci, Co, H, W = shape
+    K = 9
+    g = torch.Generator().manual_seed(7 + Ci)
+    bf = lambda t: t.to(torch.bfloat16)
+    x, gy = bf(torch.randn(B, Ci, H, W, generator=g)), bf(torch.randn(B, Co, H, W, generator=g))
+    w = bf(torch.randn(Co, Ci, K, generator=g) / (Ci * K) ** 0.5)
+    b = bf(torch.randn(Co, generator=g))
+    smap = synthetic.latitude_map(H, W, 1)
+    smap[..., 1] = (smap[..., 1] + row_shift).clamp(0, H - 1)
+    y_o = O.mapped_conv_forward(x.float(), smap, w.float(), b.float(), K, 1)
+    g_o = O.mapped_conv_backward(gy.float(), smap, x.float(), w.float(), b.float(), K, 1)
+    xd, sd, wd_, bd, gyd = dev(x, smap, w, b, gy)
+    y = _C.mapped_conv_forward(xd, sd, wd_, bd, K, 1)
+    gr = _C.mapped_conv_backward(gyd, sd, xd, wd_, bd, K, 1)
+    assert rel_err(y.float(), y_o) < 2e-2
+    for a, r, nm in zip(gr, g_o, ("grad_input", "grad_weight", "grad_bias")):
+        assert rel_err(a.float(), r) < 2e-2, nm
+
+
 def test_bf16_with_more_than_four_points_is_rejected(device):
     """bf16 storage exists on the matrix-core kernels only, which take at most four points."""
     g = torch.Generator().manual_seed(5)
