@@ -578,6 +578,30 @@ def test_pools_with_more_channels_than_one_thread_takes(interp, device):
                    O.mapped_max_unpool(gy, mi, lmap, H, W, K, interp)) < 1e-5
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("interp", [0, 1, 2])
+@pytest.mark.parametrize("K", [10, 18, 25, 28])
+def test_pools_with_more_than_nine_taps(K, interp, dtype, device):
+    """Pooling maps of more than nine taps run nine taps at a time, every pass continuing from
+    the sum or the winner the pass before left in the output: values, argmax and averages must
+    still be those of one pass over all taps in order, bit for bit - also where every tap of a
+    pixel lies outside the image (zeros, the first tap wins) and where one large value wins."""
+    g = torch.Generator().manual_seed(700 + K + interp)
+    B, C, IH, IW, OH, OW = 2, 5, 9, 40, 7, 33
+    x = torch.randn(B, C, IH, IW, generator=g, dtype=torch.float64).to(dtype)
+    smap, _ = helpers.random_map(g, OH, OW, K, 0, IH, IW, dtype)
+    smap[0, :3] = -7.0          # pixels all of whose taps lie outside
+    x[:, :, 0, 0] = 50.0        # a value that wins wherever it is sampled
+    xd, sd = dev(x, smap)
+    mo, mi = O.mapped_max_pool(x, smap, K, interp)
+    ao = O.mapped_avg_pool(x, smap, K, interp)
+    m, i = _C.mapped_max_pool(xd, sd, K, interp)
+    a = _C.mapped_avg_pool(xd, sd, K, interp)
+    assert torch.equal(m.cpu(), mo), "max-pool values must be bit-exact"
+    assert torch.equal(i.cpu(), mi), "max-pool argmax must be bit-exact"
+    assert torch.equal(a.cpu(), ao), "avg-pool gather must be bit-exact"
+
+
 @pytest.mark.parametrize("radius,interp", [(1, 1), (2, 0), (2, 1)])
 def test_unpool_list_lengths_for_both_sorting_networks(radius, interp, device):
     """Unpooling through latitude maps whose per-pixel contribution lists are 9 to 16 entries
