@@ -602,13 +602,13 @@ def test_pools_with_more_than_nine_taps(K, interp, dtype, device):
     assert torch.equal(a.cpu(), ao), "avg-pool gather must be bit-exact"
 
 
-@pytest.mark.parametrize("radius,interp", [(1, 1), (2, 0), (2, 1)])
+@pytest.mark.parametrize("radius,interp", [(1, 1), (2, 0), (2, 1), (3, 1)])
 def test_unpool_list_lengths_for_both_sorting_networks(radius, interp, device):
     """Unpooling through latitude maps whose per-pixel contribution lists are 9 to 16 entries
     long (3x3 bilinear: the 16-key sorting network) and 17 to 32 (5x5 nearest: 25 entries,
     the 32-key network) or longer (5x5 bilinear: 50 - sorted by rank, a lane per entry, and
-    gathered in passes of 24 entries that continue from the destination): same values as the
-    oracle, and the same bits on every call."""
+    gathered in passes of 24 entries that continue from the destination; 7x7 bilinear: 98, the
+    insertion sort and five passes): same values as the oracle, and the same bits on every call."""
     B, C, H, W = 2, 3, 24, 128
     K = (2 * radius + 1) ** 2
     g = torch.Generator().manual_seed(40 + radius + interp)
