@@ -35,7 +35,7 @@ TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "conv_fwd_bwd_headline_hbm_traf
 def recorded_traffic():
     """Kernel name and bytes crossing the L2 boundary per launch, per timed C-ABI call, from the
     committed counter summary (FETCH_SIZE / WRITE_SIZE passes of this script, scaled by copy
-    dispatches of known size; mappedconvolutions_amd/traffic_summary.py writes it).  Counters
+    dispatches of known size; bench_traffic_summary.py writes it).  Counters
     cannot be read from inside the process, so these are recorded figures: they are dropped when
     the kernel source has changed since the counter run."""
     import hashlib

@@ -1,7 +1,7 @@
 """Turns two rocprofv3 counter passes of `bench.py --calibration-copy` into the memory-traffic
 summary that `bench.py` reads its `roofline.traffic` figure from.
 
-    python -m mappedconvolutions_amd.traffic_summary FETCH_DIR WRITE_DIR > summary.txt
+    python bench_traffic_summary.py FETCH_DIR WRITE_DIR > summary.txt
 
 FETCH_DIR / WRITE_DIR: output folders of
     rocprofv3 --pmc FETCH_SIZE --output-format csv -d FETCH_DIR -o run -- \
@@ -20,7 +20,7 @@ import os
 import re
 import sys
 
-ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ROOT = os.path.dirname(os.path.abspath(__file__))
 KERNEL_SOURCE = "mappedconvolutions_amd/csrc/mcx_conv_mfma.hip"
 COPY_BYTES = 8 * 64 * 256 * 512 * 4  # one calibration dispatch reads and writes the input once
 

@@ -48,7 +48,8 @@ enum {
   MCX_E_SHAPE = -2,     /* a size is negative, zero where it may not be, or too large */
   MCX_E_NULL = -3,      /* a required pointer is NULL (or iw/P disagree) */
   MCX_E_WORKSPACE = -4, /* workspace missing or too small */
-  MCX_E_STATIC_LIMIT = -5 /* needs more scratch than mcx_conv_forward_static's fixed buffer */
+  MCX_E_STATIC_LIMIT = -5, /* needs more scratch than mcx_conv_forward_static's fixed buffer */
+  MCX_E_PLAN = -6 /* the plan was not built for this op, map, interpolation or size */
 };
 
 /* Library identification; bumps when a signature changes. */
@@ -202,6 +203,40 @@ int mcx_tconv_backward(const void *gy, const void *map, const void *iw, const vo
                        int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
                        int dtype, void *stream);
 
+/* ---- Map plans ---------------------------------------------------------------- */
+
+/* A plan is device memory the caller owns; what it was built for is recorded on the HOST, in a
+ * descriptor the *_plan_build call fills and the caller hands back with the plan.  Every
+ * *_planned entry point compares the descriptor with its own arguments before it enqueues
+ * anything - the operation the plan serves, interpolation (as the library canonicalises it),
+ * sizes, K, P, the data type where the plan depends on it, the address and size of the plan
+ * and, where the entry point also takes the map, the addresses of sample_map and
+ * interp_weights the plan was built from - and returns MCX_E_PLAN on any difference, so a plan
+ * of equal size built for another map or another interpolation cannot be used by mistake.  The
+ * descriptor is plain data (no pointers are followed); `check` folds the other fields so that an
+ * uninitialised or edited descriptor is refused too.  A plan is bound to the buffers it was
+ * built at and from: after copying a plan or a map elsewhere, build again.  The library cannot
+ * see writes into the map: rebuild the plan when the map's contents change. */
+enum {
+  MCX_PLAN_CONV = 1,        /* mcx_conv_plan_build */
+  MCX_PLAN_SCATTER = 2,     /* mcx_scatter_plan_build, for_max_unpool == 0 */
+  MCX_PLAN_SCATTER_MAX = 3, /* mcx_scatter_plan_build, for_max_unpool != 0 */
+  MCX_PLAN_POOL = 4         /* mcx_pool_plan_build */
+};
+typedef struct mcx_plan_desc {
+  uint32_t magic;    /* 0x4d435850 */
+  int32_t kind;      /* MCX_PLAN_* */
+  int32_t interp;    /* 0 nearest, 1 bilinear, 2 bispherical */
+  int32_t dtype;     /* MCX_F32 / MCX_F64 for plans that hold weights in the data's type; conv: MCX_F32 */
+  int64_t SH, SW;    /* the image the map points into */
+  int64_t MH, MW;    /* the map's spatial size */
+  int64_t K, P;
+  uint64_t plan;     /* device address the plan was built at */
+  uint64_t plan_bytes;
+  uint64_t map, iw;  /* device addresses of sample_map and interp_weights (0: none) */
+  uint64_t check;
+} mcx_plan_desc;
+
 /* Map plan: no counterpart in the reference, which decodes sample_map inside its kernels at
  * every call.  A network applies the same sample_map at every step, so everything that depends
  * on the map alone can be built once and reused: the transposed map of the scatter direction
@@ -219,11 +254,12 @@ int mcx_tconv_backward(const void *gy, const void *map, const void *iw, const vo
 size_t mcx_conv_plan_bytes(int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P,
                            int dtype);
 int mcx_conv_plan_build(const void *map, const void *iw, void *plan, size_t plan_bytes,
-                        int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P,
+                        mcx_plan_desc *desc, int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P,
                         int interp, int dtype, void *stream);
 int mcx_conv_backward_planned(const void *gy, const void *map, const void *iw, const void *x,
                               const void *w, void *gx, void *gw, void *gb, void *workspace,
                               size_t workspace_bytes, const void *plan, size_t plan_bytes,
+                               const mcx_plan_desc *desc,
                               int64_t B, int64_t Ci, int64_t Co, int64_t IH, int64_t IW,
                               int64_t OH, int64_t OW, int64_t K, int64_t P, int interp, int dtype,
                               void *stream);
@@ -240,32 +276,37 @@ int mcx_conv_backward_planned(const void *gy, const void *map, const void *iw, c
 size_t mcx_scatter_plan_bytes(int64_t MH, int64_t MW, int64_t DH, int64_t DW, int64_t K, int64_t P,
                               int interp, int dtype);
 int mcx_scatter_plan_build(const void *map, const void *iw, void *plan, size_t plan_bytes,
-                           int64_t MH, int64_t MW, int64_t DH, int64_t DW, int64_t K, int64_t P,
+                           mcx_plan_desc *desc, int64_t MH, int64_t MW, int64_t DH, int64_t DW, int64_t K, int64_t P,
                            int interp, int dtype, int for_max_unpool, void *stream);
-int mcx_resample_to_map_planned(const void *in, const void *plan, size_t plan_bytes, void *out,
+int mcx_resample_to_map_planned(const void *in, const void *plan, size_t plan_bytes,
+                                const mcx_plan_desc *desc, void *out,
                                 int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t OH,
                                 int64_t OW, int64_t P, int interp, int dtype, void *stream);
-int mcx_avg_unpool_planned(const void *gout, const void *plan, size_t plan_bytes, void *gin,
+int mcx_avg_unpool_planned(const void *gout, const void *plan, size_t plan_bytes,
+                           const mcx_plan_desc *desc, void *gin,
                            int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t OH, int64_t OW,
                            int64_t K, int64_t P, int interp, int dtype, void *stream);
 int mcx_max_unpool_planned(const void *gout, const int64_t *idx, const void *plan,
-                           size_t plan_bytes, void *gin, int64_t B, int64_t C, int64_t IH,
+                           size_t plan_bytes, const mcx_plan_desc *desc, void *gin, int64_t B, int64_t C, int64_t IH,
                            int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
                            int dtype, void *stream);
 
 int mcx_conv_forward_planned(const void *x, const void *map, const void *iw, const void *w,
                              const void *bias, void *y, void *workspace, size_t workspace_bytes,
-                             const void *plan, size_t plan_bytes, int64_t B, int64_t Ci,
+                             const void *plan, size_t plan_bytes, const mcx_plan_desc *desc,
+                              int64_t B, int64_t Ci,
                              int64_t Co, int64_t IH, int64_t IW, int64_t OH, int64_t OW,
                              int64_t K, int64_t P, int interp, int dtype, void *stream);
 int mcx_tconv_forward_planned(const void *x, const void *map, const void *iw, const void *w,
                               const void *bias, void *y, void *workspace, size_t workspace_bytes,
-                              const void *plan, size_t plan_bytes, int64_t B, int64_t Ci,
+                              const void *plan, size_t plan_bytes, const mcx_plan_desc *desc,
+                              int64_t B, int64_t Ci,
                               int64_t Co, int64_t IH, int64_t IW, int64_t OH, int64_t OW,
                               int64_t K, int64_t P, int interp, int dtype, void *stream);
 int mcx_tconv_backward_planned(const void *gy, const void *map, const void *iw, const void *x,
                                const void *w, void *gx, void *gw, void *gb, void *workspace,
                                size_t workspace_bytes, const void *plan, size_t plan_bytes,
+                               const mcx_plan_desc *desc,
                                int64_t B, int64_t Ci, int64_t Co, int64_t IH, int64_t IW,
                                int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
                                int dtype, void *stream);
@@ -323,6 +364,14 @@ int mcx_cube2rect(const void *cubemap, void *rect, int64_t C, int64_t cube_dim, 
                   int64_t RW, int interp, int dtype, void *stream);
 
 /* ---- icosphere map operators -------------------------------------------------- */
+
+/* gnomonic_kernel: package/layers/util/icosphere_functions.py:135-183.  A kh x kw grid of
+ * spacing (res_lon, res_lat) on the plane tangent to the unit sphere at each of V points
+ * centres [V, 2] = (longitude, latitude) in radians, carried back onto the sphere:
+ * out [V, kh*kw, 2] = (longitude in [-pi, pi), latitude).  The tap of index
+ * (kh/2)*kw + kw/2 is the centre itself.  Entries are evaluated in double and rounded once. */
+int mcx_gnomonic_samples(const float *centres, float *out, int64_t V, int64_t kh, int64_t kw,
+                         double res_lat, double res_lon, void *stream);
 
 /* get_planar_conv_operator_from_samples: package/ext_modules/include/util/cpp/sphere.h:131-175
  * (binding), package/ext_modules/src/util/cpp/sphere.cpp:1117-1270 (driver), :1055-1105

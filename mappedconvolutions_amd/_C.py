@@ -136,12 +136,12 @@ def _conv_forward(input, sample_map, interp_weights, weight, bias, kernel_size, 
     ws = _workspace(ws_bytes, input.device)
     if plan is None and map_plan_cache is not None:
         plan = _cached_plan(sample_map, interp_weights, IH, IW, interpolation, input.dtype)
-    plan_bytes = 0 if plan is None else plan.numel()
+    plan_ptr, plan_bytes, plan_desc = _plan_args(plan)
     with torch.cuda.device(input.device):
         rc = _timed("conv_forward", input.device, lambda: lib.mcx_conv_forward_planned(
             _ptr(input), _ptr(sample_map), _ptr(interp_weights), _ptr(weight), _ptr(bias),
-            _ptr(out), _ptr(ws), ws_bytes, _ptr(plan), plan_bytes, B, Ci, Co, IH, IW, OH, OW, K,
-            P, int(interpolation), dt, _stream(input)))
+            _ptr(out), _ptr(ws), ws_bytes, plan_ptr, plan_bytes, plan_desc, B, Ci, Co, IH, IW, OH,
+            OW, K, P, int(interpolation), dt, _stream(input)))
     _lib.check(rc, "mapped_conv_forward")
     return out
 
@@ -157,6 +157,30 @@ def _conv_forward(input, sample_map, interp_weights, weight, bias, kernel_size, 
 # what it needs, like the reference.
 map_plan_cache = None
 _MAP_PLAN_CACHE_ENTRIES = 16
+
+
+class MapPlan:
+    """A map plan: the device buffer, the host-side descriptor the library checks it by
+    (mcx_plan_desc: op family, interpolation, sizes, the addresses of the plan and of the map it
+    was built from) and the map tensors themselves, kept alive so that their addresses cannot
+    pass to other tensors while the plan exists."""
+    __slots__ = ("buffer", "desc", "tensors")
+
+    def __init__(self, buffer, desc, tensors):
+        self.buffer, self.desc, self.tensors = buffer, desc, tensors
+
+    def numel(self):
+        return self.buffer.numel()
+
+
+def _plan_args(plan):
+    """(device pointer, bytes, descriptor) of a MapPlan for the C ABI; NULLs for None."""
+    if plan is None:
+        return None, 0, None
+    if not isinstance(plan, MapPlan):
+        raise RuntimeError("plan must come from conv_map_plan / scatter_map_plan / pool_map_plan")
+    import ctypes
+    return plan.buffer.data_ptr(), plan.buffer.numel(), ctypes.byref(plan.desc)
 
 
 def enable_map_plan_cache(enabled=True):
@@ -186,12 +210,13 @@ def conv_map_plan(sample_map, interp_weights, input_height, input_width, interpo
     if nbytes == 0:
         return None
     plan = torch.empty((nbytes,), dtype=torch.uint8, device=sample_map.device)
+    desc = _lib.PlanDesc()
     with torch.cuda.device(sample_map.device):
         rc = lib.mcx_conv_plan_build(_ptr(sample_map), _ptr(interp_weights), _ptr(plan), nbytes,
-                                     IH, IW, OH, OW, K, P, int(interpolation), dt,
+                                     desc, IH, IW, OH, OW, K, P, int(interpolation), dt,
                                      _stream(sample_map))
     _lib.check(rc, "conv_map_plan")
-    return plan
+    return MapPlan(plan, desc, (sample_map, interp_weights))
 
 
 def _cached_plan(sample_map, interp_weights, IH, IW, interpolation, data_dtype, kind="conv",
@@ -217,7 +242,7 @@ def _cached_plan(sample_map, interp_weights, IH, IW, interpolation, data_dtype, 
 
 
 def _conv_backward(grad_output, sample_map, interp_weights, input, weight, bias, kernel_size,
-                   interpolation, plan=None):
+                   interpolation, plan=None, needs=(True, True, True)):
     _contig(input=input, sample_map=sample_map, interp_weights=interp_weights, weight=weight,
             bias=bias)
     grad_output = grad_output.contiguous()  # the reference reads it raw without a check
@@ -230,15 +255,17 @@ def _conv_backward(grad_output, sample_map, interp_weights, input, weight, bias,
     K = int(kernel_size)
     if tuple(weight.shape) != (Co, Ci, K) or tuple(sample_map.shape[:3]) != (OH, OW, K):
         raise RuntimeError("shape mismatch in mapped_conv_backward")
-    grad_input = torch.empty_like(input)
-    grad_weight = torch.empty_like(weight)
-    grad_bias = torch.empty((Co,), dtype=input.dtype, device=input.device)
+    # `needs` (grad_input, grad_weight, grad_bias): a gradient nobody asked for is not
+    # computed (the C ABI takes NULL for it) and comes back as None
+    grad_input = torch.empty_like(input) if needs[0] else None
+    grad_weight = torch.empty_like(weight) if needs[1] else None
+    grad_bias = torch.empty((Co,), dtype=input.dtype, device=input.device) if needs[2] else None
     lib = _lib.load()
     ws_bytes = lib.mcx_conv_backward_workspace(B, Ci, Co, IH, IW, OH, OW, K, P, dt)
     ws = _workspace(ws_bytes, input.device)
     if plan is None and map_plan_cache is not None:
         plan = _cached_plan(sample_map, interp_weights, IH, IW, interpolation, input.dtype)
-    plan_bytes = 0 if plan is None else plan.numel()
+    plan_ptr, plan_bytes, plan_desc = _plan_args(plan)
     # Two C-ABI calls (NULL skips a gradient) so that the input gradient and the weight
     # gradient can be timed alone; the bias gradient rides on the weight gradient's pass
     # over grad_output.
@@ -246,10 +273,12 @@ def _conv_backward(grad_output, sample_map, interp_weights, input, weight, bias,
             "conv_backward_weight": (None, grad_weight, grad_bias)}
     with torch.cuda.device(input.device):
         for label, (gx, gw, gb) in outs.items():
+            if gx is None and gw is None and gb is None:
+                continue
             rc = _timed(label, input.device, lambda: lib.mcx_conv_backward_planned(
                 _ptr(grad_output), _ptr(sample_map), _ptr(interp_weights), _ptr(input),
-                _ptr(weight), _ptr(gx), _ptr(gw), _ptr(gb), _ptr(ws), ws_bytes, _ptr(plan),
-                plan_bytes, B, Ci, Co, IH, IW, OH, OW, K, P, int(interpolation), dt,
+                _ptr(weight), _ptr(gx), _ptr(gw), _ptr(gb), _ptr(ws), ws_bytes, plan_ptr,
+                plan_bytes, plan_desc, B, Ci, Co, IH, IW, OH, OW, K, P, int(interpolation), dt,
                 _stream(input)))
             _lib.check(rc, "mapped_conv_backward")
     return [grad_input, grad_weight, grad_bias]
@@ -262,11 +291,12 @@ def mapped_conv_forward(input, sample_map, weight, bias, kernel_size, interpolat
 
 
 def mapped_conv_backward(grad_output, sample_map, input, weight, bias, kernel_size, interpolation,
-                         plan=None):
+                         plan=None, needs=(True, True, True)):
     """include/nn/layers/mapped_convolution_layer.h:90-93 -> [grad_input, grad_weight, grad_bias].
-    `plan` (optional, not in the reference): see conv_map_plan."""
+    `plan` (optional, not in the reference): see conv_map_plan.  `needs` (optional, not in the
+    reference): which of the three gradients to compute; the others come back as None."""
     return _conv_backward(grad_output, sample_map, None, input, weight, bias, kernel_size,
-                          interpolation, plan)
+                          interpolation, plan, needs)
 
 
 def weighted_mapped_conv_forward(input, sample_map, interp_weights, weight, bias, kernel_size,
@@ -277,10 +307,12 @@ def weighted_mapped_conv_forward(input, sample_map, interp_weights, weight, bias
 
 
 def weighted_mapped_conv_backward(grad_output, sample_map, interp_weights, input, weight, bias,
-                                  kernel_size, interpolation, plan=None):
-    """include/nn/layers/weighted_mapped_convolution_layer.h:97-100.  `plan`: see conv_map_plan."""
+                                  kernel_size, interpolation, plan=None,
+                                  needs=(True, True, True)):
+    """include/nn/layers/weighted_mapped_convolution_layer.h:97-100.  `plan`: see conv_map_plan;
+    `needs`: see mapped_conv_backward."""
     return _conv_backward(grad_output, sample_map, interp_weights, input, weight, bias,
-                          kernel_size, interpolation, plan)
+                          kernel_size, interpolation, plan, needs)
 
 
 # ---------------------------------------------------------------- transposed conv
@@ -303,18 +335,19 @@ def _tconv_forward(input, sample_map, interp_weights, weight, bias, output_heigh
     ws = _workspace(ws_bytes, input.device)
     if plan is None and map_plan_cache is not None:
         plan = _cached_plan(sample_map, interp_weights, OH, OW, interpolation, input.dtype)
-    plan_bytes = 0 if plan is None else plan.numel()
+    plan_ptr, plan_bytes, plan_desc = _plan_args(plan)
     with torch.cuda.device(input.device):
         rc = lib.mcx_tconv_forward_planned(_ptr(input), _ptr(sample_map), _ptr(interp_weights),
                                            _ptr(weight), _ptr(bias), _ptr(out), _ptr(ws),
-                                           ws_bytes, _ptr(plan), plan_bytes, B, Ci, Co, IH, IW,
-                                           OH, OW, K, P, int(interpolation), dt, _stream(input))
+                                           ws_bytes, plan_ptr, plan_bytes, plan_desc, B, Ci, Co,
+                                           IH, IW, OH, OW, K, P, int(interpolation), dt,
+                                           _stream(input))
     _lib.check(rc, "mapped_transposed_conv_forward")
     return out
 
 
 def _tconv_backward(grad_output, sample_map, interp_weights, input, weight, bias, kernel_size,
-                    interpolation, plan=None):
+                    interpolation, plan=None, needs=(True, True, True)):
     _contig(input=input, sample_map=sample_map, interp_weights=interp_weights, weight=weight,
             bias=bias)
     grad_output = grad_output.contiguous()
@@ -327,20 +360,23 @@ def _tconv_backward(grad_output, sample_map, interp_weights, input, weight, bias
     K = int(kernel_size)
     if tuple(weight.shape) != (Ci, Co, K) or tuple(sample_map.shape[:3]) != (IH, IW, K):
         raise RuntimeError("shape mismatch in mapped_transposed_conv_backward")
-    grad_input = torch.empty_like(input)
-    grad_weight = torch.empty_like(weight)
-    grad_bias = torch.empty((Co,), dtype=input.dtype, device=input.device)
+    grad_input = torch.empty_like(input) if needs[0] else None
+    grad_weight = torch.empty_like(weight) if needs[1] else None
+    grad_bias = torch.empty((Co,), dtype=input.dtype, device=input.device) if needs[2] else None
+    if not any(needs):
+        return [None, None, None]
     lib = _lib.load()
     ws_bytes = lib.mcx_tconv_backward_workspace(B, Ci, Co, IH, IW, OH, OW, K, P, dt)
     ws = _workspace(ws_bytes, input.device)
     if plan is None and map_plan_cache is not None:
         plan = _cached_plan(sample_map, interp_weights, OH, OW, interpolation, input.dtype)
-    plan_bytes = 0 if plan is None else plan.numel()
+    plan_ptr, plan_bytes, plan_desc = _plan_args(plan)
     with torch.cuda.device(input.device):
         rc = lib.mcx_tconv_backward_planned(
             _ptr(grad_output), _ptr(sample_map), _ptr(interp_weights), _ptr(input), _ptr(weight),
-            _ptr(grad_input), _ptr(grad_weight), _ptr(grad_bias), _ptr(ws), ws_bytes, _ptr(plan),
-            plan_bytes, B, Ci, Co, IH, IW, OH, OW, K, P, int(interpolation), dt, _stream(input))
+            _ptr(grad_input), _ptr(grad_weight), _ptr(grad_bias), _ptr(ws), ws_bytes, plan_ptr,
+            plan_bytes, plan_desc, B, Ci, Co, IH, IW, OH, OW, K, P, int(interpolation), dt,
+            _stream(input))
     _lib.check(rc, "mapped_transposed_conv_backward")
     return [grad_input, grad_weight, grad_bias]
 
@@ -354,10 +390,11 @@ def mapped_transposed_conv_forward(input, sample_map, weight, bias, output_heigh
 
 
 def mapped_transposed_conv_backward(grad_output, sample_map, input, weight, bias, kernel_size,
-                                    interpolation, plan=None):
-    """include/nn/layers/mapped_transposed_convolution_layer.h:97-100."""
+                                    interpolation, plan=None, needs=(True, True, True)):
+    """include/nn/layers/mapped_transposed_convolution_layer.h:97-100.  `needs`: see
+    mapped_conv_backward."""
     return _tconv_backward(grad_output, sample_map, None, input, weight, bias, kernel_size,
-                           interpolation, plan)
+                           interpolation, plan, needs)
 
 
 def weighted_mapped_transposed_conv_forward(input, sample_map, interp_weights, weight, bias,
@@ -369,10 +406,11 @@ def weighted_mapped_transposed_conv_forward(input, sample_map, interp_weights, w
 
 
 def weighted_mapped_transposed_conv_backward(grad_output, sample_map, interp_weights, input,
-                                             weight, bias, kernel_size, interpolation, plan=None):
+                                             weight, bias, kernel_size, interpolation, plan=None,
+                                             needs=(True, True, True)):
     """include/nn/layers/weighted_mapped_transposed_convolution_layer.h:98-100."""
     return _tconv_backward(grad_output, sample_map, interp_weights, input, weight, bias,
-                           kernel_size, interpolation, plan)
+                           kernel_size, interpolation, plan, needs)
 
 
 def scatter_map_plan(sample_map, interp_weights, dest_height, dest_width, interpolation,
@@ -398,12 +436,13 @@ def scatter_map_plan(sample_map, interp_weights, dest_height, dest_width, interp
     if nbytes == 0:
         return None
     plan = torch.empty((nbytes,), dtype=torch.uint8, device=sample_map.device)
+    desc = _lib.PlanDesc()
     with torch.cuda.device(sample_map.device):
         rc = lib.mcx_scatter_plan_build(_ptr(sample_map), _ptr(interp_weights), _ptr(plan), nbytes,
-                                        MH, MW, DH, DW, K, P, int(interpolation), dt,
+                                        desc, MH, MW, DH, DW, K, P, int(interpolation), dt,
                                         1 if for_max_unpool else 0, _stream(sample_map))
     _lib.check(rc, "scatter_map_plan")
-    return plan
+    return MapPlan(plan, desc, (sample_map, interp_weights))
 
 
 def _scatter_plan_for(kind, plan, sample_map, interp_weights, DH, DW, interpolation, kernel):
@@ -462,8 +501,8 @@ def _max_unpool(grad_output, idx_mask, sample_map, interp_weights, input_height,
                              interpolation, True)
     if plan is not None:
         with torch.cuda.device(grad_output.device):
-            rc = lib.mcx_max_unpool_planned(_ptr(grad_output), _ptr(idx_mask), _ptr(plan),
-                                            plan.numel(), _ptr(gin), B, C, IH, IW, OH, OW, K, P,
+            rc = lib.mcx_max_unpool_planned(_ptr(grad_output), _ptr(idx_mask), *_plan_args(plan),
+                                            _ptr(gin), B, C, IH, IW, OH, OW, K, P,
                                             int(interpolation), dt, _stream(grad_output))
         _lib.check(rc, "mapped_max_unpool")
         return gin
@@ -510,7 +549,7 @@ def _avg_unpool(grad_output, sample_map, interp_weights, input_height, input_wid
                              interpolation, True)
     if plan is not None:
         with torch.cuda.device(grad_output.device):
-            rc = lib.mcx_avg_unpool_planned(_ptr(grad_output), _ptr(plan), plan.numel(), _ptr(gin),
+            rc = lib.mcx_avg_unpool_planned(_ptr(grad_output), *_plan_args(plan), _ptr(gin),
                                             B, C, IH, IW, OH, OW, K, P, int(interpolation), dt,
                                             _stream(grad_output))
         _lib.check(rc, "mapped_avg_unpool")
@@ -593,7 +632,7 @@ def _resample_to_map(input, sample_map, interp_weights, output_height, output_wi
                              False)
     if plan is not None:
         with torch.cuda.device(input.device):
-            rc = lib.mcx_resample_to_map_planned(_ptr(input), _ptr(plan), plan.numel(), _ptr(out),
+            rc = lib.mcx_resample_to_map_planned(_ptr(input), *_plan_args(plan), _ptr(out),
                                                  B, C, IH, IW, OH, OW, P, int(interpolation), dt,
                                                  _stream(input))
         _lib.check(rc, "resample_to_map")
@@ -733,6 +772,22 @@ def cube2rect(cubemap, rect_height, rect_width, interpolation):
 
 
 # ------------------------------------------------------------ icosphere map operators
+def gnomonic_samples(centres, kh, kw, res_lat, res_lon):
+    """gnomonic_kernel of package/layers/util/icosphere_functions.py:135-183 on the device:
+    centres [V, 2] (longitude, latitude), float32 -> [1, V, kh*kw, 2]."""
+    _contig(centres=centres)
+    _on_gpu("spherical_coords", centres)
+    if centres.dtype != torch.float32 or centres.dim() != 2 or centres.shape[1] != 2:
+        raise RuntimeError("spherical_coords must be a float32 tensor [V, 2]")
+    V = centres.shape[0]
+    out = torch.empty((1, V, int(kh) * int(kw), 2), dtype=torch.float32, device=centres.device)
+    with torch.cuda.device(centres.device):
+        rc = _lib.load().mcx_gnomonic_samples(_ptr(centres), _ptr(out), V, int(kh), int(kw),
+                                              float(res_lat), float(res_lon), _stream(centres))
+    _lib.check(rc, "gnomonic_kernel")
+    return out
+
+
 def planar_conv_operator_from_samples(samples, vertices, faces, keepdim=True, nearest=False):
     """Sphere.get_planar_conv_operator_from_samples of the reference's `_sphere` module
     (package/ext_modules/src/util/cpp/sphere.cpp:1117-1270) over a caller-supplied mesh.

@@ -16,6 +16,17 @@ _i64 = ctypes.c_int64
 _i = ctypes.c_int
 _sz = ctypes.c_size_t
 
+
+class PlanDesc(ctypes.Structure):
+    """mcx_plan_desc of include/mcx.h: what a map plan was built for, kept on the host."""
+    _fields_ = [("magic", ctypes.c_uint32), ("kind", ctypes.c_int32), ("interp", ctypes.c_int32),
+                ("dtype", ctypes.c_int32), ("SH", _i64), ("SW", _i64), ("MH", _i64), ("MW", _i64),
+                ("K", _i64), ("P", _i64), ("plan", ctypes.c_uint64), ("plan_bytes", ctypes.c_uint64),
+                ("map", ctypes.c_uint64), ("iw", ctypes.c_uint64), ("check", ctypes.c_uint64)]
+
+
+_desc = ctypes.POINTER(PlanDesc)
+
 # name -> (restype, argtypes); mirrors include/mcx.h one to one.
 SIGNATURES = {
     "mcx_abi_version": (_i, []),
@@ -35,25 +46,26 @@ SIGNATURES = {
     "mcx_conv_backward_workspace": (_sz, [_i64] * 9 + [_i]),
     "mcx_conv_backward": (_i, [_p] * 9 + [_sz] + [_i64] * 9 + [_i, _i, _p]),
     "mcx_conv_plan_bytes": (_sz, [_i64] * 6 + [_i]),
-    "mcx_conv_plan_build": (_i, [_p] * 3 + [_sz] + [_i64] * 6 + [_i, _i, _p]),
-    "mcx_conv_backward_planned": (_i, [_p] * 9 + [_sz, _p, _sz] + [_i64] * 9 + [_i, _i, _p]),
-    "mcx_conv_forward_planned": (_i, [_p] * 7 + [_sz, _p, _sz] + [_i64] * 9 + [_i, _i, _p]),
-    "mcx_tconv_forward_planned": (_i, [_p] * 7 + [_sz, _p, _sz] + [_i64] * 9 + [_i, _i, _p]),
-    "mcx_tconv_backward_planned": (_i, [_p] * 9 + [_sz, _p, _sz] + [_i64] * 9 + [_i, _i, _p]),
+    "mcx_conv_plan_build": (_i, [_p] * 3 + [_sz, _desc] + [_i64] * 6 + [_i, _i, _p]),
+    "mcx_conv_backward_planned": (_i, [_p] * 9 + [_sz, _p, _sz, _desc] + [_i64] * 9 + [_i, _i, _p]),
+    "mcx_conv_forward_planned": (_i, [_p] * 7 + [_sz, _p, _sz, _desc] + [_i64] * 9 + [_i, _i, _p]),
+    "mcx_tconv_forward_planned": (_i, [_p] * 7 + [_sz, _p, _sz, _desc] + [_i64] * 9 + [_i, _i, _p]),
+    "mcx_tconv_backward_planned": (_i, [_p] * 9 + [_sz, _p, _sz, _desc] + [_i64] * 9 + [_i, _i, _p]),
     "mcx_tconv_forward": (_i, [_p] * 7 + [_sz] + [_i64] * 9 + [_i, _i, _p]),
     "mcx_tconv_forward_workspace": (_sz, [_i64] * 9 + [_i]),
     "mcx_tconv_backward_workspace": (_sz, [_i64] * 9 + [_i]),
     "mcx_tconv_backward": (_i, [_p] * 9 + [_sz] + [_i64] * 9 + [_i, _i, _p]),
     "mcx_scatter_plan_bytes": (_sz, [_i64] * 6 + [_i, _i]),
-    "mcx_scatter_plan_build": (_i, [_p] * 3 + [_sz] + [_i64] * 6 + [_i, _i, _i, _p]),
-    "mcx_resample_to_map_planned": (_i, [_p] * 2 + [_sz, _p] + [_i64] * 7 + [_i, _i, _p]),
-    "mcx_avg_unpool_planned": (_i, [_p] * 2 + [_sz, _p] + [_i64] * 8 + [_i, _i, _p]),
-    "mcx_max_unpool_planned": (_i, [_p] * 3 + [_sz, _p] + [_i64] * 8 + [_i, _i, _p]),
+    "mcx_scatter_plan_build": (_i, [_p] * 3 + [_sz, _desc] + [_i64] * 6 + [_i, _i, _i, _p]),
+    "mcx_resample_to_map_planned": (_i, [_p] * 2 + [_sz, _desc, _p] + [_i64] * 7 + [_i, _i, _p]),
+    "mcx_avg_unpool_planned": (_i, [_p] * 2 + [_sz, _desc, _p] + [_i64] * 8 + [_i, _i, _p]),
+    "mcx_max_unpool_planned": (_i, [_p] * 3 + [_sz, _desc, _p] + [_i64] * 8 + [_i, _i, _p]),
     "mcx_knn_workspace": (_sz, [_i64] * 3 + [_i]),
     "mcx_knn": (_i, [_p] * 5 + [_sz] + [_i64] * 5 + [_i, _p]),
     "mcx_projection_map": (_i, [_p] + [_i64] * 4 + [_i] + [_i64] * 2 + [_p]),
     "mcx_cube_projection_map": (_i, [_p] + [_i64] * 4 + [_p]),
     "mcx_cube2rect": (_i, [_p] * 2 + [_i64] * 4 + [_i, _i, _p]),
+    "mcx_gnomonic_samples": (_i, [_p] * 2 + [_i64] * 3 + [ctypes.c_double] * 2 + [_p]),
     "mcx_planar_conv_operator_workspace": (_sz, [_i64]),
     "mcx_planar_conv_operator": (_i, [_p] * 7 + [_sz] + [_i64] * 3 + [_i, _p]),
 }

@@ -10,6 +10,7 @@
 
 #include "mcx.h"
 #include "mcx_conv.h"
+#include "mcx_plan.h"
 #include "mcx_taps.h"
 
 using namespace mcx;
@@ -438,25 +439,47 @@ extern "C" size_t mcx_conv_plan_bytes(int64_t IH, int64_t IW, int64_t OH, int64_
 }
 
 extern "C" int mcx_conv_plan_build(const void *map, const void *iw, void *plan, size_t plan_bytes,
-                                   int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
-                                   int64_t P, int interp, int dtype, void *stream) {
+                                   mcx_plan_desc *desc, int64_t IH, int64_t IW, int64_t OH,
+                                   int64_t OW, int64_t K, int64_t P, int interp, int dtype,
+                                   void *stream) {
   if (IH <= 0 || IW <= 0 || OH <= 0 || OW <= 0 || K <= 0 || P < 0) return MCX_E_SHAPE;
-  if (!map || !plan || (P > 0) != (iw != nullptr)) return MCX_E_NULL;
+  if (!map || !plan || !desc || (P > 0) != (iw != nullptr)) return MCX_E_NULL;
   if (!use_mfma(dtype, P)) return MCX_E_DTYPE;
   const size_t need = mfma_scatter_plan_bytes(IH, IW, OH, OW, K, P);
   if (need == 0) return MCX_E_SHAPE;
   if (plan_bytes < need) return MCX_E_WORKSPACE;
-  return mfma_scatter_plan_build((const float *)map, (const float *)iw, plan, IH, IW, OH, OW, K,
-                                 P, interp, (hipStream_t)stream);
+  desc->magic = 0;  // (not a plan until the build has been enqueued)
+  if (int rc = mfma_scatter_plan_build((const float *)map, (const float *)iw, plan, IH, IW, OH, OW,
+                                       K, P, interp, (hipStream_t)stream))
+    return rc;
+  // (the plan holds element indices and fp32 weights: the same for fp32 and bf16 data)
+  plan_desc_fill(desc, MCX_PLAN_CONV, interp, MCX_F32, IH, IW, OH, OW, K, P, plan, need, map, iw);
+  return 0;
 }
+
+namespace {
+// A plan, when given, must be the one mcx_conv_plan_build made at this address for this map,
+// interpolation and these sizes (SH x SW: the image the map samples; MH x MW: the map).
+int check_plan(const void *plan, size_t plan_bytes, const mcx_plan_desc *desc, bool mfma,
+               int64_t SH, int64_t SW, int64_t MH, int64_t MW, int64_t K, int64_t P, int interp,
+               const void *map, const void *iw) {
+  if (!plan) return 0;
+  if (!mfma) return MCX_E_DTYPE;
+  const size_t need = mfma_scatter_plan_bytes(SH, SW, MH, MW, K, P);
+  if (need == 0 || plan_bytes < need) return MCX_E_WORKSPACE;
+  return plan_desc_check(desc, MCX_PLAN_CONV, interp, MCX_F32, SH, SW, MH, MW, K, P, plan,
+                         plan_bytes, true, map, iw);
+}
+}  // namespace
 
 extern "C" int mcx_conv_backward_planned(const void *gy, const void *map, const void *iw,
                                          const void *x, const void *w, void *gx, void *gw,
                                          void *gb, void *workspace, size_t workspace_bytes,
-                                         const void *plan, size_t plan_bytes, int64_t B,
-                                         int64_t Ci, int64_t Co, int64_t IH, int64_t IW,
-                                         int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
-                                         int dtype, void *stream) {
+                                         const void *plan, size_t plan_bytes,
+                                         const mcx_plan_desc *desc, int64_t B, int64_t Ci,
+                                         int64_t Co, int64_t IH, int64_t IW, int64_t OH,
+                                         int64_t OW, int64_t K, int64_t P, int interp, int dtype,
+                                         void *stream) {
   ProfileRequestScope profile_scope;
   const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
   if (int rc = check_dims(d, OH, OW, dtype)) return rc;
@@ -464,33 +487,19 @@ extern "C" int mcx_conv_backward_planned(const void *gy, const void *map, const 
   if (gw && !x) return MCX_E_NULL;
   hipStream_t s = (hipStream_t)stream;
   const bool mfma = use_mfma(dtype, P);
-  if (plan) {
-    if (!mfma) return MCX_E_DTYPE;
-    const size_t need = mfma_scatter_plan_bytes(IH, IW, OH, OW, K, P);
-    if (need == 0 || plan_bytes < need) return MCX_E_WORKSPACE;
-  }
+  if (int rc = check_plan(plan, plan_bytes, desc, mfma, IH, IW, OH, OW, K, P, interp, map, iw))
+    return rc;
   MCX_DISPATCH_DTYPE(dtype, conv_backward_t<T>(mfma, gy, map, iw, x, w, gx, gw, gb, workspace,
                                                workspace_bytes, d, interp, s, plan));
 }
 
-namespace {
-// A plan, when given, must be one mcx_conv_plan_build made for these sizes (SH x SW: the
-// image the map samples; MH x MW: the map).
-int check_plan(const void *plan, size_t plan_bytes, bool mfma, int64_t SH, int64_t SW, int64_t MH,
-               int64_t MW, int64_t K, int64_t P) {
-  if (!plan) return 0;
-  if (!mfma) return MCX_E_DTYPE;
-  const size_t need = mfma_scatter_plan_bytes(SH, SW, MH, MW, K, P);
-  return (need == 0 || plan_bytes < need) ? MCX_E_WORKSPACE : 0;
-}
-}  // namespace
-
 extern "C" int mcx_conv_forward_planned(const void *x, const void *map, const void *iw,
                                         const void *w, const void *bias, void *y, void *workspace,
                                         size_t workspace_bytes, const void *plan,
-                                        size_t plan_bytes, int64_t B, int64_t Ci, int64_t Co,
-                                        int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
-                                        int64_t P, int interp, int dtype, void *stream) {
+                                        size_t plan_bytes, const mcx_plan_desc *desc, int64_t B,
+                                        int64_t Ci, int64_t Co, int64_t IH, int64_t IW, int64_t OH,
+                                        int64_t OW, int64_t K, int64_t P, int interp, int dtype,
+                                        void *stream) {
   ProfileRequestScope profile_scope;
   const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
   if (int rc = check_dims(d, OH, OW, dtype)) return rc;
@@ -498,7 +507,8 @@ extern "C" int mcx_conv_forward_planned(const void *x, const void *map, const vo
   if (!bias || !y) return MCX_E_NULL;
   hipStream_t s = (hipStream_t)stream;
   const bool mfma = use_mfma(dtype, P);
-  if (int rc = check_plan(plan, plan_bytes, mfma, IH, IW, OH, OW, K, P)) return rc;
+  if (int rc = check_plan(plan, plan_bytes, desc, mfma, IH, IW, OH, OW, K, P, interp, map, iw))
+    return rc;
   MCX_DISPATCH_DTYPE(dtype, conv_forward_t<T>(mfma, x, map, iw, w, bias, y, workspace,
                                               workspace_bytes, d, interp, s, plan));
 }
@@ -506,9 +516,10 @@ extern "C" int mcx_conv_forward_planned(const void *x, const void *map, const vo
 extern "C" int mcx_tconv_forward_planned(const void *x, const void *map, const void *iw,
                                          const void *w, const void *bias, void *y,
                                          void *workspace, size_t workspace_bytes, const void *plan,
-                                         size_t plan_bytes, int64_t B, int64_t Ci, int64_t Co,
-                                         int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
-                                         int64_t P, int interp, int dtype, void *stream) {
+                                         size_t plan_bytes, const mcx_plan_desc *desc, int64_t B,
+                                         int64_t Ci, int64_t Co, int64_t IH, int64_t IW,
+                                         int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
+                                         int dtype, void *stream) {
   ProfileRequestScope profile_scope;
   const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
   if (int rc = check_dims(d, IH, IW, dtype)) return rc;
@@ -516,7 +527,8 @@ extern "C" int mcx_tconv_forward_planned(const void *x, const void *map, const v
   if (!bias || !y) return MCX_E_NULL;
   hipStream_t s = (hipStream_t)stream;
   const bool mfma = use_mfma(dtype, P);
-  if (int rc = check_plan(plan, plan_bytes, mfma, OH, OW, IH, IW, K, P)) return rc;
+  if (int rc = check_plan(plan, plan_bytes, desc, mfma, OH, OW, IH, IW, K, P, interp, map, iw))
+    return rc;
   MCX_DISPATCH_DTYPE(dtype, tconv_forward_t<T>(mfma, x, map, iw, w, bias, y, workspace,
                                                workspace_bytes, d, interp, s, plan));
 }
@@ -524,10 +536,11 @@ extern "C" int mcx_tconv_forward_planned(const void *x, const void *map, const v
 extern "C" int mcx_tconv_backward_planned(const void *gy, const void *map, const void *iw,
                                           const void *x, const void *w, void *gx, void *gw,
                                           void *gb, void *workspace, size_t workspace_bytes,
-                                          const void *plan, size_t plan_bytes, int64_t B,
-                                          int64_t Ci, int64_t Co, int64_t IH, int64_t IW,
-                                          int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
-                                          int dtype, void *stream) {
+                                          const void *plan, size_t plan_bytes,
+                                          const mcx_plan_desc *desc, int64_t B, int64_t Ci,
+                                          int64_t Co, int64_t IH, int64_t IW, int64_t OH,
+                                          int64_t OW, int64_t K, int64_t P, int interp, int dtype,
+                                          void *stream) {
   ProfileRequestScope profile_scope;
   const ConvDims d{B, Ci, Co, IH, IW, OH, OW, K, P};
   if (int rc = check_dims(d, IH, IW, dtype)) return rc;
@@ -535,7 +548,8 @@ extern "C" int mcx_tconv_backward_planned(const void *gy, const void *map, const
   if (gw && !x) return MCX_E_NULL;
   hipStream_t s = (hipStream_t)stream;
   const bool mfma = use_mfma(dtype, P);
-  if (int rc = check_plan(plan, plan_bytes, mfma, OH, OW, IH, IW, K, P)) return rc;
+  if (int rc = check_plan(plan, plan_bytes, desc, mfma, OH, OW, IH, IW, K, P, interp, map, iw))
+    return rc;
   MCX_DISPATCH_DTYPE(dtype, tconv_backward_t<T>(mfma, gy, map, iw, x, w, gx, gw, gb, workspace,
                                                 workspace_bytes, d, interp, s, plan));
 }
@@ -588,7 +602,7 @@ extern "C" int mcx_tconv_backward(const void *gy, const void *map, const void *i
                                                 workspace_bytes, d, interp, s));
 }
 
-extern "C" int mcx_abi_version(void) { return 10; }
+extern "C" int mcx_abi_version(void) { return 11; }
 
 extern "C" int mcx_profile_dominant_kernel(void *start_event, void *stop_event) {
   mcx::set_profile_events(start_event, stop_event);
@@ -602,6 +616,9 @@ extern "C" const char *mcx_error_string(int code) {
     case MCX_E_SHAPE: return "mcx: invalid or too large dimension";
     case MCX_E_NULL: return "mcx: required pointer is NULL, or interp_weights and P disagree";
     case MCX_E_WORKSPACE: return "mcx: workspace missing or too small";
+    case MCX_E_PLAN:
+      return "mcx: this plan was not built for this operation, map, interpolation or size "
+             "(or its descriptor is missing or damaged)";
     case MCX_E_STATIC_LIMIT:
       return "mcx: this problem needs more scratch than the library's static buffer holds; "
              "use the entry point that takes a workspace";

@@ -502,14 +502,25 @@ __global__ __launch_bounds__(kThreads) void knn_grid_kernel(
     // a dimension the points do not spread over (cell size 0) has them all in its cell 0
     int ge[3] = {1, 1, 1};
     T hmin = inf_t<T>();
+    // largest coordinate magnitude of a cell face: the face lo + n * h is rounded to one unit in
+    // the last place of that magnitude, and the cell index floor((c - lo) / h) of a point next to
+    // face n is off by a few units in the last place of n, i.e. of (n * h) in coordinates
+    T reach = T(0);
 #pragma unroll
     for (int d = 0; d < D; d++) {
       if (head.h[d] > T(0)) {
         ge[d] = g[d];
         hmin = head.h[d] < hmin ? head.h[d] : hmin;
+        const T lo = head.lo[d] < T(0) ? -head.lo[d] : head.lo[d];
+        const T span = (T)g[d] * head.h[d];
+        reach = lo + span > reach ? lo + span : reach;
       }
     }
     const int gmax = max(ge[0], max(ge[1], ge[2]));
+    constexpr T kUlp = sizeof(T) == 4 ? T(1.1920929e-7) : T(2.220446049250313e-16);
+    // a thousandth of a cell, plus the rounding above (which outgrows it on long one-dimensional
+    // grids: 65536 cells in fp32 put a face off by hundredths of a cell)
+    const T slack = hmin * T(1e-3) + T(16) * kUlp * reach;
     for (int rho = 0; rho < gmax; rho++) {
       // ring rho: rows of cells along the first dimension; rows on the ring's outer faces
       // are contiguous runs of cells (one run of points), the others contribute their ends
@@ -548,7 +559,7 @@ __global__ __launch_bounds__(kThreads) void knn_grid_kernel(
 #pragma unroll
       for (int j = 1; j < KMAX; j++) kth = j < k ? bd[j] : kth;
       // (the margins cover the rounding of cell assignment, faces and distances)
-      const T safe = m - hmin * T(1e-3);
+      const T safe = m - slack;
       if (safe > T(0) && kth < safe * safe * T(1.0 - 1e-5)) break;
     }
   }

@@ -10,6 +10,7 @@
 #include <type_traits>
 
 #include "mcx_device.h"
+#include "mcx_plan.h"
 
 namespace mcx {
 namespace {
@@ -1131,12 +1132,19 @@ __device__ inline void transposed_gather_planes(
       const uint32_t part = len > base ? len - base : 0u;  // this lane's entries in the pass
       const uint32_t wave_part = longest - base;
       const bool first = base == 0, last = base + kListRegs >= longest;
-      uint32_t code[kListRegs];
+      // per entry: the source element to load and, for max unpooling, the value the recorded
+      // winner must have.  An entry past the end of the lane's list loads the lane's first
+      // source element (a valid address) and is dropped by a test, never by its zero weight
+      // (an Inf or NaN in an unrelated source element must not reach the destination): the
+      // average tests its position, max unpooling is given a winner no element can record.
+      uint32_t code[kListRegs], want[OP == UN_MAX ? kListRegs : 1];
       T w[kListRegs];
 #pragma unroll
       for (int u = 0; u < kListRegs; u++) {
         const bool in = (uint32_t)u < part;
-        code[u] = e_src[in ? start + base + u : (len ? start : 0u)];
+        const uint32_t cd = e_src[in ? start + base + u : (len ? start : 0u)];
+        code[u] = OP == UN_MAX ? cd / (uint32_t)K : cd;
+        if constexpr (OP == UN_MAX) want[u] = in ? cd : 0xffffffffu;
         w[u] = in ? e_wt[start + base + u] : T(0);
       }
       for (int c = 0; c < nc; c++) {
@@ -1150,16 +1158,14 @@ __device__ inline void transposed_gather_planes(
             bool keep[kGroup];
 #pragma unroll
             for (int j = 0; j < kGroup; j++) {
-              const uint32_t cd = code[g * kGroup + j];
-              const uint32_t n = OP == UN_MAX ? cd / (uint32_t)K : cd;
+              const uint32_t n = code[g * kGroup + j];
               v[j] = sc[n];
-              // Entries past the end of a lane's list are dropped by a test, not by their zero
-              // weight (an Inf or NaN in an unrelated source element must not reach the
-              // destination).  Max unpooling keeps the recorded-winner test alone: its padded
-              // entries repeat the lane's own first entry with weight zero, and the extra test
-              // cost it a third of its speed.
-              keep[j] = OP == UN_MAX ? ic[n] == (int64_t)cd * idx_scale
-                                     : (uint32_t)(g * kGroup + j) < part;
+              // (recorded winners are offsets into the map, below 2^31: 0xffffffff * idx_scale
+              // equals none of them, nor the -1 of "no winner")
+              if constexpr (OP == UN_MAX)
+                keep[j] = ic[n] == (int64_t)want[g * kGroup + j] * idx_scale;
+              else
+                keep[j] = (uint32_t)(g * kGroup + j) < part;
             }
 #pragma unroll
             for (int j = 0; j < kGroup; j++)
@@ -1362,12 +1368,15 @@ int launch_gather(const void *in, const void *map, const void *iw, void *out, in
   // (images and channels are one run of planes, kCH of them per thread: longer runs measured
   // slower, 0.321 / 0.330 / 0.332 / 0.350 ms at 8 / 16 / 32 / 64 planes for 256 planes of
   // 512 x 1024 sampled at 256 x 1536 locations)
+  // (the planes go into the grid's second dimension, which holds 65535 workgroups: beyond
+  // that the images stay in the third)
   const bool plane_ring = OP == OP_RESAMPLE && P == 0 && K == 1 && B * C <= 0x7fffffffLL &&
-                          N * 8 < (int64_t)kOobOffset;
+                          N * 8 < (int64_t)kOobOffset && (B * C + cpt - 1) / cpt <= 65535;
   if (plane_ring) {
     C *= B;
     B = 1;
   }
+  if ((C + cpt - 1) / cpt > 65535) return MCX_E_SHAPE;
   dim3 grid(div_up(MW, Patch<OP>::kW) * div_up(MH, Patch<OP>::kH), div_up(C, cpt), (unsigned)B);
   // (the LDS-window path copies 16-byte chunks of source rows)
   const int windows = plane_ring || (tap_registers && K <= 9 && N * 8 < (int64_t)kOobOffset &&
@@ -1718,30 +1727,42 @@ extern "C" size_t mcx_scatter_plan_bytes(int64_t MH, int64_t MW, int64_t DH, int
 }
 
 extern "C" int mcx_scatter_plan_build(const void *map, const void *iw, void *plan,
-                                      size_t plan_bytes, int64_t MH, int64_t MW, int64_t DH,
-                                      int64_t DW, int64_t K, int64_t P, int interp, int dtype,
-                                      int for_max_unpool, void *stream) {
+                                      size_t plan_bytes, mcx_plan_desc *desc, int64_t MH,
+                                      int64_t MW, int64_t DH, int64_t DW, int64_t K, int64_t P,
+                                      int interp, int dtype, int for_max_unpool, void *stream) {
   if (dtype != MCX_F32 && dtype != MCX_F64) return MCX_E_DTYPE;
-  if (!map || !plan || (P > 0) != (iw != nullptr)) return MCX_E_NULL;
+  if (!map || !plan || !desc || (P > 0) != (iw != nullptr)) return MCX_E_NULL;
   if (bad_dims({MH, MW, DH, DW, K, MH * MW, DH * DW}) || P < 0) return MCX_E_SHAPE;
   hipStream_t s = (hipStream_t)stream;
+  desc->magic = 0;  // (not a plan until the build has been enqueued)
   const int rc = dtype == MCX_F32
                      ? build_transposed<float>(map, iw, plan, plan_bytes, MH * MW, K, P, DH, DW,
                                                interp, for_max_unpool != 0, s)
                      : build_transposed<double>(map, iw, plan, plan_bytes, MH * MW, K, P, DH, DW,
                                                 interp, for_max_unpool != 0, s);
-  return rc == kNotApplicable ? MCX_E_WORKSPACE : rc;
+  if (rc) return rc == kNotApplicable ? MCX_E_WORKSPACE : rc;
+  mcx::plan_desc_fill(desc, for_max_unpool ? MCX_PLAN_SCATTER_MAX : MCX_PLAN_SCATTER, interp, dtype,
+                      DH, DW, MH, MW, K, P, plan,
+                      transposed_workspace(MH * MW, K, P, DH, DW, interp, dtype), map, iw);
+  return 0;
 }
 
 namespace {
 template <int OP>
 int planned_gather(const void *src, const int64_t *idx, void *dst, const void *plan,
-                   size_t plan_bytes, int64_t B, int64_t C, int64_t SH, int64_t SW, int64_t DH,
-                   int64_t DW, int64_t K, int64_t P, int interp, int dtype, void *stream) {
+                   size_t plan_bytes, const mcx_plan_desc *desc, int64_t B, int64_t C, int64_t SH,
+                   int64_t SW, int64_t DH, int64_t DW, int64_t K, int64_t P, int interp, int dtype,
+                   void *stream) {
   if (dtype != MCX_F32 && dtype != MCX_F64) return MCX_E_DTYPE;
   if (!src || !dst || !plan || (OP == UN_MAX && !idx)) return MCX_E_NULL;
   if (bad_dims({B, C, SH, SW, DH, DW, K, SH * SW, DH * DW}) || P < 0 || B > 65535)
     return MCX_E_SHAPE;
+  // the plan must be the one built for this op (a max-unpool plan's source codes differ from
+  // the others'), interpolation, sizes and data type, at this address
+  if (int rc = mcx::plan_desc_check(desc, OP == UN_MAX ? MCX_PLAN_SCATTER_MAX : MCX_PLAN_SCATTER,
+                                    interp, dtype, DH, DW, SH, SW, K, P, plan, plan_bytes, false,
+                                    nullptr, nullptr))
+    return rc;
   hipStream_t s = (hipStream_t)stream;
   const int rc = dtype == MCX_F32
                      ? gather_transposed<float, OP>(src, idx, dst, plan, plan_bytes, B * C, SH * SW,
@@ -1753,25 +1774,27 @@ int planned_gather(const void *src, const int64_t *idx, void *dst, const void *p
 }  // namespace
 
 extern "C" int mcx_resample_to_map_planned(const void *in, const void *plan, size_t plan_bytes,
-                                           void *out, int64_t B, int64_t C, int64_t IH, int64_t IW,
-                                           int64_t OH, int64_t OW, int64_t P, int interp, int dtype,
+                                           const mcx_plan_desc *desc, void *out, int64_t B,
+                                           int64_t C, int64_t IH, int64_t IW, int64_t OH,
+                                           int64_t OW, int64_t P, int interp, int dtype,
                                            void *stream) {
-  return planned_gather<UN_RESAMPLE>(in, nullptr, out, plan, plan_bytes, B, C, IH, IW, OH, OW, 1, P,
+  return planned_gather<UN_RESAMPLE>(in, nullptr, out, plan, plan_bytes, desc, B, C, IH, IW, OH, OW, 1, P,
                                      interp, dtype, stream);
 }
 
 extern "C" int mcx_avg_unpool_planned(const void *gout, const void *plan, size_t plan_bytes,
-                                      void *gin, int64_t B, int64_t C, int64_t IH, int64_t IW,
-                                      int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
-                                      int dtype, void *stream) {
-  return planned_gather<UN_AVG>(gout, nullptr, gin, plan, plan_bytes, B, C, OH, OW, IH, IW, K, P,
+                                      const mcx_plan_desc *desc, void *gin, int64_t B, int64_t C,
+                                      int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
+                                      int64_t P, int interp, int dtype, void *stream) {
+  return planned_gather<UN_AVG>(gout, nullptr, gin, plan, plan_bytes, desc, B, C, OH, OW, IH, IW, K, P,
                                 interp, dtype, stream);
 }
 
 extern "C" int mcx_max_unpool_planned(const void *gout, const int64_t *idx, const void *plan,
-                                      size_t plan_bytes, void *gin, int64_t B, int64_t C,
-                                      int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
-                                      int64_t P, int interp, int dtype, void *stream) {
-  return planned_gather<UN_MAX>(gout, idx, gin, plan, plan_bytes, B, C, OH, OW, IH, IW, K, P, interp,
+                                      size_t plan_bytes, const mcx_plan_desc *desc, void *gin,
+                                      int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t OH,
+                                      int64_t OW, int64_t K, int64_t P, int interp, int dtype,
+                                      void *stream) {
+  return planned_gather<UN_MAX>(gout, idx, gin, plan, plan_bytes, desc, B, C, OH, OW, IH, IW, K, P, interp,
                                 dtype, stream);
 }

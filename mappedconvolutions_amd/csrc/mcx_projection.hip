@@ -33,6 +33,18 @@ __device__ inline void spherical_to_image(double lon, double lat, int H, int W, 
   y = ((H - 1) / 2.0) * (-2.0 * lat / kPi + 1.0);
 }
 
+// A point (x, y) of the plane tangent to the unit sphere at latitude `lat` (x towards growing
+// longitude, y towards growing latitude), carried back onto the sphere: its latitude and
+// its longitude relative to the point of tangency.  (0, 0) gives 0 / 0, as the reference's
+// expression does; callers set that tap themselves.
+__device__ inline void tangent_plane_to_sphere(double x, double y, double lat, double &dlon,
+                                               double &lat_out) {
+  const double rho = sqrt(x * x + y * y);
+  const double nu = atan(rho);
+  lat_out = asin(cos(nu) * sin(lat) + y * sin(nu) * cos(lat) / rho);
+  dlon = atan2(x * sin(nu), rho * cos(lat) * cos(nu) - y * sin(lat) * sin(nu));
+}
+
 // Tap k of a pixel in row i: everything but the pixel's own longitude depends on (i, k)
 // alone.  Returns the tap's latitude and its longitude relative to the pixel (spherical
 // projections), or its row and column offset (perspective).
@@ -68,11 +80,30 @@ __device__ inline void row_tap(int proj, int H, int W, int kh, int kw, int dilat
     lat_or_row = lat;
     dlon = 0.0;
   } else {
-    const double rho = sqrt(x * x + y * y);
-    const double nu = atan(rho);
-    lat_or_row = asin(cos(nu) * sin(lat) + y * sin(nu) * cos(lat) / rho);
-    dlon = atan2(x * sin(nu), rho * cos(lat) * cos(nu) - y * sin(lat) * sin(nu));
+    tangent_plane_to_sphere(x, y, lat, dlon, lat_or_row);
   }
+}
+
+// Gnomonic kernels about arbitrary points of the sphere (the vertices of a mesh):
+// package/layers/util/icosphere_functions.py:135-183.  out[v][k] = (lon, lat) of tap k =
+// (k / kw - kh / 2, k % kw - kw / 2) x (res_lat, res_lon) on the plane tangent at
+// centres[v] = (lon, lat); the tap of index (kh / 2) * kw + kw / 2 is the centre itself;
+// longitudes wrapped into [-pi, pi).  Evaluated in double, rounded once.
+__global__ void gnomonic_samples_kernel(const float *__restrict__ centres, float *__restrict__ out,
+                                        int kh, int kw, double res_lat, double res_lon,
+                                        int64_t total) {
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= total) return;
+  const int K = kh * kw;
+  const int k = (int)(e % K);
+  const int64_t v = e / K;
+  const double lon = centres[v * 2], lat = centres[v * 2 + 1];
+  double dlon = 0.0, lat_out = lat;
+  if (k != (kh / 2) * kw + kw / 2)
+    tangent_plane_to_sphere((k % kw - kw / 2) * res_lon, (k / kw - kh / 2) * res_lat, lat, dlon,
+                            lat_out);
+  reinterpret_cast<float2 *>(out)[e] =
+      make_float2((float)(py_mod(lon + dlon + kPi, 2.0 * kPi) - kPi), (float)lat_out);
 }
 
 // out[oi][oj][k] = (x, y); pixel (oi*stride, oj*stride) of the H x W grid, tap k = (k / kw,
@@ -307,6 +338,18 @@ int mcx_cube_projection_map(float *out, int64_t cube_dim, int64_t kh, int64_t kw
   hipLaunchKernelGGL(cube_projection_map_kernel, dim3(div_up(total, 256)), dim3(256), 0,
                      (hipStream_t)stream, out, (int)cube_dim, (int)kh, (int)kw, (int)stride,
                      (int)OW, total);
+  MCX_HIP_CHECK_LAUNCH();
+  return 0;
+}
+
+int mcx_gnomonic_samples(const float *centres, float *out, int64_t V, int64_t kh, int64_t kw,
+                         double res_lat, double res_lon, void *stream) {
+  using namespace mcx;
+  if (!centres || !out) return MCX_E_NULL;
+  if (V < 1 || kh < 1 || kw < 1 || kh * kw > 0x7fff || V > 0x7fffffffLL) return MCX_E_SHAPE;
+  const int64_t total = V * kh * kw;
+  hipLaunchKernelGGL(gnomonic_samples_kernel, dim3(div_up(total, 256)), dim3(256), 0,
+                     (hipStream_t)stream, centres, out, (int)kh, (int)kw, res_lat, res_lon, total);
   MCX_HIP_CHECK_LAUNCH();
   return 0;
 }

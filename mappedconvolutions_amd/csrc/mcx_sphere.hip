@@ -111,7 +111,10 @@ __global__ __launch_bounds__(kThreads) void planar_operator_kernel(
     const int nf = min(kThreads, F - f0);
     for (int j = 0; j < nf; j++) {
       const float4 c = tile[j];
-      if (ray.x * c.x + ray.y * c.y + ray.z * c.z < c.w) continue;
+      // (written so that a NaN direction passes no cone: faces with vertex indices out of range
+      // carry a cosine of 2, which no finite direction reaches either, so their vertices are
+      // never read; a sample with a non-finite coordinate gets face -1)
+      if (!(ray.x * c.x + ray.y * c.y + ray.z * c.z >= c.w)) continue;
       const int f = f0 + j;
       float s, t, u;
       if (live && point_in_face(vertex(verts, faces[f * 3]), vertex(verts, faces[f * 3 + 1]),

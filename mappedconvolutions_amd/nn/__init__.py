@@ -1,7 +1,9 @@
 """Mapped layers with the reference's `mapped_convolution.nn` names
-(layers/nn/__init__.py:6-10).  The plain `Convolution` / `TransposedConvolution`
-re-implementations of torch.nn.Conv2d that the reference also exports are not
-part of the mapped hot path and are not provided."""
+(layers/nn/__init__.py:6-10).  The plain `Convolution` / `TransposedConvolution` that the
+reference also exports re-implement torch.nn.Conv2d and are no part of the mapped hot path:
+the layer classes are not defined here; `mappedconvolutions_amd.install_aliases()` registers
+the extension modules behind them (`_convolution`, `_transposed_convolution`) as calls of the
+library convolution, so that the reference's own layer files import."""
 from .mapped_convolution_layer import MappedConvolution
 from .mapped_transposed_convolution_layer import MappedTransposedConvolution
 from .mapped_max_pooling_layer import MappedMaxPool

@@ -101,3 +101,22 @@ def check_args(input, sample_map, interp_weights, in_channels, kernel_size):
         check_sample_map_shape(sample_map, kernel_size)
     if interp_weights is not None:
         check_interp_weights_shape(sample_map, interp_weights)
+
+
+class OwnedPlan:
+    """The map plan of a layer whose sample map stays the same from call to call (a layer
+    built with cache_plan=True): one plan, rebuilt when the layer is handed another map
+    tensor, a map that was modified in place (torch's version counter; writes through
+    `.data` are not seen), or another sampled size or data type."""
+
+    def __init__(self):
+        self.key, self.plan = None, None
+
+    def get(self, build, sample_map, interp_weights, *rest):
+        def ident(t):
+            return None if t is None else (t.data_ptr(), t._version, tuple(t.shape), t.device)
+        key = (ident(sample_map), ident(interp_weights)) + tuple(rest)
+        if key != self.key:
+            self.plan = build()
+            self.key = key
+        return self.plan

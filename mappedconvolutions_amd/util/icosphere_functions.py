@@ -7,8 +7,6 @@ package/layers/util/icosphere_functions.py:132-262 with the mesh handed over as 
     idx, w = kernel_map_from_samples(samples, vertices, faces)     # [1, V, K, 3, 2], [1, V, K, 3]
     y = MappedConvolution(C, C2, kh*kw, 'nearest')(x, idx, w)      # x: [B, C, 1, V]
 """
-import math
-
 import torch
 
 from .. import _C
@@ -22,26 +20,11 @@ def convert_3d_to_spherical(xyz):
 
 
 def gnomonic_kernel(spherical_coords, kh, kw, res_lat, res_lon):
-    """icosphere_functions.py:132-180: a kh x kw grid of spacing (res_lon, res_lat) on the
-    tangent plane at every (lon, lat) of `spherical_coords` [V, 2], projected back onto the
-    sphere.  Returns [1, V, kh*kw, 2] (lon, lat) on the input's device."""
-    dev = spherical_coords.device
-    lon = spherical_coords[..., 0].reshape(1, -1, 1)
-    lat = spherical_coords[..., 1].reshape(1, -1, 1)
-    j = torch.arange(kw, device=dev, dtype=spherical_coords.dtype) - (kw // 2)
-    i = torch.arange(kh, device=dev, dtype=spherical_coords.dtype) - (kh // 2)
-    x = (j * res_lon).repeat(kh).view(1, 1, kh * kw)
-    y = (i * res_lat).repeat_interleave(kw).view(1, 1, kh * kw)
-    rho = (x ** 2 + y ** 2).sqrt()
-    nu = rho.atan()
-    out_lat = (nu.cos() * lat.sin() + y * nu.sin() * lat.cos() / rho).asin()
-    out_lon = lon + torch.atan2(x * nu.sin(),
-                                rho * lat.cos() * nu.cos() - y * lat.sin() * nu.sin())
-    centre = (kh // 2) * kw + kw // 2  # rho == 0 there: 0 / 0 above
-    out_lat[..., centre] = lat[..., 0]
-    out_lon[..., centre] = lon[..., 0]
-    out_lon = ((out_lon + math.pi) % (2 * math.pi)) - math.pi
-    return torch.stack((out_lon, out_lat), -1)
+    """icosphere_functions.py:135-183: a kh x kw grid of spacing (res_lon, res_lat) on the
+    tangent plane at every (lon, lat) of `spherical_coords` [V, 2], carried back onto the
+    sphere by a device kernel.  Returns [1, V, kh*kw, 2] (lon, lat) on the input's device."""
+    centres = spherical_coords.reshape(-1, 2).float().contiguous()
+    return _C.gnomonic_samples(centres, kh, kw, res_lat, res_lon)
 
 
 def kernel_map_from_samples(samples, vertices, faces, nearest=False):

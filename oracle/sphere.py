@@ -94,3 +94,34 @@ def planar_conv_operator(samples, vertices, faces, nearest=False, chunk=512):
         w[sl] = np.where(found[:, None], stu, F32(0))
         passing[sl] = inside
     return face, vidx, w, passing
+
+
+def gnomonic_kernel(spherical_coords, kh, kw, res_lat, res_lon, dt=np.float32):
+    """package/layers/util/icosphere_functions.py:135-183: a kh x kw grid of spacing (res_lon,
+    res_lat) on the plane tangent at every (lon, lat) of spherical_coords [V, 2], carried back
+    onto the sphere; [1, V, kh*kw, 2] (lon in [-pi, pi), lat).  dt=float32 follows the
+    reference's arithmetic, dt=float64 gives the formulas' value.  Pinned by mathematics in
+    tests/test_sphere.py (the textbook forward gnomonic projection about the centre returns the
+    grid; the reference holds no test or fixture for it): parity otherwise unpinned."""
+    sc = np.asarray(spherical_coords, dtype=dt)
+    lon = sc[..., 0].reshape(1, -1, 1)
+    lat = sc[..., 1].reshape(1, -1, 1)
+    x = np.zeros(kh * kw, dtype=dt)
+    y = np.zeros(kh * kw, dtype=dt)
+    for i in range(kh):
+        for j in range(kw):
+            x[i * kw + j] = dt(j - kw // 2) * dt(res_lon)
+            y[i * kw + j] = dt(i - kh // 2) * dt(res_lat)
+    x, y = x.reshape(1, 1, -1), y.reshape(1, 1, -1)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        rho = np.sqrt(x ** 2 + y ** 2)
+        nu = np.arctan(rho)
+        out_lat = np.arcsin(np.cos(nu) * np.sin(lat) + y * np.sin(nu) * np.cos(lat) / rho)
+        out_lon = lon + np.arctan2(x * np.sin(nu),
+                                   rho * np.cos(lat) * np.cos(nu) - y * np.sin(lat) * np.sin(nu))
+    centre = (kh // 2) * kw + kw // 2
+    out_lat[..., centre] = lat[..., 0]
+    out_lon[..., centre] = lon[..., 0]
+    pi = dt(np.pi)
+    out_lon = np.mod(out_lon + pi, dt(2) * pi) - pi
+    return np.stack([out_lon, out_lat], -1).astype(dt)

@@ -266,6 +266,31 @@ def test_bf16_weight_gradient_over_many_tiles_per_workgroup(shape, row_shift, in
     assert torch.equal(got[1], again[1]) and torch.equal(got[2], again[2])
 
 
+@pytest.mark.parametrize("row_shift", [0.0, 0.37])
+@pytest.mark.parametrize("radius", [1, 2])
+def test_bf16_weight_gradient_over_many_tiles_against_the_oracle(radius, row_shift, device):
+    """The same walk over several row tiles per workgroup, against the ORACLE: 24 x 8192 pixels
+    are 1536 tiles of 128, which the 1280 (9 taps) or 512 (25 taps) pixel ranges of this channel
+    split take two or three at a time (three: a run padded to a whole ring period), with ragged
+    channel groups on both sides (24 of 128 plain, 40 = 32 + 8 gathered) and both forms of the
+    kernel (integral rows: two pairs per tap; shifted rows: four)."""
+    B, Co, Ci, H, W = 1, 24, 40, 24, 8192
+    K = (2 * radius + 1) ** 2
+    g = torch.Generator().manual_seed(191 + radius)
+    bf = lambda t: t.to(torch.bfloat16)
+    x, gy = bf(torch.randn(B, Ci, H, W, generator=g)), bf(torch.randn(B, Co, H, W, generator=g))
+    w = bf(torch.randn(Co, Ci, K, generator=g) / (Ci * K) ** 0.5)
+    b = bf(torch.randn(Co, generator=g))
+    smap = synthetic.latitude_map(H, W, radius)
+    smap[..., 1] = (smap[..., 1] + row_shift).clamp(0, H - 1)
+    g_o = O.mapped_conv_backward(gy.float(), smap, x.float(), w.float(), b.float(), K, 1)
+    xd, sd, wd_, bd, gyd = dev(x, smap, w, b, gy)
+    gr = _C.mapped_conv_backward(gyd, sd, xd, wd_, bd, K, 1)
+    for a, r, nm in zip(gr, g_o, ("grad_input", "grad_weight", "grad_bias")):
+        assert rel_err(a.float(), r) < 2e-2, nm
+    assert_close_elementwise(gr[1].float(), g_o[1], 2e-2, "grad_weight")
+
+
 @pytest.mark.parametrize("interp", [1, 2])
 @pytest.mark.parametrize("with_plan", [False, True])
 def test_bf16_transposed_conv_under_a_map_with_integral_rows(with_plan, interp, device):
@@ -397,8 +422,36 @@ def test_known_answers_through_fp32_and_bf16_kernels(name, dtype, device):
         torch.testing.assert_close(out.float().cpu(), want, rtol=1e-5, atol=1e-5)
     else:
         torch.testing.assert_close(out.float().cpu(), want, rtol=2e-2, atol=2e-2)
-    out.backward(torch.ones_like(out))
-    assert x.grad is not None and torch.isfinite(x.grad.float()).all()
+    gout = torch.arange(out.numel(), dtype=torch.float32).view(out.shape).remainder(7).sub(3)
+    out.backward(gout.to(dtype).cuda())
+    # every gradient against the oracle's backward of the same case (the reference runs
+    # gradcheck on these cases, package/tests/utils.py:63-96; gout holds small integers so that
+    # the bf16 inputs of the backward are exact too)
+    xf, sm, iwc = x.detach().float().cpu(), smap.cpu(), None if iw is None else iw.cpu()
+    k, interp = KNOWN["kernel_size"], helpers.INTERP[case["interpolation"]]
+    tol = TOL[dtype]
+    op = case["op"]
+    if op in ("conv", "tconv"):
+        if op == "conv":
+            want = O.weighted_mapped_conv_backward(gout, sm, iwc, xf, w, b, k, interp)
+        else:
+            want = O.weighted_mapped_transposed_conv_backward(gout, sm, iwc, xf, w, b, k, interp)
+        got = (x.grad, layer.weight.grad, layer.bias.grad)
+        for a, r, nm in zip(got, want, ("grad_input", "grad_weight", "grad_bias")):
+            assert a is not None and a.dtype == dtype
+            assert rel_err(a.float(), r) < tol, nm
+            assert_close_elementwise(a.float(), r, 2 * tol, nm)
+    else:
+        H, W = xf.shape[2:]
+        if op == "max_pool":
+            _, idx = O.weighted_mapped_max_pool(xf, sm, iwc, k, interp)
+            want = O.weighted_mapped_max_unpool(gout, idx, sm, iwc, H, W, k, interp)
+        elif op == "avg_pool":
+            want = O.weighted_mapped_avg_unpool(gout, sm, iwc, H, W, k, interp)
+        else:  # Unresample: the gradient of a gather is the scatter through the same map
+            want = O.weighted_resample_to_map(gout, sm, iwc, H, W, interp)
+        assert rel_err(x.grad.float(), want) < tol, "grad_input"
+        assert_close_elementwise(x.grad.float(), want, 2 * tol, "grad_input")
 
 
 # ------------------------------------------------------------ full-size configurations 3 and 5
@@ -484,6 +537,83 @@ def _picks(OH, OW, count, seed):
     fixed = [0, OW - 1, n - OW, n - 1, OW, 2 * OW - 1, (OH // 2) * OW, (OH // 2) * OW + OW - 1]
     rnd = torch.randperm(n, generator=g)[:count].tolist()
     return torch.tensor(sorted(set(p for p in fixed + rnd if p < n)), dtype=torch.int64)
+
+
+@pytest.mark.parametrize("interp", [0, 1])
+def test_config2_full_size(interp, device):
+    """The headline shape: B=8, 64 -> 64 channels, 256 x 512, 3 x 3 latitude map, fp32, nearest
+    and bilinear: forward and all three gradients at 2 048 sampled output pixels (corners,
+    seam columns, pole rows, random ones) of the first and the last image against the oracle."""
+    B, C, H, W, K = 8, 64, 256, 512, 9
+    smap = synthetic.latitude_map(H, W, 1).cuda()
+    torch.manual_seed(22 + interp)
+    x = torch.randn(B, C, H, W, device=device)
+    w = torch.randn(C, C, K, device=device) / (C * K) ** 0.5
+    b = torch.randn(C, device=device)
+    y = _sampled_conv_check(x, w, b, smap, None, K, interp, _picks(H, W, 2040, 2), [0, B - 1],
+                            1e-5, 23)
+    _dense_properties(x, w, b, smap, None, K, interp, y, 1e-5, 24)
+
+
+def test_layers_skip_the_gradients_nobody_asks_for(device):
+    """A layer whose input needs no gradient (a network's first layer) or whose parameters are
+    frozen gets None for those gradients from the op and the right values for the others;
+    cache_plan=True layers build one plan per map and give the same results."""
+    g = torch.Generator().manual_seed(808)
+    B, Ci, Co, H, W, K = 2, 12, 20, 10, 40, 9
+    smap = synthetic.latitude_map(H, W, 1).cuda()
+    x = torch.randn(B, Ci, H, W, generator=g).cuda()
+    gy = torch.randn(B, Co, H, W, generator=g).cuda()
+    for make in (lambda **kw: nn.MappedConvolution(Ci, Co, K, **kw),
+                 lambda **kw: nn.MappedTransposedConvolution(Ci, Co, K, **kw)):
+        layer = make().cuda()
+        call = (lambda l, inp: l(inp, smap)) if isinstance(layer, nn.MappedConvolution) else \
+            (lambda l, inp: l(inp, H, W, smap))
+        xr = x.clone().requires_grad_(True)
+        call(layer, xr).backward(gy)
+        full = (xr.grad.clone(), layer.weight.grad.clone(), layer.bias.grad.clone())
+        # first layer: no input gradient
+        layer.zero_grad()
+        call(layer, x).backward(gy)
+        assert torch.equal(layer.weight.grad, full[1]) and torch.equal(layer.bias.grad, full[2])
+        # frozen parameters: the input gradient alone
+        layer.zero_grad()
+        layer.weight.requires_grad_(False)
+        layer.bias.requires_grad_(False)
+        xr = x.clone().requires_grad_(True)
+        call(layer, xr).backward(gy)
+        # (the slots of a transposed-map cell are handed out in the order the builder's atomics
+        # land, so the input gradient's additions may be reordered from call to call)
+        assert rel_err(xr.grad, full[0]) < 1e-6 and layer.weight.grad is None
+        # the op itself
+        bwd = _C.mapped_conv_backward if isinstance(layer, nn.MappedConvolution) else \
+            _C.mapped_transposed_conv_backward
+        got = bwd(gy, smap, x, layer.weight.data, layer.bias.data, K, 1,
+                  needs=(False, True, False))
+        assert got[0] is None and got[2] is None and torch.equal(got[1], full[1])
+        got = bwd(gy, smap, x, layer.weight.data, layer.bias.data, K, 1,
+                  needs=(False, False, True))
+        assert got[0] is None and got[1] is None and rel_err(got[2], full[2]) < 1e-6
+        # a layer that owns its plan
+        owner = make(cache_plan=True).cuda()
+        owner.load_state_dict(layer.state_dict())
+        xr = x.clone().requires_grad_(True)
+        for _ in range(2):
+            owner.zero_grad()
+            xr.grad = None
+            call(owner, xr).backward(gy)
+        first_plan = owner._plan.plan
+        assert first_plan is not None
+        for a, r in zip((xr.grad, owner.weight.grad, owner.bias.grad), full):
+            assert rel_err(a, r) < 1e-5
+        smap2 = (smap + 0.5).contiguous()    # another map: the layer builds another plan
+        call(owner, x)
+        assert owner._plan.plan is first_plan
+        if isinstance(owner, nn.MappedConvolution):
+            owner(x, smap2)
+        else:
+            owner(x, H, W, smap2)
+        assert owner._plan.plan is not first_plan
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

@@ -147,3 +147,28 @@ def test_grid_knn_full_size_equals_walk_over_all_points(device):
     ws = torch.empty(need, dtype=torch.uint8, device=device)
     assert lib.mcx_knn(ref.data_ptr(), qry.data_ptr(), gi.data_ptr(), gd.data_ptr(),
                        ws.data_ptr(), need - 1, 1, 3, 30000, 50000, 16, 0, None) == -4
+
+
+@pytest.mark.parametrize("offset", [0.0, 4096.0])
+def test_grid_knn_long_one_dimensional_grid(offset, device):
+    """65 536 cells along one axis in fp32: the cell index of a point and the position of a
+    cell face are rounded by amounts that grow with the index, up to hundredths of a cell at
+    the far end (more when the coordinates sit far from the origin), so the early stop has to
+    allow for them.  Points on a regular lattice of half a cell put a point on or next to
+    every face; queries sit next to faces too.  Oracle on a sample, the walk over all points
+    for the rest."""
+    g = torch.Generator().manual_seed(77)
+    R, Q = 131072, 8192
+    step = 1.0 / 3.0
+    ref = (torch.arange(R, dtype=torch.float64) * step + offset)
+    ref = ref + (torch.rand(R, generator=g, dtype=torch.float64) - 0.5) * 1e-3 * step
+    ref = ref[torch.randperm(R, generator=g)].float().view(1, 1, R).contiguous()
+    at = torch.randint(0, R, (Q,), generator=g).double() * step + offset
+    qry = (at + (torch.rand(Q, generator=g, dtype=torch.float64) - 0.5) * 4 * step).float()
+    qry = qry.view(1, 1, Q).contiguous()
+    assert _lib.load().mcx_knn_workspace(1, 1, R, 0) > 0
+    gi, gd = _raw_knn(ref.cuda(), qry.cuda(), 8, True)
+    wi, wd = _raw_knn(ref.cuda(), qry.cuda(), 8, False)
+    assert torch.equal(gi, wi) and torch.equal(gd, wd)
+    io, do = O.knn_forward(ref, qry[:, :, :256].contiguous(), 8)
+    assert torch.equal(gi[:, :, :256].cpu(), io) and torch.equal(gd[:, :, :256].cpu(), do)

@@ -164,3 +164,58 @@ def test_plan_cache_serves_every_op(device):
         _C.enable_map_plan_cache(False)
     for a, r in zip(cached, plain):
         assert rel_err(a, r) < 1e-5
+
+
+def test_a_plan_is_refused_where_it_was_not_built_for(device):
+    """Plans of equal size are not interchangeable: one built for bilinear does not serve
+    bispherical, one built from another map tensor of the same shape does not serve this map,
+    an average-unpool plan does not serve max unpooling (their source codes differ), a plan
+    for another destination size or data type is not taken, and neither is a descriptor that
+    was edited after the build.  Each is rejected before anything is enqueued."""
+    g = torch.Generator().manual_seed(2400)
+    B, C, H, W, K = 1, 8, 12, 24, 9
+    x, gy = torch.randn(B, C, H, W, generator=g).cuda(), torch.randn(B, C, H, W, generator=g).cuda()
+    w, b = (torch.randn(C, C, K, generator=g) / 9).cuda(), torch.randn(C, generator=g).cuda()
+    smap = synthetic.latitude_map(H, W, 1).cuda()
+    other = (smap + 0.25).contiguous()
+    plan = _C.conv_map_plan(smap, None, H, W, 1)
+    want = _C.mapped_conv_forward(x, smap, w, b, K, 1)
+    assert torch.equal(_C.mapped_conv_forward(x, smap, w, b, K, 1, plan=plan), want)
+    refused = dict(match="plan was not built for")
+    with pytest.raises(RuntimeError, **refused):      # other interpolation, same sizes
+        _C.mapped_conv_forward(x, smap, w, b, K, 2, plan=plan)
+    with pytest.raises(RuntimeError, **refused):
+        _C.mapped_conv_backward(gy, smap, x, w, b, K, 2, plan=plan)
+    with pytest.raises(RuntimeError, **refused):      # other map of the same shape
+        _C.mapped_conv_forward(x, other, w, b, K, 1, plan=plan)
+    with pytest.raises(RuntimeError, **refused):      # a transposed conv's map samples its output:
+        _C.mapped_transposed_conv_forward(x, smap, w, b, H, W // 2, K, 1, plan=plan)  # H x W/2 here
+    with pytest.raises(RuntimeError, match="workspace missing or too small"):  # (too small a plan)
+        _C.mapped_transposed_conv_forward(x, smap, w, b, H, 2 * W, K, 1, plan=plan)
+    # (any code other than 1 or 2 is nearest: a plan built with 0 serves 7)
+    plan0 = _C.conv_map_plan(smap, None, H, W, 0)
+    assert torch.equal(_C.mapped_conv_forward(x, smap, w, b, K, 7, plan=plan0),
+                       _C.mapped_conv_forward(x, smap, w, b, K, 0))
+    # scatter plans
+    _, idx = _C.mapped_max_pool(x, smap, K, 1)
+    plan_a = _C.scatter_map_plan(smap, None, H, W, 1)
+    plan_m = _C.scatter_map_plan(smap, None, H, W, 1, for_max_unpool=True)
+    assert plan_a.numel() == plan_m.numel()
+    _C.mapped_avg_unpool(gy, smap, H, W, K, 1, plan=plan_a)
+    _C.mapped_max_unpool(gy, idx, smap, H, W, K, 1, plan=plan_m)
+    with pytest.raises(RuntimeError, **refused):
+        _C.mapped_max_unpool(gy, idx, smap, H, W, K, 1, plan=plan_a)
+    with pytest.raises(RuntimeError, **refused):
+        _C.mapped_avg_unpool(gy, smap, H, W, K, 1, plan=plan_m)
+    with pytest.raises(RuntimeError, **refused):
+        _C.mapped_avg_unpool(gy, smap, H, W, K, 2, plan=plan_a)
+    with pytest.raises(RuntimeError, **refused):      # built for float32 weights
+        _C.mapped_avg_unpool(gy.double(), smap.double(), H, W, K, 1, plan=plan_a)
+    with pytest.raises(RuntimeError, **refused):      # a conv plan is not a scatter plan
+        _C.mapped_avg_unpool(gy, smap, H, W, K, 1, plan=plan)
+    # an edited descriptor no longer matches its own check word
+    plan_a.desc.K = K + 1
+    with pytest.raises(RuntimeError, **refused):
+        _C.mapped_avg_unpool(gy, smap, H, W, K, 1, plan=plan_a)
+    with pytest.raises(RuntimeError, match="plan must come from"):
+        _C.mapped_avg_unpool(gy, smap, H, W, K, 1, plan=plan_m.buffer)

@@ -352,7 +352,7 @@ def test_conv_backward_with_map_plan(case, device):
     b = torch.randn(Co, generator=g).to(dtype)
     xd, sd, iwd, wd_, bd, gyd = dev(x, smap, iw, w, b, gy)
     plan = _C.conv_map_plan(sd, iwd, shape_in[2], shape_in[3], interp, dtype)
-    assert plan is not None and plan.is_cuda
+    assert plan is not None and plan.buffer.is_cuda
     if iw is None:
         g_o = O.mapped_conv_backward(gy.float(), smap, x.float(), w.float(), b.float(), K, interp)
         plain = _C.mapped_conv_backward(gyd, sd, xd, wd_, bd, K, interp)
@@ -665,6 +665,94 @@ def test_config4_full_size_scatter_properties(device):
     assert abs(lhs - rhs) < 1e-6 * (x.double() * au.double()).abs().sum()
     # sorted entry lists: the gather form gives the same bits on every call
     assert torch.equal(au, _C.mapped_avg_unpool(y, lmap, H, W, 9, 1))
+
+
+def _sub_map(smap, picks):
+    """The entries of `picks` (flat locations) of a map [H, W, ...] as a one-row map [1, n, ...]."""
+    flat = smap.reshape((smap.shape[0] * smap.shape[1],) + tuple(smap.shape[2:]))
+    return flat[picks].unsqueeze(0).contiguous()
+
+
+def _random_picks(n, count, seed):
+    g = torch.Generator().manual_seed(seed)
+    fixed = torch.tensor([0, 1, n // 2, n - 2, n - 1])
+    return torch.unique(torch.cat([fixed, torch.randperm(n, generator=g)[:count]]))
+
+
+def test_config4_full_size_against_the_oracle_at_sampled_positions(device):
+    """Configuration 4 at its own size - B=4, C=64, cube map 256 x 1536 <-> equirectangular
+    512 x 1024, 3 x 3 latitude-map pooling - against the oracle evaluated on sampled positions
+    only (a one-row map holding the sampled locations' entries):
+    gathers (resample_from_map, pooled values, argmax) bit-exact at about 4 000 positions;
+    scatters (resample_to_map, both unpoolings) within 1e-5 on inputs that are zero except at
+    the sampled source positions, compared over the whole destination."""
+    F, H, W, B, C, K = 256, 512, 1024, 4, 64, 9
+    g = torch.Generator().manual_seed(404)
+    cmap = synthetic.cube_to_equirect_map(F, H, W)
+    lmap = synthetic.latitude_map(H, W, 1)
+    y = torch.rand(B, C, H, W, generator=g)
+    yd = y.cuda()
+    for interp in (1, 2):
+        # resample_from_map: equirectangular image sampled at the cube map's pixels
+        picks = _random_picks(F * 6 * F, 4000, 10 + interp)
+        want = O.resample_from_map(y, _sub_map(cmap, picks), interp)
+        got = _C.resample_from_map(yd, cmap.cuda(), interp).view(B, C, -1)[:, :, picks.cuda()]
+        assert torch.equal(got.cpu(), want[:, :, 0]), "resample_from_map at sampled positions"
+        del got
+        # resample_to_map: a cube image that is zero except at the sampled pixels
+        vals = torch.rand(B, C, 1, len(picks), generator=g)
+        cube = torch.zeros(B, C, F * 6 * F)
+        cube[:, :, picks] = vals[:, :, 0]
+        want = O.resample_to_map(vals, _sub_map(cmap, picks), H, W, interp)
+        got = _C.resample_to_map(cube.view(B, C, F, 6 * F).cuda(), cmap.cuda(), H, W, interp)
+        assert rel_err(got, want) < 1e-5, "resample_to_map"
+        helpers.assert_close_elementwise(got, want, 1e-5, "resample_to_map")
+        del got, cube
+    # pooling over the equirectangular image
+    picks = _random_picks(H * W, 4000, 20)
+    sub = _sub_map(lmap, picks)
+    ld = lmap.cuda()
+    for interp in (0, 1):
+        mo, mi = O.mapped_max_pool(y, sub, K, interp)
+        ao = O.mapped_avg_pool(y, sub, K, interp)
+        m, i = _C.mapped_max_pool(yd, ld, K, interp)
+        a = _C.mapped_avg_pool(yd, ld, K, interp)
+        pc = picks.cuda()
+        assert torch.equal(m.view(B, C, -1)[:, :, pc].cpu(), mo[:, :, 0]), "max-pool values"
+        assert torch.equal(a.view(B, C, -1)[:, :, pc].cpu(), ao[:, :, 0]), "avg-pool values"
+        # the oracle's winners are offsets into its one-row map: the tap is (offset / 2) % K
+        tap = (mi[:, :, 0] // 2) % K
+        full_idx = torch.where(mi[:, :, 0] >= 0, (picks.view(1, 1, -1) * K + tap) * 2, mi[:, :, 0])
+        assert torch.equal(i.view(B, C, -1)[:, :, pc].cpu(), full_idx), "max-pool argmax"
+        # unpoolings: a gradient that is zero except at the sampled pooled pixels
+        gvals = torch.randn(B, C, 1, len(picks), generator=g)
+        gout = torch.zeros(B, C, H * W)
+        gout[:, :, picks] = gvals[:, :, 0]
+        goutd = gout.view(B, C, H, W).cuda()
+        want_a = O.mapped_avg_unpool(gvals, sub, H, W, K, interp)
+        got_a = _C.mapped_avg_unpool(goutd, ld, H, W, K, interp)
+        assert rel_err(got_a, want_a) < 1e-5, "avg unpool"
+        helpers.assert_close_elementwise(got_a, want_a, 1e-5, "avg unpool")
+        del got_a, want_a
+        want_m = O.mapped_max_unpool(gvals, mi, sub, H, W, K, interp)
+        got_m = _C.mapped_max_unpool(goutd, i, ld, H, W, K, interp)
+        assert rel_err(got_m, want_m) < 1e-5, "max unpool"
+        helpers.assert_close_elementwise(got_m, want_m, 1e-5, "max unpool")
+        del got_m, want_m, m, i, a, goutd
+
+
+def test_config4_knn_full_size_against_the_oracle_at_sampled_queries(device):
+    """524 288 queries against 40 962 reference points on the unit sphere, k = 8: indices and
+    distances of 2 048 sampled queries bit-exact against the oracle."""
+    ref = synthetic.sphere_points(40962, seed=1)
+    qry = synthetic.sphere_points(524288, seed=2)
+    idx, dist = knn(ref.cuda(), qry.cuda(), 8)
+    g = torch.Generator().manual_seed(8)
+    pick = torch.unique(torch.cat([torch.tensor([0, 524287]),
+                                   torch.randint(0, 524288, (2046,), generator=g)]))
+    io, do = O.knn_forward(ref, qry[:, :, pick].contiguous(), 8)
+    assert torch.equal(idx[:, :, pick.cuda()].cpu(), io), "KNN indices must be bit-exact"
+    assert torch.equal(dist[:, :, pick.cuda()].cpu(), do)
 
 
 def test_config5_bf16_5x5(device):

@@ -53,11 +53,21 @@ def test_rejected_arguments_return_codes_without_a_gpu():
     # map plans: sized for the matrix-core paths only; too small a buffer is refused
     need = lib.mcx_conv_plan_bytes(8, 8, 8, 8, 9, 0, 0)
     assert need > 0 and lib.mcx_conv_plan_bytes(8, 8, 8, 8, 9, 0, 1) == 0
-    assert lib.mcx_conv_plan_build(1, None, 1, need - 1, 8, 8, 8, 8, 9, 0, 1, 0, None) == -4
-    assert lib.mcx_conv_plan_build(1, None, None, need, 8, 8, 8, 8, 9, 0, 1, 0, None) == -3
-    assert lib.mcx_conv_plan_build(1, None, 1, need, 8, 8, 8, 8, 9, 0, 1, 1, None) == -1
-    assert lib.mcx_conv_backward_planned(1, 1, None, 1, 1, 1, 1, 1, 1, 1 << 30, 1, need - 1, 1, 4,
-                                         4, 8, 8, 8, 8, 9, 0, 1, 0, None) == -4
+    desc = _lib.PlanDesc()
+    assert lib.mcx_conv_plan_build(1, None, 1, need - 1, desc, 8, 8, 8, 8, 9, 0, 1, 0, None) == -4
+    assert lib.mcx_conv_plan_build(1, None, None, need, desc, 8, 8, 8, 8, 9, 0, 1, 0, None) == -3
+    assert lib.mcx_conv_plan_build(1, None, 1, need, None, 8, 8, 8, 8, 9, 0, 1, 0, None) == -3
+    assert lib.mcx_conv_plan_build(1, None, 1, need, desc, 8, 8, 8, 8, 9, 0, 1, 1, None) == -1
+    assert lib.mcx_conv_backward_planned(1, 1, None, 1, 1, 1, 1, 1, 1, 1 << 30, 1, need - 1, desc,
+                                         1, 4, 4, 8, 8, 8, 8, 9, 0, 1, 0, None) == -4
+    # a plan without a descriptor, or with one that no build call filled in, is refused
+    assert lib.mcx_conv_backward_planned(1, 1, None, 1, 1, 1, 1, 1, 1, 1 << 30, 1, need, None,
+                                         1, 4, 4, 8, 8, 8, 8, 9, 0, 1, 0, None) == -3
+    assert lib.mcx_conv_backward_planned(1, 1, None, 1, 1, 1, 1, 1, 1, 1 << 30, 1, need, desc,
+                                         1, 4, 4, 8, 8, 8, 8, 9, 0, 1, 0, None) == -6
+    assert lib.mcx_avg_unpool_planned(1, 1, 1 << 20, desc, 1, 1, 1, 8, 8, 8, 8, 9, 0, 1, 0,
+                                      None) == -6
+    assert b"plan" in lib.mcx_error_string(-6)
 
 
 def test_layer_api_and_parameter_shapes():

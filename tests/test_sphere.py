@@ -254,3 +254,89 @@ def test_gpu_vertex_kernel_map_drives_a_mapped_convolution(device):
     ones = torch.ones(1, 8, 1, V, device=device)
     want = layer.weight.sum((1, 2)) + layer.bias
     torch.testing.assert_close(layer(ones, idx, w)[0, :, 0].mean(1), want, atol=1e-4, rtol=1e-4)
+
+
+def _forward_gnomonic(lon, lat, lon0, lat0):
+    """Textbook gnomonic projection about (lon0, lat0): plane coordinates of (lon, lat)."""
+    cosc = np.sin(lat0) * np.sin(lat) + np.cos(lat0) * np.cos(lat) * np.cos(lon - lon0)
+    x = np.cos(lat) * np.sin(lon - lon0) / cosc
+    y = (np.cos(lat0) * np.sin(lat) - np.sin(lat0) * np.cos(lat) * np.cos(lon - lon0)) / cosc
+    return x, y
+
+
+def _gnomonic_case():
+    g = np.random.default_rng(21)
+    centres = np.stack([g.uniform(-np.pi, np.pi, 200), g.uniform(-1.45, 1.45, 200)], -1)
+    centres[:4] = [[3.1, 0.2], [-3.1, -0.2], [0.0, 1.5], [1.0, -1.5]]  # seam and near the poles
+    return centres.astype(np.float32), 3, 5, 0.031, 0.047
+
+
+def test_oracle_gnomonic_kernel_mathematics():
+    """The mesh kernels' sample locations: projected forward about their centre they are the
+    regular grid (j - kw/2) * res_lon, (i - kh/2) * res_lat; the centre tap is the centre;
+    longitudes lie in [-pi, pi); float32 stays within its rounding of float64."""
+    centres, kh, kw, rlat, rlon = _gnomonic_case()
+    s64 = osph.gnomonic_kernel(centres, kh, kw, rlat, rlon, np.float64)
+    assert s64.shape == (1, 200, kh * kw, 2)
+    c64 = centres.astype(np.float64)
+    x, y = _forward_gnomonic(s64[0, :, :, 0], s64[0, :, :, 1], c64[:, None, 0], c64[:, None, 1])
+    jj = (np.arange(kh * kw) % kw - kw // 2) * rlon
+    ii = (np.arange(kh * kw) // kw - kh // 2) * rlat
+    np.testing.assert_allclose(x, np.broadcast_to(jj, x.shape), atol=1e-12)
+    np.testing.assert_allclose(y, np.broadcast_to(ii, y.shape), atol=1e-12)
+    centre = (kh // 2) * kw + kw // 2
+    np.testing.assert_array_equal(s64[0, :, centre], c64)
+    assert (s64[..., 0] >= -np.pi).all() and (s64[..., 0] < np.pi).all()
+    s32 = osph.gnomonic_kernel(centres, kh, kw, rlat, rlon, np.float32)
+    dlon = np.abs((s32[..., 0] - s64[..., 0] + np.pi) % (2 * np.pi) - np.pi)
+    # (near a pole a longitude is ill-conditioned: compare on the sphere there)
+    assert (dlon * np.cos(s64[..., 1])).max() < 2e-6
+    assert np.abs(s32[..., 1] - s64[..., 1]).max() < 2e-6
+
+
+@pytest.mark.gpu
+def test_gpu_gnomonic_kernel_matches_oracle(device):
+    """The device evaluates every entry in double and rounds once: within a float32 ulp of the
+    float64 restatement (longitudes on the circle), within float32 rounding of the float32 one."""
+    from mappedconvolutions_amd import util
+    centres, kh, kw, rlat, rlon = _gnomonic_case()
+    got = util.gnomonic_kernel(torch.tensor(centres).cuda(), kh, kw, rlat, rlon).cpu().numpy()
+    s64 = osph.gnomonic_kernel(centres, kh, kw, rlat, rlon, np.float64)
+    assert got.shape == s64.shape and got.dtype == np.float32
+    dlon = np.abs((got[..., 0].astype(np.float64) - s64[..., 0] + np.pi) % (2 * np.pi) - np.pi)
+    assert dlon.max() <= 2.5e-7 and np.abs(got[..., 1] - s64[..., 1]).max() <= 1.2e-7
+    s32 = osph.gnomonic_kernel(centres, kh, kw, rlat, rlon, np.float32)
+    dlon = np.abs((got[..., 0] - s32[..., 0] + np.pi) % (2 * np.pi) - np.pi)
+    assert (dlon * np.cos(s64[..., 1])).max() < 2e-6
+    assert np.abs(got[..., 1] - s32[..., 1]).max() < 2e-6
+    assert (got[..., 0] >= -np.float32(np.pi)).all() and (got[..., 0] <= np.float32(np.pi)).all()
+
+
+@pytest.mark.gpu
+def test_gpu_operator_with_non_finite_samples_and_invalid_faces(device):
+    """A sample direction with a NaN or infinite coordinate gets face -1 (and zeros), also in
+    a mesh that holds faces with vertex indices out of range: those are culled before their
+    vertices are read, for every sample.  All other samples are unaffected."""
+    from mappedconvolutions_amd import _C, util
+    verts, faces = util.synthetic.subdivided_icosahedron(2)
+    g = torch.Generator().manual_seed(9)
+    lon = (torch.rand(300, generator=g) * 2 - 1) * 3.1
+    lat = (torch.rand(300, generator=g) - 0.5) * 3.0
+    samples = torch.stack([lon, lat], -1)
+    clean = _C.planar_conv_operator_from_samples(samples.view(30, 10, 2).cuda(), verts.cuda(),
+                                                 faces.cuda())
+    bad = samples.clone()
+    bad[7, 0] = float("nan")
+    bad[11, 1] = float("inf")
+    bad[13] = float("nan")
+    faces_bad = torch.cat([faces, torch.tensor([[0, 1, 10 ** 9], [-5, 2, 3]])]).contiguous()
+    got = _C.planar_conv_operator_from_samples(bad.view(30, 10, 2).cuda(), verts.cuda(),
+                                               faces_bad.cuda())
+    for a, b in zip(got, clean):
+        a, b = a.cpu().reshape(300, -1), b.cpu().reshape(300, -1)
+        keep = torch.ones(300, dtype=torch.bool)
+        keep[[7, 11, 13]] = False
+        assert torch.equal(a[keep], b[keep])
+    face, vidx, wts = [t.cpu().reshape(300, -1) for t in got]
+    assert (face[[7, 11, 13]] == -1).all() and (vidx[[7, 11, 13]] == -1).all()
+    assert (wts[[7, 11, 13]] == 0).all()
