@@ -74,6 +74,12 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float floatx2 __attribute__((ext_vector_type(2)));
 
+// acc + w.lo * word.lo + w.hi * word.hi (v_dot2_f32_bf16: products exact, fp32 sum)
+__device__ inline float dot_bf16(unsigned word, unsigned w, float acc) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, word),
+                                         __builtin_bit_cast(bf16x2, w), acc, false);
+}
+
 template <typename TD>
 __global__ void pack_weights_bf16_kernel(const TD *__restrict__ w, uint16_t *__restrict__ wb,
                                          int O, int G, int K, int Opad, int Gpad,
@@ -556,6 +562,279 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
           const float start = accumulate ? to_f32(yb[(int64_t)o * N]) : (bias ? to_f32(bias[o]) : 0.f);
           yb[(int64_t)o * N] = from_f32<TD>(acc[m][i] + start + (ab ? ab[o] : 0.f));
         }
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// gather_product for bf16 images, direct form.  With bf16 MFMA the products of a unit (one
+// tap x 16 source channels) are short, and matrix and vector instructions of a SIMD all but
+// take turns: the general kernel above spends its time on the vector instructions around the
+// samples (unpacking, fp32 interpolation, the way through LDS) and on re-reading the weight
+// tile once per 32 pixels.  Here
+//   * a lane gathers and interpolates exactly the elements its MFMA B operand holds
+//     (v_mfma_f32_32x32x16_bf16: lane (l31, lhi) holds channels lhi*8 .. lhi*8+7 of pixel column
+//     l31), so samples never touch LDS, and a wave multiplies two 32-pixel blocks by all 64*OG
+//     output channels per weight fetch: half the LDS bytes per product;
+//   * a tap is NA (pixel, weight) entries; a 32-bit word of an entry (two channels of its
+//     pixel) is multiplied by {w, 0} for the even and by {0, w} for the odd channel with
+//     v_dot2_f32_bf16: one instruction per channel and entry, nothing to unpack (v_perm_b32,
+//     which could bring the same channel of two pixels into one word, runs at half rate).  The
+//     weights are rounded to bf16, the precision of the samples they multiply;
+//   * gathers are buffer loads (scalar block offset + the lane's 32-bit offset: no address
+//     arithmetic in the loop), the loads of kDepth units are in flight, and the LDS reads of a
+//     unit are issued a step ahead of their use.
+// Only the weights (linear copies of the pre-packed slices) go through LDS, double buffered,
+// one barrier per unit.  A workgroup is 4 waves = 256 consecutive pixels of an image (in the
+// order of the flattened map, so any image width works) x 64*OG output channels.  The source is
+// the copy in blocks of 8 channels per pixel (to_channel_blocks_kernel).  PACKED: the taps come
+// from a packed map (a transposed map or a plan's gather part: four (pixel, weight) entries per
+// tap); else from sample_map under single-point bilinear / bispherical interpolation.  NA counts
+// the leading entries of a tap that are read (2 or 4); the launches of both values are gated
+// like those of the general kernel (pair_mask / row_mask).
+constexpr int kDgPx = 256;
+
+template <bool PACKED, int NA, int OG>
+__global__ __launch_bounds__(kThreads, 2) void gather_product_bf16_direct_kernel(
+    const bf16_t *__restrict__ src, const float *__restrict__ map, const float *__restrict__ iw,
+    const uint16_t *__restrict__ wb, const bf16_t *__restrict__ bias, bf16_t *__restrict__ y,
+    int O, int Opad, int Gpad, int SH, int SW, int N, int OW, int K, int weighted, int wrap,
+    int tiles_per_img, const int *__restrict__ gate, int run_if_zero,
+    const float *__restrict__ addend, const int *__restrict__ pair_mask, int run_if_leading,
+    const int *__restrict__ row_mask) {
+  static_assert(NA == 2 || NA == 4, "two or four entries per tap");
+  constexpr int NPR = NA / 2;              // entry pairs per tap
+  constexpr int TG = NA <= 2 ? 9 : 4;      // taps resolved into LDS at a time
+  constexpr int kDepth = NA <= 2 ? 3 : 2;  // units whose loads are in flight
+  typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+  __shared__ __attribute__((aligned(16))) unsigned TapOff[TG][kDgPx][NA];
+  __shared__ __attribute__((aligned(16))) unsigned TapW[TG][kDgPx][NPR];  // bf16 weights, two per word
+  __shared__ __attribute__((aligned(16))) uint4 Wt[2][2][kOT * OG];
+  if (gate && ((*gate == 0) != (run_if_zero != 0))) return;  // device-side path selection
+  const int tid = threadIdx.x;
+  const int tile = xcd_contiguous_tile(blockIdx.x, gridDim.x);
+  const int b = tile / tiles_per_img;
+  const int n0 = (tile - b * tiles_per_img) * kDgPx;
+  if (pair_mask) {
+    // the two-entry form serves every tile none of whose rows uses a later entry
+    bool leading = (unsigned)*pair_mask < (1u << 2);
+    if (!leading && row_mask) {
+      int any = 0;
+      for (int r = n0 / OW; r <= min(n0 + kDgPx - 1, N - 1) / OW; r++) any |= row_mask[r];
+      leading = any == 0;
+    }
+    if (leading != (run_if_leading != 0)) return;
+  }
+  const int o0 = blockIdx.y * (kOT * OG);
+  const int64_t plane = (int64_t)SH * SW;
+  const unsigned bstride = (unsigned)plane * 16u;  // bytes of a block of 8 channels of an image
+  const int chunks = Gpad / kGC;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l31 = lane & 31, lhi = lane >> 5;
+  const int px[2] = {wave * 64 + l31, wave * 64 + 32 + l31};  // this lane's pixels of the tile
+  // the image's staged copy as a buffer: the lane's offset selects pixel and (through lhi) the
+  // upper or lower block of a chunk, the scalar offset the chunk
+  const auto img = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<bf16_t *>(src) + (int64_t)b * Gpad * plane, (short)0,
+      (int)((unsigned)(Gpad / 8) * bstride), 0x00020000);
+  const unsigned lane_block = (unsigned)lhi * bstride;
+  const auto wbuf = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t *>(wb), (short)0, (int)((unsigned)K * chunks * 2u * Opad * 16u),
+      0x00020000);
+  // this thread's 16 bytes of a unit's weights: [kg][output][8 channels]
+  constexpr int kPerKg = kOT * OG;
+  const int wt = min(tid, 2 * kPerKg - 1);
+  const unsigned w_lane = ((unsigned)(wt / kPerKg) * Opad + o0 + wt % kPerKg) * 16u;
+
+  floatx16 acc[2 * OG][2];
+#pragma unroll
+  for (int m = 0; m < 2 * OG; m++)
+#pragma unroll
+    for (int q = 0; q < 2; q++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) acc[m][q][i] = 0.f;
+
+  int buf = 0;
+  for (int k0 = 0; k0 < K; k0 += TG) {
+    const int kn = min(TG, K - k0);
+    __syncthreads();  // the previous group's units are done with the tap cache
+    {                 // thread tid resolves the group's taps of pixel tid
+      const int n = n0 + tid;
+      const bool live = n < N;
+      const int64_t ng = live ? n : 0;
+      for (int kl = 0; kl < kn; kl++) {
+        unsigned off[4];
+        float wgt[4];
+        if constexpr (PACKED) {
+          // pre-resolved entries [tap][slot][pixel]: (pixel index of the source as bits, weight)
+#pragma unroll
+          for (int r = 0; r < NA; r++) {
+            const float2 q =
+                reinterpret_cast<const float2 *>(map)[((int64_t)(k0 + kl) * 4 + r) * N + ng];
+            off[r] = __builtin_bit_cast(unsigned, q.x) * 16u;
+            wgt[r] = live ? q.y : 0.f;
+          }
+        } else {
+          const int64_t e = ng * K + k0 + kl;
+          PairTap<4> t;
+          resolve_pairs<4, 16>(map[e * 2], map[e * 2 + 1], SH, SW, wrap != 0,
+                               live ? (weighted ? iw[e] : 1.f) : 0.f, t);
+#pragma unroll
+          for (int r = 0; r < NA; r++) {
+            off[r] = t.off[r];
+            wgt[r] = t.wt[r];
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < NA; r++) TapOff[kl][tid][r] = off[r];
+        // entry r weighs w[r] (rounded to bf16, the precision of the samples themselves): the
+        // word of entries 2r and 2r + 1 holds both, lane-side shifts make {w, 0} and {0, w}
+#pragma unroll
+        for (int r = 0; r < NPR; r++)
+          TapW[kl][tid][r] = __builtin_bit_cast(
+              unsigned, __builtin_convertvector(floatx2{wgt[2 * r], wgt[2 * r + 1]}, bf16x2));
+      }
+    }
+    __syncthreads();
+
+    // units: chunk-major, the tap fastest (a chunk's source rows stay in cache for all taps)
+    const int units = chunks * kn;
+    u32x4 ring[kDepth][2][NA];
+    u32x4 wring[kDepth];
+    int ki = 0, ci = 0, ks = 0;
+    // `offn`: the offsets of the unit whose loads are issued next; `wnext`: the packed weights
+    // of the unit that is interpolated next (both read from LDS a step ahead)
+    unsigned offn[2][NA], wnext[2][NPR];
+    auto fetch_offsets = [&]() __attribute__((always_inline)) {
+#pragma unroll
+      for (int q = 0; q < 2; q++)
+#pragma unroll
+        for (int r = 0; r < NA; r++) offn[q][r] = TapOff[ki][px[q]][r] + lane_block;
+    };
+    auto fetch_weights = [&]() __attribute__((always_inline)) {
+#pragma unroll
+      for (int q = 0; q < 2; q++)
+#pragma unroll
+        for (int r = 0; r < NPR; r++) wnext[q][r] = TapW[ks][px[q]][r];
+    };
+    auto issue_slot = [&](int d) __attribute__((always_inline)) {
+      // (wave-uniform by construction; said so explicitly, or the loads get a loop over lanes)
+      const int cc = __builtin_amdgcn_readfirstlane(min(ci, chunks - 1));
+      const int chunk_off = (int)((unsigned)cc * 2u * bstride);
+      const int w_off = __builtin_amdgcn_readfirstlane(
+          (int)((unsigned)((k0 + ki) * chunks + cc) * 2u * (unsigned)Opad * 16u));
+#pragma unroll
+      for (int q = 0; q < 2; q++)
+#pragma unroll
+        for (int r = 0; r < NA; r++)
+          ring[d][q][r] = __builtin_bit_cast(
+              u32x4, __builtin_amdgcn_raw_buffer_load_b128(img, (int)offn[q][r], chunk_off, 0));
+      wring[d] = __builtin_bit_cast(
+          u32x4, __builtin_amdgcn_raw_buffer_load_b128(wbuf, (int)w_lane, w_off, 0));
+      if (++ki == kn) {
+        ki = 0;
+        ++ci;
+      }
+    };
+    bf16x8 bq[2];
+    auto stage_slot = [&](int d, int bb) __attribute__((always_inline)) {
+#pragma unroll
+      for (int q = 0; q < 2; q++) {
+        float sv[8];
+#pragma unroll
+        for (int ch = 0; ch < 8; ch++) sv[ch] = 0.f;
+#pragma unroll
+        for (int r = 0; r < NPR; r++) {
+          // a word of an entry holds channels 2j (low half) and 2j + 1 of its pixel: against
+          // {w, 0} the dot product weighs the even channel, against {0, w} the odd one
+          const unsigned wp2 = wnext[q][r];
+          const unsigned w_even[2] = {wp2 & 0xffffu, wp2 >> 16};
+          const unsigned w_odd[2] = {wp2 << 16, wp2 & 0xffff0000u};
+#pragma unroll
+          for (int e = 0; e < 2; e++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+              const unsigned word = ring[d][q][2 * r + e][j];
+              sv[2 * j] = dot_bf16(word, w_even[e], sv[2 * j]);
+              sv[2 * j + 1] = dot_bf16(word, w_odd[e], sv[2 * j + 1]);
+            }
+        }
+        u32x4 pk;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          pk[j] = __builtin_bit_cast(
+              unsigned, __builtin_convertvector(floatx2{sv[2 * j], sv[2 * j + 1]}, bf16x2));
+        bq[q] = __builtin_bit_cast(bf16x8, pk);
+      }
+      if (tid < 2 * kPerKg)
+        *reinterpret_cast<u32x4 *>(&Wt[bb][tid / kPerKg][tid % kPerKg]) = wring[d];
+      if (++ks == kn) ks = 0;
+    };
+    bf16x8 aq[2 * OG];
+    auto fetch_operands = [&](int bb) __attribute__((always_inline)) {
+#pragma unroll
+      for (int m = 0; m < 2 * OG; m++)
+        aq[m] = __builtin_bit_cast(bf16x8, Wt[bb][lhi][32 * m + l31]);
+    };
+    auto products = [&]() __attribute__((always_inline)) {
+#pragma unroll
+      for (int m = 0; m < 2 * OG; m++)
+#pragma unroll
+        for (int q = 0; q < 2; q++)
+          acc[m][q] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aq[m], bq[q], acc[m][q], 0, 0, 0);
+    };
+    // (loads are issued unconditionally, past the last unit too, where they read the last
+    // chunk again: a load behind a branch would make every later wait a full one)
+    fetch_offsets();
+#pragma unroll
+    for (int d = 0; d < kDepth; d++) {
+      issue_slot(d);
+      fetch_offsets();
+    }
+    fetch_weights();
+    int u = 0;
+    for (; u + kDepth <= units; u += kDepth) {
+#pragma unroll
+      for (int d = 0; d < kDepth; d++) {
+        stage_slot(d, buf);
+        __syncthreads();
+        fetch_operands(buf);
+        fetch_weights();
+        issue_slot(d);
+        fetch_offsets();
+        products();
+        buf ^= 1;
+      }
+    }
+#pragma unroll
+    for (int d = 0; d < kDepth - 1; d++) {
+      if (u + d < units) {
+        stage_slot(d, buf);
+        __syncthreads();
+        fetch_operands(buf);
+        fetch_weights();
+        products();
+        buf ^= 1;
+      }
+    }
+  }
+
+  // epilogue: block (m, q) of the lane holds pixel px[q] and 16 output channels
+  const float *ab_img = (addend && gate && gate[1] > 0) ? addend : nullptr;
+#pragma unroll
+  for (int q = 0; q < 2; q++) {
+    const int n = n0 + px[q];
+    if (n >= N) continue;
+    bf16_t *yb = y + (int64_t)b * O * N + n;
+    const float *ab = ab_img ? ab_img + ((int64_t)b * N + n) * Opad : nullptr;
+#pragma unroll
+    for (int m = 0; m < 2 * OG; m++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        const int o = o0 + 32 * m + (i >> 2) * 8 + lhi * 4 + (i & 3);
+        if (o < O)
+          yb[(int64_t)o * N] = from_f32<bf16_t>(acc[m][q][i] + (bias ? to_f32(bias[o]) : 0.f) +
+                                                (ab ? ab[o] : 0.f));
       }
   }
 }
@@ -1195,14 +1474,22 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_bf16_ring_kernel(
         PairTap<4> tp;
         resolve_pairs<4, 16>(mxy[t].x, mxy[t].y, GH, GW, wrap != 0,
                              (live && k_base + k < K) ? 1.f : 0.f, tp);
+        // (weights are kept as bf16 in the low half of a word, the high half zero: the form
+        // v_dot2_f32_bf16 multiplies a word of two channels by to get the even one)
+        auto wbits = [](float w) {
+          return __builtin_bit_cast(
+              float, __builtin_bit_cast(unsigned,
+                                        __builtin_convertvector(floatx2{w, 0.f}, bf16x2)));
+        };
         if constexpr (NA == 2) {
           *reinterpret_cast<uint2 *>(&TapOff[par][k][p][0]) = make_uint2(tp.off[0], tp.off[1]);
-          *reinterpret_cast<float2 *>(&TapWt[par][k][p][0]) = make_float2(tp.wt[0], tp.wt[1]);
+          *reinterpret_cast<float2 *>(&TapWt[par][k][p][0]) =
+              make_float2(wbits(tp.wt[0]), wbits(tp.wt[1]));
         } else {
           *reinterpret_cast<uint4 *>(&TapOff[par][k][p][0]) =
               make_uint4(tp.off[0], tp.off[1], tp.off[2], tp.off[3]);
           *reinterpret_cast<float4 *>(&TapWt[par][k][p][0]) =
-              make_float4(tp.wt[0], tp.wt[1], tp.wt[2], tp.wt[3]);
+              make_float4(wbits(tp.wt[0]), wbits(tp.wt[1]), wbits(tp.wt[2]), wbits(tp.wt[3]));
         }
       }
     }
@@ -1241,8 +1528,15 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_bf16_ring_kernel(
         wv[4 * h] = t.x; wv[4 * h + 1] = t.y; wv[4 * h + 2] = t.z; wv[4 * h + 3] = t.w;
       }
     }
-    auto lo = [](unsigned v) { return __builtin_bit_cast(float, v << 16); };
-    auto hi = [](unsigned v) { return __builtin_bit_cast(float, v & 0xffff0000u); };
+    // a word of a gathered record holds channels 2j (low half) and 2j + 1: against {w, 0} the
+    // two-element dot product weighs the even channel, against {0, w} the odd one (one
+    // instruction per sample and pair, nothing to unpack; the weights are bf16 like the samples)
+    unsigned w_even[2 * NA], w_odd[2 * NA];
+#pragma unroll
+    for (int i = 0; i < 2 * NA; i++) {
+      w_even[i] = __builtin_bit_cast(unsigned, wv[i]);
+      w_odd[i] = w_even[i] << 16;
+    }
 #pragma unroll
     for (int j = 0; j < 4; j++) {  // channels 2j and 2j + 1 of the wave's eight
       float e[2] = {0.f, 0.f}, o[2] = {0.f, 0.f};  // [pixel of the pair]
@@ -1252,8 +1546,8 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_bf16_ring_kernel(
         for (int i = 0; i < NA; i++) {  // in the order of the pairs, like every other kernel
           const uint4 t = q[SLOT][px * NA + i];
           const unsigned word = j == 0 ? t.x : j == 1 ? t.y : j == 2 ? t.z : t.w;
-          e[px] = __builtin_fmaf(wv[px * NA + i], lo(word), e[px]);
-          o[px] = __builtin_fmaf(wv[px * NA + i], hi(word), o[px]);
+          e[px] = dot_bf16(word, w_even[px * NA + i], e[px]);
+          o[px] = dot_bf16(word, w_odd[px * NA + i], o[px]);
         }
       // (hardware round-to-nearest-even, the two pixels of a channel in one word)
       *reinterpret_cast<unsigned *>(&SB[buf][wave * 8 + 2 * j][2 * pp]) =
@@ -1840,6 +2134,56 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
   if (SH * SW * (int64_t)sizeof(TD) > 0xffffffffLL) return MCX_E_SHAPE;
   // bf16 storage with at least 128 output channels: 128 outputs per workgroup
   const bool wide = sizeof(TD) == 2 && Opad % (2 * kOT) == 0;
+  if constexpr (sizeof(TD) == 2) {
+    // bf16 images: the direct form, over pair words (taps straight from the map) or over
+    // 8-channel blocks (entries of a packed map)
+    // (a staged image and the packed weights are addressed as buffers of less than 4 GiB)
+    const ModeArgs m0 = mode_args(interp, P);
+    const bool from_map = blocked && !packed_map && m0.mode != kInterpNearest && m0.np == 1;
+    const bool from_packed = blocked && packed_map && m0.mode == kInterpNearest &&
+                             m0.np == 4;  // (the four entries of a packed map's cell)
+    if ((from_map || from_packed) && !accumulate && OH * OW <= 0x7fffffffLL - kDgPx &&
+        (int64_t)(Gpad / 8) * SH * SW * 16 < 0xffffff00LL &&
+        K * (int64_t)(Gpad / kGC) * 2 * Opad * 16 < 0xffffff00LL) {
+      const int64_t tiles_per_img = (OH * OW + kDgPx - 1) / kDgPx;
+      if (tiles_per_img * B > 0x7fffffffLL) return MCX_E_SHAPE;
+      const dim3 dgrid((unsigned)(tiles_per_img * B), (unsigned)(Opad / (wide ? 2 * kOT : kOT)));
+#define MCX_LAUNCH_DIRECT(FORM, NA, OG, MASK, LEAD)                                              \
+  hipLaunchKernelGGL((gather_product_bf16_direct_kernel<FORM, NA, OG>), dgrid, dim3(kThreads),   \
+                     0, s, reinterpret_cast<const bf16_t *>(src), map, iw,                       \
+                     reinterpret_cast<const uint16_t *>(wp),                                     \
+                     reinterpret_cast<const bf16_t *>(bias), reinterpret_cast<bf16_t *>(y),      \
+                     (int)O, Opad, Gpad, (int)SH, (int)SW, (int)(OH * OW), (int)OW, (int)K,      \
+                     m0.weighted, m0.wrap, (int)tiles_per_img, gate, run_if_zero, addend, MASK,  \
+                     LEAD, row_mask)
+#define MCX_LAUNCH_DIRECT_NA(FORM, OG)                                  \
+  if (pair_mask) {                                                      \
+    MCX_LAUNCH_DIRECT(FORM, 2, OG, pair_mask, 1);                       \
+    MCX_LAUNCH_DIRECT(FORM, 4, OG, pair_mask, 0);                       \
+  } else {                                                              \
+    MCX_LAUNCH_DIRECT(FORM, 4, OG, (const int *)nullptr, 0);            \
+  }
+      profile_begin(s);
+      if (from_map) {
+        if (wide) {
+          MCX_LAUNCH_DIRECT_NA(false, 2)
+        } else {
+          MCX_LAUNCH_DIRECT_NA(false, 1)
+        }
+      } else {
+        if (wide) {
+          MCX_LAUNCH_DIRECT_NA(true, 2)
+        } else {
+          MCX_LAUNCH_DIRECT_NA(true, 1)
+        }
+      }
+      profile_end(s);
+#undef MCX_LAUNCH_DIRECT_NA
+#undef MCX_LAUNCH_DIRECT
+      MCX_HIP_CHECK_LAUNCH();
+      return 0;
+    }
+  }
   dim3 grid((unsigned)t.total, (unsigned)(Opad / (wide ? 2 * kOT : kOT)));
   const ModeArgs m = mode_args(interp, P);
   // `pair_mask` (four-pair taps only): launch the two-pair form as well; the mask picks one
@@ -1958,8 +2302,9 @@ int mfma_gather_product(const TD *src, const float *map, const float *iw, const 
   // resolved measured the same within 1 %, so there only the plan's pair mask is used and the
   // 32 bytes per tap of the resolved form are not read; single-row sources and bf16 storage
   // gain from the resolved form)
+  // (bf16 images under single-point bilinear taps read pair words, which beats both)
   const bool resolved_pays =
-      !(sizeof(TD) == 4 && SH > 1 && canonical_interp(interp) != kInterpNearest);
+      !(SH > 1 && canonical_interp(interp) != kInterpNearest && (sizeof(TD) == 4 || P <= 1));
   if (plan && resolved_pays && gather_plan_applies(interp, P) &&
       OH * OW * K * kPlanSlots * 2 <= 0x7fffffffLL) {
     // the map's taps were resolved when the plan was built: read them as four pre-resolved
