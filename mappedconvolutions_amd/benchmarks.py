@@ -229,7 +229,70 @@ def plans(dev):
           _time(lambda: _C.mapped_conv_backward(gy, smap, x, w, b, K, 1)), flops=2 * flop)
 
 
-WORKLOADS = {"config3": config3, "config4": config4, "knn": knn, "config5": config5,
+def _launches(fn):
+    """Kernel launches of one call, counted by torch's profiler (0 when it cannot tell)."""
+    try:
+        from torch.profiler import ProfilerActivity, profile
+        fn()
+        torch.cuda.synchronize()
+        with profile(activities=[ProfilerActivity.CUDA]) as prof:
+            fn()
+            torch.cuda.synchronize()
+        return sum(1 for e in prof.events() if e.device_type.name == "CUDA" and
+                   "memcpy" not in e.name.lower() and "memset" not in e.name.lower())
+    except Exception:  # noqa: BLE001 - the count is an extra, the timing is the result
+        return 0
+
+
+def small(dev):
+    """Latency at small shapes.  Configuration 1 (B=1, 16 -> 32 channels, 64 x 128, 3 x 3
+    latitude map, bilinear, fp32) and the reference's own size sweep
+    (profile/profile_mapped_convolution.py:45-57: B=1, 10 -> 1 channels, K=9, bilinear over a
+    pixel-shuffle map, 10 x 10 ... 2000 x 2500) in the reference's float64 (scalar kernels
+    here) and in float32 (matrix-core kernels), next to the library's plain 3 x 3 convolution
+    the reference times beside it.  Microseconds per call and kernel launches per call."""
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(0)
+    B, Ci, Co, H, W, K = 1, 16, 32, 64, 128, 9
+    x = torch.randn(B, Ci, H, W, generator=g).to(dev)
+    w = (torch.randn(Co, Ci, K, generator=g) / (Ci * K) ** 0.5).to(dev)
+    b = torch.zeros(Co, device=dev)
+    gy = torch.randn(B, Co, H, W, generator=g).to(dev)
+    smap = synthetic.latitude_map(H, W, 1).to(dev)
+    plan = _C.conv_map_plan(smap, None, H, W, 1)
+    for tag, pl in (("", None), (" with a map plan", plan)):
+        fwd = lambda: _C.mapped_conv_forward(x, smap, w, b, K, 1, plan=pl)
+        bwd = lambda: _C.mapped_conv_backward(gy, smap, x, w, b, K, 1, plan=pl)
+        _line("config1 conv forward fp32 B1 16->32 64x128 K9" + tag, _time(fwd, iters=50),
+              flops=2.0 * B * H * W * Co * Ci * K, launches=_launches(fwd))
+        _line("config1 conv backward fp32" + tag, _time(bwd, iters=50),
+              flops=4.0 * B * H * W * Co * Ci * K, launches=_launches(bwd))
+    sizes = [(10, 10), (20, 25), (20, 50), (50, 100), (100, 100), (200, 250), (200, 500),
+             (500, 1000), (1000, 1000), (2000, 2500)]
+    Ci, Co = 10, 1
+    for dtype in (torch.float64, torch.float32):
+        name = str(dtype).split(".")[-1]
+        wgt = (torch.randn(Co, Ci, K, generator=g) / (Ci * K) ** 0.5).to(dev, dtype)
+        bias = torch.zeros(Co, device=dev, dtype=dtype)
+        for (h, wd) in sizes:
+            data = torch.randn(1, Ci, h, wd, generator=g).to(dev, dtype)
+            gout = torch.rand(1, Co, h, wd, generator=g).to(dev, dtype)
+            m = synthetic.pixel_shuffle_map(h, wd, 1, dtype).to(dev)
+            w33 = wgt.view(Co, Ci, 3, 3)
+            fwd = lambda: _C.mapped_conv_forward(data, m, wgt, bias, K, 1)
+            bwd = lambda: _C.mapped_conv_backward(gout, m, data, wgt, bias, K, 1)
+            it = 50 if h * wd <= 250000 else 10
+            print(json.dumps({
+                "workload": "sweep %s %dx%d B1 10->1 K9 bilinear pixel-shuffle map" % (name, h, wd),
+                "mapped_forward_us": round(_time(fwd, iters=it) * 1e3, 1),
+                "mapped_backward_us": round(_time(bwd, iters=it) * 1e3, 1),
+                "plain_conv_forward_us": round(
+                    _time(lambda: F.conv2d(data, w33, bias, padding=1), iters=it) * 1e3, 1),
+                "launches_forward": _launches(fwd), "launches_backward": _launches(bwd)}),
+                flush=True)
+
+
+WORKLOADS = {"small": small, "config3": config3, "config4": config4, "knn": knn, "config5": config5,
              "maps": maps, "plans": plans}
 
 

@@ -46,30 +46,72 @@ __device__ inline int xcd_contiguous_tile(int wg, int total) {
   return xcd * q + min(xcd, r) + slot;
 }
 
-// Repack W[o][g][k] -> Wp[k][g][o] with g padded to 16 and o padded to 64 (zeros),
-// so that a reduction chunk's weights are 16 rows of contiguous floats.
-// `transposed` reads W[g][o][k] instead (weights stored source-channel major).
-template <typename TD>
-__global__ void pack_weights_kernel(const TD *__restrict__ w, float *__restrict__ wp, int O,
-                                    int G, int K, int Opad, int Gpad, int transposed,
-                                    int *__restrict__ clear) {
-  if (clear && blockIdx.x == 0 && threadIdx.x == 0) *clear = 0;  // a flag word of the caller
-  const int64_t total = (int64_t)K * Gpad * Opad;
-  for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total;
-       e += (int64_t)gridDim.x * blockDim.x) {
-    const int o = (int)(e % Opad);
-    const int g = (int)((e / Opad) % Gpad);
-    const int k = (int)(e / ((int64_t)Opad * Gpad));
-    const int64_t wi = transposed ? ((int64_t)g * O + o) * K + k : ((int64_t)o * G + g) * K + k;
-    wp[e] = (o < O && g < G) ? to_f32(w[wi]) : 0.f;
-  }
+// Whether a pair beyond the first two of a tap is in use anywhere in the map, from the pair
+// mask: one word (at least 4 then), or `words` words of which any may say so (one per block
+// of the launch that examined the map).  Called by whole waves.
+__device__ inline bool later_pairs_in_use(const int *__restrict__ mask, int words) {
+  if (words <= 1) return (unsigned)*mask >= (1u << 2);
+  const int lane = threadIdx.x & 63;
+  const unsigned v = (unsigned)mask[lane < words ? lane : 0];
+  return __builtin_amdgcn_ballot_w64(v >= (1u << 2)) != 0;
 }
 
-// bf16 storage feeds v_mfma_f32_32x32x16_bf16: one instruction multiplies a 32 x 16 block
-// of weights by a 16 x 32 block of samples, a lane holding 8 consecutive reduction
-// elements (channels kg*8 .. kg*8+7, kg = lane / 32) of its row or column in 16 bytes.
-// Weights are therefore packed as Wb[k][chunk][kg][o][8] bf16: the 64 x 16 slice of a
-// (tap, chunk) is two runs of 64 x 16 bytes that are copied linearly into LDS.
+// Small jobs that ride on the weight-packing launch (a launch costs 4 to 8 us even when its
+// kernel does next to nothing, and small problems are made of launches):
+//   * ZeroJob: clear a region of the scratch (counters and flags of a transposed map);
+//   * PairMaskJob: the pair mask of a SMALL map, by the launch's last `blocks` (at most 64)
+//     blocks, each of which stores the bits it found into a word of its own - no clearing
+//     launch before, no atomics; the readers OR the words (later_pairs_in_use).
+struct ZeroJob {
+  uint4 *ptr;      // 16-byte aligned
+  int64_t count;   // 16-byte words
+};
+struct PairMaskJob {
+  const float *map, *iw;
+  int *mask;       // `blocks` words; nullptr: no job
+  int blocks, np, weighted, wrap, gh, gw, ncorn;
+  int64_t total;   // (location, tap) entries
+};
+
+// Bits of the (point, corner) pairs with a nonzero weight anywhere among the entries this
+// block walks (block `block` of `blocks`); valid in every thread on return.
+template <int NCORN>
+__device__ inline unsigned block_pair_mask(const float *__restrict__ map,
+                                           const float *__restrict__ iw, int np, int weighted,
+                                           int wrap, int GH, int GW, int64_t total, int block,
+                                           int blocks) {
+  __shared__ unsigned block_mask;
+  if (threadIdx.x == 0) block_mask = 0;
+  __syncthreads();
+  unsigned m = 0;
+  const int64_t first = (int64_t)block * blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)blocks * blockDim.x;
+  for (int64_t e = first; e < total; e += stride) {
+    for (int sp = 0; sp < np; sp++) {
+      const int64_t q = e * np + sp;
+      PairTap<NCORN> t;
+      resolve_pairs<NCORN, 4>(map[q * 2], map[q * 2 + 1], GH, GW, wrap != 0,
+                              weighted ? iw[q] : 1.f, t);
+#pragma unroll
+      for (int i = 0; i < NCORN; i++)
+        if (t.wt[i] != 0.f) m |= 1u << (sp * NCORN + i);
+    }
+  }
+  for (int d = 32; d > 0; d >>= 1) m |= __shfl_xor(m, d);
+  if ((threadIdx.x & 63) == 0 && m) atomicOr(&block_mask, m);
+  __syncthreads();
+  return block_mask;
+}
+
+// Repack W[o][g][k] for the matrix-core kernels, with g padded to 16 and o padded to 64
+// (zeros); `transposed` reads W[g][o][k] instead (weights stored source-channel major).
+//   fp32 storage: Wp[k][g][o] floats, so that a reduction chunk's weights are 16 rows of
+//   contiguous floats.
+//   bf16 storage feeds v_mfma_f32_32x32x16_bf16: one instruction multiplies a 32 x 16 block of
+//   weights by a 16 x 32 block of samples, a lane holding 8 consecutive reduction elements
+//   (channels kg*8 .. kg*8+7, kg = lane / 32) of its row or column in 16 bytes.  Weights are
+//   therefore packed as Wb[k][chunk][kg][o][8] bf16: the 64 x 16 slice of a (tap, chunk) is two
+//   runs of 64 x 16 bytes that are copied linearly into LDS.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float floatx2 __attribute__((ext_vector_type(2)));
@@ -81,23 +123,51 @@ __device__ inline float dot_bf16(unsigned word, unsigned w, float acc) {
 }
 
 template <typename TD>
-__global__ void pack_weights_bf16_kernel(const TD *__restrict__ w, uint16_t *__restrict__ wb,
-                                         int O, int G, int K, int Opad, int Gpad,
-                                         int transposed, int *__restrict__ clear) {
+__global__ __launch_bounds__(256) void pack_weights_kernel(
+    const TD *__restrict__ w, void *__restrict__ packed_out, int O, int G, int K, int Opad,
+    int Gpad, int transposed, int *__restrict__ clear, ZeroJob zero, PairMaskJob pm) {
   if (clear && blockIdx.x == 0 && threadIdx.x == 0) *clear = 0;  // a flag word of the caller
-  const int chunks = Gpad / kGC;
-  const int64_t total = (int64_t)K * Gpad * Opad;
-  for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total;
-       e += (int64_t)gridDim.x * blockDim.x) {
-    const int j = (int)(e & 7);
-    const int o = (int)((e >> 3) % Opad);
-    const int kg = (int)((e / ((int64_t)8 * Opad)) & 1);
-    const int c = (int)((e / ((int64_t)16 * Opad)) % chunks);
-    const int k = (int)(e / ((int64_t)16 * Opad * chunks));
-    const int g = c * kGC + kg * 8 + j;
-    const int64_t wi = transposed ? ((int64_t)g * O + o) * K + k : ((int64_t)o * G + g) * K + k;
-    wb[e] = (o < O && g < G) ? from_f32<bf16_t>(to_f32(w[wi])).v : (uint16_t)0;
+  int blocks = gridDim.x;
+  if (pm.mask) {
+    blocks -= pm.blocks;
+    if ((int)blockIdx.x >= blocks) {  // the last blocks: the map's pair mask, nothing else
+      const int mb = (int)blockIdx.x - blocks;
+      const unsigned m =
+          pm.ncorn == 1 ? block_pair_mask<1>(pm.map, pm.iw, pm.np, pm.weighted, pm.wrap, pm.gh,
+                                             pm.gw, pm.total, mb, pm.blocks)
+                        : block_pair_mask<4>(pm.map, pm.iw, pm.np, pm.weighted, pm.wrap, pm.gh,
+                                             pm.gw, pm.total, mb, pm.blocks);
+      if (threadIdx.x == 0) pm.mask[mb] = (int)m;
+      return;
+    }
   }
+  const int64_t first = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)blocks * blockDim.x;
+  const int64_t total = (int64_t)K * Gpad * Opad;
+  if constexpr (sizeof(TD) == 2) {
+    uint16_t *wb = reinterpret_cast<uint16_t *>(packed_out);
+    const int chunks = Gpad / kGC;
+    for (int64_t e = first; e < total; e += stride) {
+      const int j = (int)(e & 7);
+      const int o = (int)((e >> 3) % Opad);
+      const int kg = (int)((e / ((int64_t)8 * Opad)) & 1);
+      const int c = (int)((e / ((int64_t)16 * Opad)) % chunks);
+      const int k = (int)(e / ((int64_t)16 * Opad * chunks));
+      const int g = c * kGC + kg * 8 + j;
+      const int64_t wi = transposed ? ((int64_t)g * O + o) * K + k : ((int64_t)o * G + g) * K + k;
+      wb[e] = (o < O && g < G) ? from_f32<bf16_t>(to_f32(w[wi])).v : (uint16_t)0;
+    }
+  } else {
+    float *wp = reinterpret_cast<float *>(packed_out);
+    for (int64_t e = first; e < total; e += stride) {
+      const int o = (int)(e % Opad);
+      const int g = (int)((e / Opad) % Gpad);
+      const int k = (int)(e / ((int64_t)Opad * Gpad));
+      const int64_t wi = transposed ? ((int64_t)g * O + o) * K + k : ((int64_t)o * G + g) * K + k;
+      wp[e] = (o < O && g < G) ? to_f32(w[wi]) : 0.f;
+    }
+  }
+  for (int64_t i = first; i < zero.count; i += stride) zero.ptr[i] = make_uint4(0u, 0u, 0u, 0u);
 }
 
 // x[b][g][n] -> xt[b][n][Gpad] (channels past G zero): 64 pixels x 64 channels per
@@ -180,7 +250,8 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
     int O, int Opad, int Gpad, int SH, int SW, int OH, int OW, int K, int weighted, int wrap,
     int tiles_x, int tiles_per_img, int tw_shift, const int *__restrict__ gate, int run_if_zero,
     const float *__restrict__ addend, const int *__restrict__ pair_mask, int run_if_leading,
-    int packed_map, int accumulate, int cl_blocked, const int *__restrict__ row_mask) {
+    int packed_map, int accumulate, int cl_blocked, const int *__restrict__ row_mask,
+    int mask_words) {
   constexpr int NE = NP * NCORN;         // (offset, weight) pairs per pixel and tap
   static_assert(NA >= 1 && NA <= NE, "NA counts leading pairs");
   constexpr bool kMasked = NA == NE;
@@ -198,7 +269,8 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
   // accumulated.
   __shared__ unsigned TapMask[TG][2][2];
   if (gate && ((*gate == 0) != (run_if_zero != 0))) return;  // device-side path selection
-  if (pair_mask && !row_mask && (((unsigned)*pair_mask < (1u << 2)) != (run_if_leading != 0)))
+  if (pair_mask && !row_mask &&
+      (!later_pairs_in_use(pair_mask, mask_words) != (run_if_leading != 0)))
     return;
   // a pass that adds onto y (the second level of a transposed map) has nothing to do when
   // no pair of its map is in use
@@ -601,7 +673,7 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_bf16_direct_kernel
     int O, int Opad, int Gpad, int SH, int SW, int N, int OW, int K, int weighted, int wrap,
     int tiles_per_img, const int *__restrict__ gate, int run_if_zero,
     const float *__restrict__ addend, const int *__restrict__ pair_mask, int run_if_leading,
-    const int *__restrict__ row_mask) {
+    const int *__restrict__ row_mask, int mask_words) {
   static_assert(NA == 2 || NA == 4, "two or four entries per tap");
   constexpr int NPR = NA / 2;              // entry pairs per tap
   constexpr int TG = NA <= 2 ? 9 : 4;      // taps resolved into LDS at a time
@@ -617,7 +689,7 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_bf16_direct_kernel
   const int n0 = (tile - b * tiles_per_img) * kDgPx;
   if (pair_mask) {
     // the two-entry form serves every tile none of whose rows uses a later entry
-    bool leading = (unsigned)*pair_mask < (1u << 2);
+    bool leading = !later_pairs_in_use(pair_mask, mask_words);
     if (!leading && row_mask) {
       int any = 0;
       for (int r = n0 / OW; r <= min(n0 + kDgPx - 1, N - 1) / OW; r++) any |= row_mask[r];
@@ -878,26 +950,13 @@ template <int NCORN>
 __global__ void map_pair_mask_kernel(const float *__restrict__ map, const float *__restrict__ iw,
                                      int *__restrict__ mask, int np, int weighted, int wrap,
                                      int GH, int GW, int64_t total) {
-  __shared__ unsigned block_mask;
-  if (threadIdx.x == 0) block_mask = 0;
-  __syncthreads();
-  unsigned m = 0;
-  for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total;
-       e += (int64_t)gridDim.x * blockDim.x) {
-    for (int sp = 0; sp < np; sp++) {
-      const int64_t q = e * np + sp;
-      PairTap<NCORN> t;
-      resolve_pairs<NCORN, 4>(map[q * 2], map[q * 2 + 1], GH, GW, wrap != 0,
-                              weighted ? iw[q] : 1.f, t);
-#pragma unroll
-      for (int i = 0; i < NCORN; i++)
-        if (t.wt[i] != 0.f) m |= 1u << (sp * NCORN + i);
-    }
+  const unsigned m = block_pair_mask<NCORN>(map, iw, np, weighted, wrap, GH, GW, total,
+                                            (int)blockIdx.x, (int)gridDim.x);
+  if (gridDim.x == 1) {  // a launch of one block owns the word: no clearing before it
+    if (threadIdx.x == 0) *mask = (int)m;
+    return;
   }
-  for (int d = 32; d > 0; d >>= 1) m |= __shfl_xor(m, d);
-  if ((threadIdx.x & 63) == 0 && m) atomicOr(&block_mask, m);
-  __syncthreads();
-  report_pairs_beyond_two(mask, block_mask);
+  report_pairs_beyond_two(mask, m);
 }
 
 // CL: `gath` is a channel-last copy [B][GH*GW][Gpad] of the gathered operand (see the
@@ -2110,7 +2169,8 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
                           int interp, const int *gate, int run_if_zero, hipStream_t s,
                           const float *addend = nullptr, bool staged = false,
                           const int *pair_mask = nullptr, bool packed_map = false,
-                          bool accumulate = false, const int *row_mask = nullptr) {
+                          bool accumulate = false, const int *row_mask = nullptr,
+                          int mask_words = 1) {
   const int Opad = (int)round_up(O, kOT), Gpad = (int)round_up(G, kGC);
   const bool blocked = stage != nullptr && use_channel_blocks(SH, interp, sizeof(TD)) &&
                        SH * SW * 8 * (int64_t)sizeof(TD) <= 0xffffffffLL;
@@ -2155,7 +2215,7 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
                      reinterpret_cast<const bf16_t *>(bias), reinterpret_cast<bf16_t *>(y),      \
                      (int)O, Opad, Gpad, (int)SH, (int)SW, (int)(OH * OW), (int)OW, (int)K,      \
                      m0.weighted, m0.wrap, (int)tiles_per_img, gate, run_if_zero, addend, MASK,  \
-                     LEAD, row_mask)
+                     LEAD, row_mask, mask_words)
 #define MCX_LAUNCH_DIRECT_NA(FORM, OG)                                  \
   if (pair_mask) {                                                      \
     MCX_LAUNCH_DIRECT(FORM, 2, OG, pair_mask, 1);                       \
@@ -2192,7 +2252,8 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
                      dim3(kThreads), 0, s, src, map, iw, wp, bias, y, (int)G, (int)O, Opad,      \
                      Gpad, (int)SH, (int)SW, (int)OH, (int)OW, (int)K, m.weighted, m.wrap,       \
                      t.tiles_x, t.tiles_per_img, t.tw_shift, gate, run_if_zero, addend, MASK,    \
-                     LEAD, packed_map ? 1 : 0, accumulate ? 1 : 0, blocked ? 1 : 0, row_mask)
+                     LEAD, packed_map ? 1 : 0, accumulate ? 1 : 0, blocked ? 1 : 0, row_mask,     \
+                     mask_words)
 #define MCX_LAUNCH_CL(NCORN, NP, OG, CL)                                      \
   if constexpr (NCORN * NP == 4) {                                            \
     if (pair_mask) {                                                          \
@@ -2235,35 +2296,50 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
   return 0;
 }
 
+// Maps of up to kSmallMapEntries (location, tap) entries have their pair mask made on the
+// weight-packing launch of a forward call (a word per block, see PairMaskJob); elsewhere a map
+// of up to kTinyMapEntries gets a launch of one block, which needs no clearing launch before it.
+constexpr int64_t kSmallMapEntries = 262144;
+constexpr int64_t kTinyMapEntries = 4096;
+
 template <typename TD>
 int launch_pack_weights(const TD *w, float *wp, int64_t O, int64_t G, int64_t K, int transposed,
-                        hipStream_t s, int *clear = nullptr) {
+                        hipStream_t s, int *clear = nullptr, ZeroJob zero = ZeroJob{nullptr, 0},
+                        PairMaskJob pm = PairMaskJob{}) {
   const int Opad = (int)round_up(O, kOT), Gpad = (int)round_up(G, kGC);
   const int64_t packed = (int64_t)K * Gpad * Opad;
-  const dim3 grid((unsigned)std::min<int64_t>((packed + 255) / 256, 4096));
-  if (sizeof(TD) == 2)  // bf16 storage: bf16 MFMA operand layout (same scratch, half the bytes)
-    hipLaunchKernelGGL(pack_weights_bf16_kernel<TD>, grid, dim3(256), 0, s, w,
-                       reinterpret_cast<uint16_t *>(wp), (int)O, (int)G, (int)K, Opad, Gpad,
-                       transposed, clear);
-  else
-    hipLaunchKernelGGL(pack_weights_kernel<TD>, grid, dim3(256), 0, s, w, wp, (int)O, (int)G,
-                       (int)K, Opad, Gpad, transposed, clear);
+  // (bf16 storage: the bf16 MFMA operand layout in the same scratch, half the bytes)
+  const int64_t work = std::max(packed, zero.count * 4);
+  const dim3 grid((unsigned)std::min<int64_t>((work + 255) / 256, 4096) +
+                  (pm.mask ? (unsigned)pm.blocks : 0u));
+  hipLaunchKernelGGL(pack_weights_kernel<TD>, grid, dim3(256), 0, s, w, (void *)wp, (int)O, (int)G,
+                     (int)K, Opad, Gpad, transposed, clear, zero, pm);
   MCX_HIP_CHECK_LAUNCH();
   return 0;
+}
+
+inline PairMaskJob pair_mask_job(const float *map, const float *iw, int *mask, const ModeArgs &m,
+                                 int64_t GH, int64_t GW, int64_t samples) {
+  // (a block of 256 threads per 2048 entries, 64 at most: the readers load a word per lane)
+  const int blocks = (int)std::min<int64_t>(64, (samples + 2047) / 2048);
+  return PairMaskJob{map, iw, mask, blocks, m.np, m.weighted, m.wrap, (int)GH, (int)GW,
+                     m.mode == kInterpNearest ? 1 : 4, samples};
 }
 
 // mask[0] >= 4 iff the map uses a pair beyond the first two of a tap.
 // `cleared`: an earlier kernel on the stream has zeroed the mask.
 int launch_pair_mask(const float *map, const float *iw, int *mask, const ModeArgs &m, int64_t GH,
                      int64_t GW, int64_t samples, hipStream_t s, bool cleared = false) {
-  if (!cleared)
+  const bool small = samples <= kTinyMapEntries;  // one block, which stores the word outright
+  if (!cleared && !small)
     if (int rc = fill_f32((float *)mask, 1, 0.f, s)) return rc;
-  const dim3 mg((unsigned)std::min<int64_t>((samples + 255) / 256, 2048));
+  const dim3 mg(small ? 1u : (unsigned)std::min<int64_t>((samples + 255) / 256, 2048));
+  const dim3 threads(small ? 1024 : 256);
   if (m.mode == kInterpNearest)
-    hipLaunchKernelGGL(map_pair_mask_kernel<1>, mg, dim3(256), 0, s, map, iw, mask, m.np,
+    hipLaunchKernelGGL(map_pair_mask_kernel<1>, mg, threads, 0, s, map, iw, mask, m.np,
                        m.weighted, m.wrap, (int)GH, (int)GW, samples);
   else
-    hipLaunchKernelGGL(map_pair_mask_kernel<4>, mg, dim3(256), 0, s, map, iw, mask, m.np,
+    hipLaunchKernelGGL(map_pair_mask_kernel<4>, mg, threads, 0, s, map, iw, mask, m.np,
                        m.weighted, m.wrap, (int)GH, (int)GW, samples);
   MCX_HIP_CHECK_LAUNCH();
   return 0;
@@ -2328,19 +2404,29 @@ int mfma_gather_product(const TD *src, const float *map, const float *iw, const 
       (char *)scratch + align256((size_t)(K * round_up(G, kGC) * round_up(O, kOT)) * 4));
   TD *stage = (SH == 1 || sizeof(TD) == 2) ? reinterpret_cast<TD *>((char *)pair_mask + 256)
                                            : nullptr;
-  if (int rc = launch_pack_weights<TD>(w, wp, O, G, K, 0, s, pair_mask)) return rc;
   const ModeArgs m = mode_args(interp, P);
   const bool four_pairs = m.np * (m.mode == kInterpNearest ? 1 : 4) == 4;
   const int *mask = pair_mask;
+  // the pair mask of a small map is made by the last block of the packing launch
+  const bool mask_on_pack = four_pairs && !plan && OH * OW * K <= kSmallMapEntries;
+  if (int rc = launch_pack_weights<TD>(
+          w, wp, O, G, K, 0, s, mask_on_pack ? nullptr : pair_mask, ZeroJob{nullptr, 0},
+          mask_on_pack ? pair_mask_job(map, iw, pair_mask, m, SH, SW, OH * OW * K)
+                       : PairMaskJob{}))
+    return rc;
   if (four_pairs) {
     if (plan)  // flag word 4 of a plan built for this map
       mask = (const int *)plan + SH * SW * K + 4;
-    else if (int rc = launch_pair_mask(map, iw, pair_mask, m, SH, SW, OH * OW * K, s, true))
-      return rc;
+    else if (!mask_on_pack)
+      if (int rc = launch_pair_mask(map, iw, pair_mask, m, SH, SW, OH * OW * K, s, true))
+        return rc;
   }
+  const PairMaskJob job = mask_on_pack ? pair_mask_job(map, iw, pair_mask, m, SH, SW, OH * OW * K)
+                                       : PairMaskJob{};
   return launch_gather_product<TD>(src, map, iw, wp, bias, y, stage, B, G, O, SH, SW, OH, OW, K,
                                    P, interp, nullptr, 0, s, nullptr, false,
-                                   four_pairs ? mask : nullptr);
+                                   four_pairs ? mask : nullptr, false, false, nullptr,
+                                   mask_on_pack ? job.blocks : 1);
 }
 
 // ---- weight gradient ---------------------------------------------------------------
@@ -2775,13 +2861,15 @@ ScatterScratch scatter_scratch(int64_t B, int64_t S, int64_t D, int64_t K, int64
 // (or plan) region that starts at `cnt`.
 int build_transposed_map(const ScatterScratch &sc, const float *map, const float *iw, int *cnt,
                          const ModeArgs &m, int64_t DH, int64_t DW, int64_t MH, int64_t MW,
-                         int64_t K, hipStream_t s) {
+                         int64_t K, hipStream_t s, bool cleared = false) {
   char *region = (char *)cnt - sc.cnt;
   float2 *tmap = (float2 *)(region + sc.tmap);
   float2 *tmap2 = sc.two_level ? (float2 *)(region + sc.tmap2) : nullptr;
   OverflowEntry *ovf = (OverflowEntry *)(region + sc.ovf);
   int *flag = cnt + DH * DW * K;
-  if (int rc = fill_f32((float *)cnt, (int64_t)((sc.ovf - sc.cnt) / 4), 0.f, s)) return rc;
+  // (`cleared`: an earlier kernel on the stream has zeroed the region up to the overflow list)
+  if (!cleared)
+    if (int rc = fill_f32((float *)cnt, (int64_t)((sc.ovf - sc.cnt) / 4), 0.f, s)) return rc;
   const int64_t entries = MH * MW * K;
   const unsigned blocks = (unsigned)((entries + 255) / 256);
   if (m.mode == kInterpNearest)
@@ -2885,9 +2973,15 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
     gate = flag;
     OverflowEntry *ovf = (OverflowEntry *)(pbase + sc.ovf);
     TD *stage = (MH == 1 || sizeof(TD) == 2) ? (TD *)(base + sc.stage) : nullptr;
+    // (the packing launch also clears the transposed map's counters, flags and slots)
+    if (int rc = launch_pack_weights<TD>(
+            w, wpt, D, S, K, 1, s, nullptr,
+            plan ? ZeroJob{nullptr, 0}
+                 : ZeroJob{reinterpret_cast<uint4 *>(cnt), (int64_t)((sc.ovf - sc.cnt) / 16)}))
+      return rc;
     if (!plan)
-      if (int rc = build_transposed_map(sc, map, iw, cnt, m, DH, DW, MH, MW, K, s)) return rc;
-    if (int rc = launch_pack_weights<TD>(w, wpt, D, S, K, 1, s)) return rc;
+      if (int rc = build_transposed_map(sc, map, iw, cnt, m, DH, DW, MH, MW, K, s, true))
+        return rc;
     // What did not fit the four slots of its cell is accumulated with float atomics into a
     // channel-last fp32 image (cleared only when there is anything to add), which the
     // gather's epilogue adds.

@@ -70,6 +70,24 @@ def cube_to_equirect_map(face_dim, height, width, dtype=torch.float32):
     return torch.from_numpy(np.ascontiguousarray(out)).to(dtype)
 
 
+def pixel_shuffle_map(height, width, seed=0, dtype=torch.float32):
+    """The map of the reference's timing sweep (profile/profile_mapped_convolution.py:16-37,
+    78-81): the pixels of an H x W image are shuffled by a random permutation; tap (a, b) of
+    output pixel (i, j) points at the shuffled position of grid cell (i + a - 1, j + b - 1)
+    (cells outside the grid at (-1, -1)), plus 0.5 in x and y so that a bilinear tap blends four
+    unrelated pixels.  Returns [H, W, 9, 2]."""
+    rng = np.random.default_rng(seed)
+    perm = rng.permutation(height * width)
+    x = np.full((height + 2, width + 2), -1.0)
+    y = np.full((height + 2, width + 2), -1.0)
+    x[1:-1, 1:-1] = (perm % width).reshape(height, width)
+    y[1:-1, 1:-1] = (perm // width).reshape(height, width)
+    taps = [np.stack([x[a:a + height, b:b + width], y[a:a + height, b:b + width]], -1)
+            for a in range(3) for b in range(3)]
+    out = np.stack(taps, axis=2) + 0.5
+    return torch.from_numpy(np.ascontiguousarray(out)).to(dtype)
+
+
 def mesh_weighted_map(num_vertices, kernel_size, num_points, seed=0, dtype=torch.float32):
     """Weighted map of a mesh signal stored as a [1, V] image: every tap blends
     `num_points` vertices.  x = integer vertex index ~ U{0..V-1} (stored as a
