@@ -676,7 +676,7 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_bf16_direct_kernel
     const int *__restrict__ row_mask, int mask_words) {
   static_assert(NA == 2 || NA == 4, "two or four entries per tap");
   constexpr int NPR = NA / 2;              // entry pairs per tap
-  constexpr int TG = NA <= 2 ? 9 : 4;      // taps resolved into LDS at a time
+  constexpr int TG = NA <= 2 ? 13 : 4;     // taps resolved into LDS at a time
   constexpr int kDepth = NA <= 2 ? 3 : 2;  // units whose loads are in flight
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
   __shared__ __attribute__((aligned(16))) unsigned TapOff[TG][kDgPx][NA];
@@ -891,8 +891,14 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_bf16_direct_kernel
     }
   }
 
-  // epilogue: block (m, q) of the lane holds pixel px[q] and 16 output channels
+  // epilogue: block (m, q) of the lane holds pixel px[q] and 16 output channels, consecutive
+  // ones in consecutive elements.  Neighbouring lanes hold neighbouring pixels: with an even
+  // pixel count per plane a pair of lanes swaps one value of every two channels, so that the
+  // even lane stores two pixels of the even channel in one 32-bit word and the odd lane two
+  // pixels of the odd channel (half the store instructions of 2-byte stores).
   const float *ab_img = (addend && gate && gate[1] > 0) ? addend : nullptr;
+  const bool pack2 = (N & 1) == 0 && (reinterpret_cast<uintptr_t>(y) & 3) == 0;
+  const bool odd = (l31 & 1) != 0;
 #pragma unroll
   for (int q = 0; q < 2; q++) {
     const int n = n0 + px[q];
@@ -902,11 +908,27 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_bf16_direct_kernel
 #pragma unroll
     for (int m = 0; m < 2 * OG; m++)
 #pragma unroll
-      for (int i = 0; i < 16; i++) {
-        const int o = o0 + 32 * m + (i >> 2) * 8 + lhi * 4 + (i & 3);
-        if (o < O)
-          yb[(int64_t)o * N] = from_f32<bf16_t>(acc[m][q][i] + (bias ? to_f32(bias[o]) : 0.f) +
-                                                (ab ? ab[o] : 0.f));
+      for (int t = 0; t < 8; t++) {
+        const int oa = o0 + 32 * m + (t >> 1) * 8 + lhi * 4 + (t & 1) * 2, ob = oa + 1;
+        // (channels past O read a valid bias element; they are not stored)
+        const float va = acc[m][q][2 * t] + (bias ? to_f32(bias[min(oa, O - 1)]) : 0.f) +
+                         (ab ? ab[oa] : 0.f);
+        const float vb = acc[m][q][2 * t + 1] + (bias ? to_f32(bias[min(ob, O - 1)]) : 0.f) +
+                         (ab ? ab[ob] : 0.f);
+        if (pack2) {
+          const float send = odd ? va : vb;
+          const float recv = __builtin_bit_cast(
+              float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, send), 0xB1, 0xf, 0xf,
+                                              true));  // quad_perm [1, 0, 3, 2]
+          const int o = odd ? ob : oa;
+          const unsigned two = __builtin_bit_cast(
+              unsigned, __builtin_convertvector(floatx2{odd ? recv : va, odd ? vb : recv}, bf16x2));
+          if (o < O)
+            *reinterpret_cast<unsigned *>(yb + (int64_t)o * N - (odd ? 1 : 0)) = two;
+        } else {
+          if (oa < O) yb[(int64_t)oa * N] = from_f32<bf16_t>(va);
+          if (ob < O) yb[(int64_t)ob * N] = from_f32<bf16_t>(vb);
+        }
       }
   }
 }
