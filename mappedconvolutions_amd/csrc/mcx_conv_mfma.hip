@@ -217,19 +217,20 @@ __global__ __launch_bounds__(256) void to_channel_blocks_kernel(const TD *__rest
 }
 
 // LDS operand tiles of the gather-product kernel, double-buffered.
-template <typename TD>
+template <typename TD, int OG>
 struct OperandTiles {  // fp32: samples S[chunk channel][pixel], weights Wt[chunk channel][o]
   float S[2][kGC][kTilePx];
-  float Wt[2][kGC][kWtLd];
+  float Wt[2][kGC][kOT * OG + 4];
 };
-template <>
-struct OperandTiles<bf16_t> {  // bf16: 16-byte groups of 8 channels, [kg][pixel] and [kg][o]
+template <int OG>
+struct OperandTiles<bf16_t, OG> {  // bf16: 16-byte groups of 8 channels, [kg][pixel] and [kg][o]
   uint4 S[2][2][kTilePx];
   uint4 Wt[2][2][2 * kOT];
 };
 
-// OG: groups of 64 output channels per workgroup (2 only with bf16 storage, where the
-// gather, not the MFMA, bounds the kernel and is shared by twice the outputs).
+// OG: groups of 64 output channels per workgroup: 2 where the gather, not the MFMA, bounds the
+// kernel and is then shared by twice the outputs (bf16 storage; fp32 over a channel-last
+// source, whose every entry is a read of an unrelated record).
 // CL: `src` is a channel-last copy [B][SH*SW][Gpad] of the source (made by
 // to_channel_last_kernel): a sample's 8 channels are then one or two 16-byte loads from
 // one cache line instead of 8 loads from 8 lines.  Used for single-row sources (mesh
@@ -260,7 +261,7 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
   constexpr int kPairs = (NA <= 2 && OG == 1) ? kTapCache / 2 : kTapCache;
   constexpr int TG = NA <= 2 ? kPairs / NA : (kTapCache / NE > 0 ? kTapCache / NE : 1);
   constexpr bool kBf16 = sizeof(TD) == 2;
-  __shared__ __attribute__((aligned(16))) OperandTiles<TD> T;
+  __shared__ __attribute__((aligned(16))) OperandTiles<TD, OG> T;
   __shared__ __attribute__((aligned(16))) unsigned TapOff[TG][kTilePx][NA];
   __shared__ __attribute__((aligned(16))) float TapWt[TG][kTilePx][NA];
   // Bit e of TapMask[kl][h]: some pixel of the half-tile resolved by wave pair h has a
@@ -315,7 +316,7 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
   float wt[NE];
   float v[8][NE];
   unsigned tmask = 0;
-  float4 wv;   // fp32: this thread's share of the next weight chunk
+  float4 wv[OG];  // fp32: this thread's share of the next weight chunk
   unsigned wb8[2 * OG];  // bf16: likewise, 8 * OG bytes
   const int w_off = (tid >> 4) * Opad + (tid & 15) * 4;
 
@@ -389,7 +390,9 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
     } else {
       // weights of this chunk: 16 rows x 64 floats, one float4 per thread
       const float *wchunk = wp + ((int64_t)k * Gpad + c * kGC) * Opad + o0;  // uniform
-      wv = *reinterpret_cast<const float4 *>(wchunk + w_off);
+#pragma unroll
+      for (int og = 0; og < OG; og++)
+        wv[og] = *reinterpret_cast<const float4 *>(wchunk + w_off + og * kOT);
     }
   };
   auto stage = [&](int buf) {
@@ -418,7 +421,9 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
 #pragma unroll
       for (int ch = 0; ch < 8; ch++) T.S[buf][half * 8 + ch][p] = sv[ch];
       const int cc = tid >> 4, o4 = (tid & 15) * 4;
-      *reinterpret_cast<float4 *>(&T.Wt[buf][cc][o4]) = wv;
+#pragma unroll
+      for (int og = 0; og < OG; og++)
+        *reinterpret_cast<float4 *>(&T.Wt[buf][cc][og * kOT + o4]) = wv[og];
     }
   };
 
@@ -472,7 +477,12 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
     __syncthreads();
 
     // Units run chunk-major with the tap fastest: the source rows a 16-channel chunk
-    // touches are reused by all taps of the group while they are still in cache.
+    // touches are reused by all taps of the group while they are still in cache.  A
+    // channel-last source (a mesh signal: every entry of a tap points at an unrelated vertex,
+    // whose channels lie in one record) runs tap-major with the chunk fastest instead, so that
+    // a record is used up while its lines are in cache: chunk-major re-read every record once
+    // per chunk from memory.
+    const bool chunk_fastest = CL && !cl_blocked;
     const int units = chunks * kn;
     if constexpr (CL && kBf16) {
       // bf16 storage, staged source: a unit is NA 16-byte loads per thread and four short
@@ -484,7 +494,7 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
       u32x4 ring[kDepth][NA];
       u32x4 wring[kDepth];  // this thread's share of the unit's weights (8 * OG bytes)
       int ki = 0, ci = 0;   // the unit whose loads are issued next
-      int ks = 0;           // tap of the unit that is staged next
+      int ks = 0, cs = 0;   // tap (and, tap-major, chunk) of the unit that is staged next
       // (issued unconditionally, past the last unit too, where it reads the last chunk
       // again: a load that depends on a branch would make every later wait a full one)
       auto issue_slot = [&](int d) {
@@ -503,7 +513,12 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
         } else {
           wring[d] = *reinterpret_cast<const u32x4 *>(wchunk + (tid & 127) * 16);
         }
-        if (++ki == kn) {
+        if (chunk_fastest) {
+          if (++ci == chunks) {
+            ci = 0;
+            ki = min(ki + 1, kn - 1);  // (past the last unit: the last tap again)
+          }
+        } else if (++ki == kn) {
           ki = 0;
           ++ci;
         }
@@ -534,7 +549,14 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
               uint2{wring[d][0], wring[d][1]};
         else
           *reinterpret_cast<u32x4 *>(&T.Wt[b][tid >> 7][tid & 127]) = wring[d];
-        if (++ks == kn) ks = 0;
+        if (chunk_fastest) {
+          if (++cs == chunks) {
+            cs = 0;
+            ks = min(ks + 1, kn - 1);
+          }
+        } else if (++ks == kn) {
+          ks = 0;
+        }
       };
       auto products = [&](int b) {
         const bf16x8 bq = __builtin_bit_cast(bf16x8, T.S[b][lhi][wave * 32 + l31]);
@@ -577,7 +599,13 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
     for (int u = 0; u < units; ++u) {
       stage(buf);
       __syncthreads();
-      if (++kl == kn) {
+      if (chunk_fastest) {
+        if (++c == chunks) {
+          c = 0;
+          ++kl;
+        }
+        set_chunk(c);
+      } else if (++kl == kn) {
         kl = 0;
         ++c;
         set_chunk(c);
@@ -597,19 +625,19 @@ __global__ __launch_bounds__(kThreads, OG == 1 ? 4 : 3) void gather_product_mfma
         for (int m = 0; m < 2 * OG; m++)
           acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aq[m], bq, acc[m], 0, 0, 0);
       } else {
-        float bv[kGC / 2], a0[kGC / 2], a1[kGC / 2];
+        float bv[kGC / 2], av[2 * OG][kGC / 2];
 #pragma unroll
         for (int s = 0; s < kGC / 2; s++) {
           const int kk = 2 * s + lhi;
           bv[s] = T.S[buf][kk][wave * 32 + l31];
-          a0[s] = T.Wt[buf][kk][l31];
-          a1[s] = T.Wt[buf][kk][32 + l31];
+#pragma unroll
+          for (int m = 0; m < 2 * OG; m++) av[m][s] = T.Wt[buf][kk][32 * m + l31];
         }
 #pragma unroll
-        for (int s = 0; s < kGC / 2; s++) {
-          acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[s], bv[s], acc[0], 0, 0, 0);
-          acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[s], bv[s], acc[1], 0, 0, 0);
-        }
+        for (int s = 0; s < kGC / 2; s++)
+#pragma unroll
+          for (int m = 0; m < 2 * OG; m++)
+            acc[m] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[m][s], bv[s], acc[m], 0, 0, 0);
       }
       buf ^= 1;
     }
@@ -2215,7 +2243,9 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
   // tap offsets are 32-bit byte offsets inside a source plane
   if (SH * SW * (int64_t)sizeof(TD) > 0xffffffffLL) return MCX_E_SHAPE;
   // bf16 storage with at least 128 output channels: 128 outputs per workgroup
-  const bool wide = sizeof(TD) == 2 && Opad % (2 * kOT) == 0;
+  // (also fp32 over a channel-last source: a mesh signal's gather is a stream of unrelated
+  // records from memory, which 128 outputs share instead of 64)
+  const bool wide = Opad % (2 * kOT) == 0 && (sizeof(TD) == 2 || (cl && !blocked));
   if constexpr (sizeof(TD) == 2) {
     // bf16 images: the direct form, over pair words (taps straight from the map) or over
     // 8-channel blocks (entries of a packed map)
@@ -2298,7 +2328,7 @@ int launch_gather_product(const TD *src, const float *map, const float *iw, cons
     MCX_LAUNCH_CL(NCORN, NP, OG, false);       \
   }
 #define MCX_LAUNCH(NCORN, NP)                               \
-  if constexpr (sizeof(TD) == 2) {                          \
+  if constexpr (sizeof(TD) == 2 || NCORN == 1) {            \
     if (wide) {                                             \
       MCX_LAUNCH_OG(NCORN, NP, 2);                          \
     } else {                                                \
