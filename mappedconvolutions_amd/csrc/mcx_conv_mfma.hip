@@ -2632,8 +2632,12 @@ namespace {
 // scatter equals a weighted, nearest-neighbour gather-product over the transposed
 // map, which needs no atomics at all and reuses the forward kernel.  This kernel
 // builds that map: tmap[k][slot][p] = (index of source pixel n as bits, corner weight);
-// a slot counter per (p, k) hands out slots and an overflow flag selects the scatter
+// a slot counter per (k, p) hands out slots and an overflow flag selects the scatter
 // kernel instead (both kernels are always enqueued; the flag gates them on the device).
+// A wave takes 64 consecutive map pixels of one tap: under an image-like map they land on
+// neighbouring destination pixels, so its counter updates and slot writes fall into a few
+// cache lines (counters are [tap][pixel] like the slots); the taps of a run of pixels are
+// neighbouring waves, which read the same lines of the map.
 constexpr int kTransSlots = 4;
 constexpr int kTransSlotsConst = kTransSlots;
 
@@ -2653,11 +2657,14 @@ __global__ void build_transposed_map_kernel(const float *__restrict__ map,
                                             int *__restrict__ overflow,
                                             OverflowEntry *__restrict__ ovf, int ovf_cap, int np,
                                             int weighted, int wrap, int DH, int DW, int MW, int K,
-                                            int64_t total) {
-  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (e >= total) return;
-  const int k = (int)(e % K);
-  const int64_t n = e / K;
+                                            int64_t pixels) {
+  const int64_t t0 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t run = t0 / (64 * (int64_t)K);  // 64 map pixels x K taps
+  const int r = (int)(t0 - run * 64 * K);
+  const int k = r >> 6;
+  const int64_t n = run * 64 + (r & 63);
+  if (n >= pixels) return;
+  const int64_t e = n * K + k;
   const int64_t DHW = (int64_t)DH * DW;
   const float nbits = __builtin_bit_cast(float, (int)n);
   for (int sp = 0; sp < np; sp++) {
@@ -2669,7 +2676,7 @@ __global__ void build_transposed_map_kernel(const float *__restrict__ map,
     for (int c = 0; c < NCORN; c++) {
       if (!(t.ok & (1u << c)) || t.wt[c] == 0.f) continue;
       const int64_t pix = (int64_t)t.yy[c] * DW + t.xx[c];
-      const int64_t cell = pix * K + k;
+      const int64_t cell = (int64_t)k * DHW + pix;
       const int slot = atomicAdd(&cnt[cell], 1);
       // slots are stored [tap][slot][pixel] (see the gather-product kernel's packed maps)
       if (slot < kTransSlots) {
@@ -2751,7 +2758,7 @@ __global__ void after_transposed_map_kernel(const int *__restrict__ cnt, int64_t
                                             int *__restrict__ mask, int two_level,
                                             float *__restrict__ img, int64_t total,
                                             const int *__restrict__ overflow,
-                                            int *__restrict__ row_mask, int row_cells) {
+                                            int *__restrict__ row_mask, int64_t plane, int row_px) {
   __shared__ unsigned block_mask;
   if (threadIdx.x == 0) block_mask = 0;
   __syncthreads();
@@ -2761,8 +2768,8 @@ __global__ void after_transposed_map_kernel(const int *__restrict__ cnt, int64_t
     const int c = cnt[e];
     m |= (1u << min(c, 2 * kTransSlots)) - 1u;
     // row_mask[y] != 0 iff a cell of destination row y holds more than two entries (cells are
-    // [pixel][tap], row_cells of them per row; every writer stores the same value)
-    if (c > 2) row_mask[e / row_cells] = 1;
+    // [tap][pixel], `plane` pixels in rows of row_px; every writer stores the same value)
+    if (c > 2) row_mask[(e % plane) / row_px] = 1;
   }
   for (int d = 32; d > 0; d >>= 1) m |= __shfl_xor(m, d);
   if ((threadIdx.x & 63) == 0 && m) atomicOr(&block_mask, m);
@@ -2922,16 +2929,16 @@ int build_transposed_map(const ScatterScratch &sc, const float *map, const float
   // (`cleared`: an earlier kernel on the stream has zeroed the region up to the overflow list)
   if (!cleared)
     if (int rc = fill_f32((float *)cnt, (int64_t)((sc.ovf - sc.cnt) / 4), 0.f, s)) return rc;
-  const int64_t entries = MH * MW * K;
-  const unsigned blocks = (unsigned)((entries + 255) / 256);
+  const int64_t pixels = MH * MW;
+  const unsigned blocks = (unsigned)(((pixels + 63) / 64 * 64 * K + 255) / 256);
   if (m.mode == kInterpNearest)
     hipLaunchKernelGGL(build_transposed_map_kernel<1>, dim3(blocks), dim3(256), 0, s, map, iw, cnt,
                        tmap, tmap2, flag, ovf, (int)sc.ovf_cap, m.np, m.weighted, m.wrap, (int)DH,
-                       (int)DW, (int)MW, (int)K, entries);
+                       (int)DW, (int)MW, (int)K, pixels);
   else
     hipLaunchKernelGGL(build_transposed_map_kernel<4>, dim3(blocks), dim3(256), 0, s, map, iw, cnt,
                        tmap, tmap2, flag, ovf, (int)sc.ovf_cap, m.np, m.weighted, m.wrap, (int)DH,
-                       (int)DW, (int)MW, (int)K, entries);
+                       (int)DW, (int)MW, (int)K, pixels);
   MCX_HIP_CHECK_LAUNCH();
   return 0;
 }
@@ -2973,7 +2980,7 @@ int mfma_scatter_plan_build(const float *map, const float *iw, void *plan, int64
   hipLaunchKernelGGL(after_transposed_map_kernel,
                      dim3((unsigned)std::min<int64_t>((cells + 255) / 256, 4096)), dim3(256), 0, s,
                      cnt, cells, flag + 2, sc.two_level ? 1 : 0, (float *)nullptr, (int64_t)0,
-                     flag, flag + 8, (int)(K * DW));
+                     flag, flag + 8, DH * DW, (int)DW);
   MCX_HIP_CHECK_LAUNCH();
   if (m.np * (m.mode == kInterpNearest ? 1 : 4) == 4)
     if (int rc = launch_pair_mask(map, iw, flag + 4, m, DH, DW, MH * MW * K, s, true)) return rc;
@@ -3047,7 +3054,7 @@ int mfma_product_scatter(const TD *src, const float *map, const float *iw, const
                        dim3((unsigned)std::min<int64_t>(
                            std::max((total_img + 1023) / 1024, (cells + 255) / 256), 4096)),
                        dim3(256), 0, s, cnt, plan ? (int64_t)0 : cells, flag + 2,
-                       sc.two_level ? 1 : 0, img, total_img, flag, flag + 8, (int)(K * DW));
+                       sc.two_level ? 1 : 0, img, total_img, flag, flag + 8, DH * DW, (int)DW);
     MCX_HIP_CHECK_LAUNCH();
     if (cl) {  // the overflow pass reads the channel-last copy before the gather would make it
       dim3 tg((unsigned)((MH * MW + 63) / 64), (unsigned)((Spad16 + 63) / 64), (unsigned)B);
