@@ -218,22 +218,21 @@ int mcx_tconv_backward(const void *gy, const void *map, const void *iw, const vo
  * built at and from: after copying a plan or a map elsewhere, build again.  The library cannot
  * see writes into the map: rebuild the plan when the map's contents change. */
 enum {
-  MCX_PLAN_CONV = 1,        /* mcx_conv_plan_build */
-  MCX_PLAN_SCATTER = 2,     /* mcx_scatter_plan_build, for_max_unpool == 0 */
-  MCX_PLAN_SCATTER_MAX = 3, /* mcx_scatter_plan_build, for_max_unpool != 0 */
-  MCX_PLAN_POOL = 4         /* mcx_pool_plan_build */
+  MCX_PLAN_CONV = 1,       /* mcx_conv_plan_build */
+  MCX_PLAN_SCATTER = 2,    /* mcx_scatter_plan_build, for_max_unpool == 0 */
+  MCX_PLAN_SCATTER_MAX = 3 /* mcx_scatter_plan_build, for_max_unpool != 0 */
 };
 typedef struct mcx_plan_desc {
-  uint32_t magic;    /* 0x4d435850 */
-  int32_t kind;      /* MCX_PLAN_* */
-  int32_t interp;    /* 0 nearest, 1 bilinear, 2 bispherical */
-  int32_t dtype;     /* MCX_F32 / MCX_F64 for plans that hold weights in the data's type; conv: MCX_F32 */
-  int64_t SH, SW;    /* the image the map points into */
-  int64_t MH, MW;    /* the map's spatial size */
+  uint32_t magic; /* 0x4d435850 */
+  int32_t kind;   /* MCX_PLAN_* */
+  int32_t interp; /* 0 nearest, 1 bilinear, 2 bispherical */
+  int32_t dtype;  /* scatter plans hold weights in the data's type (MCX_F32 / MCX_F64); conv: MCX_F32 */
+  int64_t SH, SW; /* the image the map points into */
+  int64_t MH, MW; /* the map's spatial size */
   int64_t K, P;
-  uint64_t plan;     /* device address the plan was built at */
+  uint64_t plan; /* device address the plan was built at */
   uint64_t plan_bytes;
-  uint64_t map, iw;  /* device addresses of sample_map and interp_weights (0: none) */
+  uint64_t map, iw; /* device addresses of sample_map and interp_weights (0: none) */
   uint64_t check;
 } mcx_plan_desc;
 
@@ -254,15 +253,32 @@ typedef struct mcx_plan_desc {
 size_t mcx_conv_plan_bytes(int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P,
                            int dtype);
 int mcx_conv_plan_build(const void *map, const void *iw, void *plan, size_t plan_bytes,
-                        mcx_plan_desc *desc, int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P,
-                        int interp, int dtype, void *stream);
+                        mcx_plan_desc *desc, int64_t IH, int64_t IW, int64_t OH, int64_t OW,
+                        int64_t K, int64_t P, int interp, int dtype, void *stream);
+int mcx_conv_forward_planned(const void *x, const void *map, const void *iw, const void *w,
+                             const void *bias, void *y, void *workspace, size_t workspace_bytes,
+                             const void *plan, size_t plan_bytes, const mcx_plan_desc *desc,
+                             int64_t B, int64_t Ci, int64_t Co, int64_t IH, int64_t IW,
+                             int64_t OH, int64_t OW, int64_t K, int64_t P, int interp, int dtype,
+                             void *stream);
 int mcx_conv_backward_planned(const void *gy, const void *map, const void *iw, const void *x,
                               const void *w, void *gx, void *gw, void *gb, void *workspace,
                               size_t workspace_bytes, const void *plan, size_t plan_bytes,
-                               const mcx_plan_desc *desc,
+                              const mcx_plan_desc *desc, int64_t B, int64_t Ci, int64_t Co,
+                              int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P,
+                              int interp, int dtype, void *stream);
+int mcx_tconv_forward_planned(const void *x, const void *map, const void *iw, const void *w,
+                              const void *bias, void *y, void *workspace, size_t workspace_bytes,
+                              const void *plan, size_t plan_bytes, const mcx_plan_desc *desc,
                               int64_t B, int64_t Ci, int64_t Co, int64_t IH, int64_t IW,
                               int64_t OH, int64_t OW, int64_t K, int64_t P, int interp, int dtype,
                               void *stream);
+int mcx_tconv_backward_planned(const void *gy, const void *map, const void *iw, const void *x,
+                               const void *w, void *gx, void *gw, void *gb, void *workspace,
+                               size_t workspace_bytes, const void *plan, size_t plan_bytes,
+                               const mcx_plan_desc *desc, int64_t B, int64_t Ci, int64_t Co,
+                               int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
+                               int64_t P, int interp, int dtype, void *stream);
 
 /* Scatter plans: no counterpart in the reference.  resample_to_map and the two unpoolings run
  * as gathers through the transposed form of their sample map (per destination pixel the sorted
@@ -276,40 +292,21 @@ int mcx_conv_backward_planned(const void *gy, const void *map, const void *iw, c
 size_t mcx_scatter_plan_bytes(int64_t MH, int64_t MW, int64_t DH, int64_t DW, int64_t K, int64_t P,
                               int interp, int dtype);
 int mcx_scatter_plan_build(const void *map, const void *iw, void *plan, size_t plan_bytes,
-                           mcx_plan_desc *desc, int64_t MH, int64_t MW, int64_t DH, int64_t DW, int64_t K, int64_t P,
-                           int interp, int dtype, int for_max_unpool, void *stream);
+                           mcx_plan_desc *desc, int64_t MH, int64_t MW, int64_t DH, int64_t DW,
+                           int64_t K, int64_t P, int interp, int dtype, int for_max_unpool,
+                           void *stream);
 int mcx_resample_to_map_planned(const void *in, const void *plan, size_t plan_bytes,
-                                const mcx_plan_desc *desc, void *out,
-                                int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t OH,
-                                int64_t OW, int64_t P, int interp, int dtype, void *stream);
+                                const mcx_plan_desc *desc, void *out, int64_t B, int64_t C,
+                                int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t P,
+                                int interp, int dtype, void *stream);
 int mcx_avg_unpool_planned(const void *gout, const void *plan, size_t plan_bytes,
-                           const mcx_plan_desc *desc, void *gin,
-                           int64_t B, int64_t C, int64_t IH, int64_t IW, int64_t OH, int64_t OW,
-                           int64_t K, int64_t P, int interp, int dtype, void *stream);
-int mcx_max_unpool_planned(const void *gout, const int64_t *idx, const void *plan,
-                           size_t plan_bytes, const mcx_plan_desc *desc, void *gin, int64_t B, int64_t C, int64_t IH,
+                           const mcx_plan_desc *desc, void *gin, int64_t B, int64_t C, int64_t IH,
                            int64_t IW, int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
                            int dtype, void *stream);
-
-int mcx_conv_forward_planned(const void *x, const void *map, const void *iw, const void *w,
-                             const void *bias, void *y, void *workspace, size_t workspace_bytes,
-                             const void *plan, size_t plan_bytes, const mcx_plan_desc *desc,
-                              int64_t B, int64_t Ci,
-                             int64_t Co, int64_t IH, int64_t IW, int64_t OH, int64_t OW,
-                             int64_t K, int64_t P, int interp, int dtype, void *stream);
-int mcx_tconv_forward_planned(const void *x, const void *map, const void *iw, const void *w,
-                              const void *bias, void *y, void *workspace, size_t workspace_bytes,
-                              const void *plan, size_t plan_bytes, const mcx_plan_desc *desc,
-                              int64_t B, int64_t Ci,
-                              int64_t Co, int64_t IH, int64_t IW, int64_t OH, int64_t OW,
-                              int64_t K, int64_t P, int interp, int dtype, void *stream);
-int mcx_tconv_backward_planned(const void *gy, const void *map, const void *iw, const void *x,
-                               const void *w, void *gx, void *gw, void *gb, void *workspace,
-                               size_t workspace_bytes, const void *plan, size_t plan_bytes,
-                               const mcx_plan_desc *desc,
-                               int64_t B, int64_t Ci, int64_t Co, int64_t IH, int64_t IW,
-                               int64_t OH, int64_t OW, int64_t K, int64_t P, int interp,
-                               int dtype, void *stream);
+int mcx_max_unpool_planned(const void *gout, const int64_t *idx, const void *plan,
+                           size_t plan_bytes, const mcx_plan_desc *desc, void *gin, int64_t B,
+                           int64_t C, int64_t IH, int64_t IW, int64_t OH, int64_t OW, int64_t K,
+                           int64_t P, int interp, int dtype, void *stream);
 
 /* ---- KNN -------------------------------------------------------------------- */
 
