@@ -216,6 +216,46 @@ __global__ __launch_bounds__(256) void to_channel_blocks_kernel(const TD *__rest
   reinterpret_cast<Block *>(xt)[((int64_t)b * gridDim.y + g8) * plane + n] = v;
 }
 
+// y[b][a][pixel] -> yt[b][tile][a / 32][mb][s4][lane][8]: the plain operand of a weight gradient
+// cut into pixel tiles of 128 (tw_shift: the tile is (128 >> tw_shift) rows of 1 << tw_shift
+// pixels; pixels outside the image and channels past A are zeros) and, inside a tile, into the
+// MFMA fragments of weight_grad_bf16_ring_kernel: a slab is 32 channels, the rows of one wave;
+// fragment (mb, s4) holds, for lane (l15 = lane & 15, lq = lane >> 4), pixels 32 * s4 + 8 * lq
+// .. + 7 of channel 16 * mb + l15 of the slab.  A wave of that kernel then loads a fragment as
+// one contiguous kilobyte straight into its operand registers.
+// One workgroup: one slab of one tile through LDS (reads: 256-byte runs of a channel's row;
+// writes: the slab's 8 KB in one piece).  MW is a multiple of 8.
+__global__ __launch_bounds__(256) void to_plain_fragments_kernel(const bf16_t *__restrict__ y,
+                                                                 bf16_t *__restrict__ yt, int A,
+                                                                 int MH, int MW, int tiles_x,
+                                                                 int tiles_per_img, int tw_shift) {
+  __shared__ __attribute__((aligned(16))) uint16_t T[32][kTilePx + 8];
+  const int tile = blockIdx.x, slab = blockIdx.y, b = blockIdx.z;
+  const int tile_y = tile / tiles_x, tile_x = tile - tile_y * tiles_x;
+  const int px = (threadIdx.x & 15) * 8;
+  const int si = tile_y * (kTilePx >> tw_shift) + (px >> tw_shift);
+  const int sj = (tile_x << tw_shift) + (px & ((1 << tw_shift) - 1));
+  const bool inside = si < MH && sj < MW;
+  const int64_t N = (int64_t)MH * MW;
+#pragma unroll
+  for (int h = 0; h < 2; h++) {
+    const int row = h * 16 + (threadIdx.x >> 4), a = slab * 32 + row;
+    uint4 v = make_uint4(0u, 0u, 0u, 0u);
+    if (inside && a < A)
+      v = *reinterpret_cast<const uint4 *>(y + ((int64_t)b * A + a) * N + (int64_t)si * MW + sj);
+    *reinterpret_cast<uint4 *>(&T[row][px]) = v;
+  }
+  __syncthreads();
+  uint4 *dst = reinterpret_cast<uint4 *>(yt) +
+               (((int64_t)b * tiles_per_img + tile) * gridDim.y + slab) * 512;
+#pragma unroll
+  for (int h = 0; h < 2; h++) {
+    const int o = h * 256 + threadIdx.x;  // (mb, s4, lane)
+    const int mb = o >> 8, s4 = (o >> 6) & 3, lane = o & 63;
+    dst[o] = *reinterpret_cast<const uint4 *>(&T[mb * 16 + (lane & 15)][32 * s4 + 8 * (lane >> 4)]);
+  }
+}
+
 // LDS operand tiles of the gather-product kernel, double-buffered.
 template <typename TD, int OG>
 struct OperandTiles {  // fp32: samples S[chunk channel][pixel], weights Wt[chunk channel][o]
@@ -1449,6 +1489,45 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(
 //   * five taps per pass keep the accumulators at 80 registers, which leaves room for the
 //     rings at two workgroups per CU.
 // Partial sums leave in the layout of weight_grad_mfma_kernel.
+// The taps of a bilinear map resolved once for weight_grad_bf16_ring_kernel, in the order its
+// workgroups read them: table[tile of an image][tap][pixel of the tile][NA words of byte offsets into a
+// channel block (16 bytes per pixel), then NA words of weights as bf16 in the low half].  Every
+// workgroup of a pixel range (channel groups x tap passes) would otherwise resolve the same
+// taps from the map again, about a hundred instructions per tap, which is as much as its
+// products need.  Pixels outside the image weigh zero.  One workgroup per tile: its threads
+// walk the taps of their pixel two apart, so the tile's piece of the map stays in cache.
+template <int NA>
+__global__ __launch_bounds__(256) void resolve_tap_table_kernel(
+    const float *__restrict__ map, unsigned *__restrict__ table, int GH, int GW, int MH, int MW,
+    int K, int wrap, int tiles_x, int tw_shift, const int *__restrict__ pair_mask) {
+  if (pair_mask && (((unsigned)*pair_mask < (1u << 2)) != (NA == 2))) return;
+  const int tile = blockIdx.x, p = threadIdx.x & (kTilePx - 1);
+  const int tile_y = tile / tiles_x, tile_x = tile - tile_y * tiles_x;
+  const int gi = tile_y * (kTilePx >> tw_shift) + (p >> tw_shift);
+  const int gj = (tile_x << tw_shift) + (p & ((1 << tw_shift) - 1));
+  const bool live = gi < MH && gj < MW;
+  const int64_t n_g = (int64_t)min(gi, MH - 1) * MW + min(gj, MW - 1);
+  const float2 *entry = reinterpret_cast<const float2 *>(map) + n_g * K;
+  uint4 *out = reinterpret_cast<uint4 *>(table) + ((int64_t)tile * K * kTilePx + p) * (NA / 2);
+  // (a weight as bf16 in the low half of a word, the high half zero: the form
+  // v_dot2_f32_bf16 multiplies a word of two channels by to get the even one)
+  auto wbits = [](float w) {
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(floatx2{w, 0.f}, bf16x2));
+  };
+  for (int k = threadIdx.x >> 7; k < K; k += 2) {
+    const float2 xy = entry[k];
+    PairTap<4> t;
+    resolve_pairs<4, 16>(xy.x, xy.y, GH, GW, wrap != 0, live ? 1.f : 0.f, t);
+    uint4 *e = out + (int64_t)k * kTilePx * (NA / 2);
+    if constexpr (NA == 2) {
+      e[0] = make_uint4(t.off[0], t.off[1], wbits(t.wt[0]), wbits(t.wt[1]));
+    } else {
+      e[0] = make_uint4(t.off[0], t.off[1], t.off[2], t.off[3]);
+      e[1] = make_uint4(wbits(t.wt[0]), wbits(t.wt[1]), wbits(t.wt[2]), wbits(t.wt[3]));
+    }
+  }
+}
+
 constexpr int kRgKT = 5;      // taps per pass
 constexpr int kRgG = 32;      // gathered channels per workgroup
 constexpr int kRgA = 128;     // plain channels per workgroup
@@ -1469,10 +1548,9 @@ inline int ring_weight_grad_ranges(int64_t total_tiles, int64_t A, int64_t G, in
 template <int NA>
 __global__ __launch_bounds__(kThreads, 2) void weight_grad_bf16_ring_kernel(
     const bf16_t *__restrict__ plain, const bf16_t *__restrict__ gath,
-    const float *__restrict__ map, float *__restrict__ part, int A, int G, int Gpad, int GH,
-    int GW, int MH, int MW, int K, int wrap, int tiles_x, int tiles_per_img, int tw_shift,
-    int total_tiles, int ranges, int cgroups, int passes, float *__restrict__ plain_sum_part,
-    const int *__restrict__ pair_mask) {
+    const unsigned *__restrict__ table, float *__restrict__ part, int A, int G, int Gpad, int GH,
+    int GW, int K, int tiles_per_img, int total_tiles, int ranges, int cgroups, int passes,
+    float *__restrict__ plain_sum_part, const int *__restrict__ pair_mask) {
   // NA == 2 runs while no tap of the map uses a pair beyond its first two, NA == 4 otherwise
   if (pair_mask && (((unsigned)*pair_mask < (1u << 2)) != (NA == 2))) return;
   static_assert(NA == 2 || NA == 4, "two or four pairs per tap");
@@ -1480,7 +1558,6 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_bf16_ring_kernel(
   constexpr int kDepth = kCross ? kRgDepth : 1;  // units in flight
   constexpr int kTapBufs = kCross ? 2 : 1;
   constexpr int MB = kRgA / 64, NB = kRgG / 16;
-  __shared__ __attribute__((aligned(16))) uint16_t PtB[kRgA][kRgLd];
   __shared__ __attribute__((aligned(16))) uint16_t SB[2][kRgG][kRgLd];
   __shared__ __attribute__((aligned(16))) unsigned TapOff[kTapBufs][kRgKT][kTilePx][NA];
   __shared__ __attribute__((aligned(16))) float TapWt[kTapBufs][kRgKT][kTilePx][NA];
@@ -1498,19 +1575,17 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_bf16_ring_kernel(
   const int k_base = pass * kRgKT;
   const int tpr = (total_tiles + ranges - 1) / ranges;
   const int t_begin = range * tpr, t_end = min(total_tiles, t_begin + tpr);
-  const int tw_mask = (1 << tw_shift) - 1, th = kTilePx >> tw_shift;
-  const int N = MH * MW;
   const int64_t gplane = (int64_t)GH * GW;
   const int g_first = cg * kRgG;
 
-  // roles.  Tap resolution: pixel p, taps half, half + 2, ...  Gather: pixel pair pp, the
-  // wave's 8 channels.  Plain tile: 16 lanes per row of 128 pixels, 16 rows per step.
+  // roles.  Tap cache: pixel p, taps half, half + 2, ...  Gather: pixel pair pp, the
+  // wave's 8 channels.  Plain operand: the wave's own MFMA fragments, straight from memory.
   const int p = tid & (kTilePx - 1), half = tid >> 7;
   const int pp = lane;
   const int64_t group = min(g_first / 8 + wave, Gpad / 8 - 1);  // (past Gpad: not stored)
   constexpr int kTapsPerThread = (kRgKT + 1) / 2;
-  constexpr int kRowsPerStep = kThreads / 16, kSteps = kRgA / kRowsPerStep;
-  const int px0 = (tid & 15) * 8;
+  static_assert(MB == 2, "a wave's rows are one slab of to_plain_fragments_kernel");
+  const int slabs = (A + 31) / 32;
 
   floatx4 acc[kRgKT][NB][MB];
 #pragma unroll
@@ -1524,81 +1599,60 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_bf16_ring_kernel(
 #pragma unroll
   for (int mb = 0; mb < MB; mb++) plain_sum[mb] = 0.f;
 
-  uint4 raw[kSteps];
-  float2 mxy[kTapsPerThread];
+  // plain operand of this tile and of the next, by the tile's parity in the range
+  bf16x8 aregb[2][MB][4];
+  uint4 tapreg[kTapsPerThread][NA / 2];
   uint4 q[kDepth][2 * NA];  // [unit in flight][pixel of the pair * NA + pair of the tap]
 
   // (tiles past the range's end, which pad it to a whole number of ring periods, are fetched
   // as zeros and weigh zero; their addresses are those of the last tile)
-  auto tile_origin = [&](int tile, int &b, int &i0, int &j0) __attribute__((always_inline)) {
-    tile = min(tile, t_end - 1);
-    b = tile / tiles_per_img;
-    const int t_in = tile - b * tiles_per_img;
-    const int tile_y = t_in / tiles_x, tile_x = t_in - tile_y * tiles_x;
-    i0 = tile_y * th;
-    j0 = tile_x << tw_shift;
-  };
-  // (the plain operand of an image as a buffer: rows past the last channel lie beyond its end
-  // and read as zeros, like the pieces outside the image, which get an offset out of range;
-  // a piece of 8 pixels never straddles the image's edge because MW is a multiple of 8)
-  const unsigned plain_rows = (unsigned)min(A - a0, kRgA);
-  auto fetch_plain = [&](int tile) __attribute__((always_inline)) {
-    int b, i0, j0;
-    tile_origin(tile, b, i0, j0);
-    const int si = i0 + (px0 >> tw_shift), sj = j0 + (px0 & tw_mask);
+  // (`plain` is the copy to_plain_fragments_kernel made: the wave's slab of a tile is 8 KB,
+  // fragment (mb, s4) a kilobyte of it, a lane's piece 16 bytes; a slab past the last channel
+  // does not exist in the copy and a tile past the range's end is not to be read: both get a
+  // buffer of no bytes and read as zeros)
+  const int slab = blockIdx.y * (kRgA / 32) + wave;
+  auto fetch_plain = [&](int tile, const int SET) __attribute__((always_inline)) {
+    const bool live = tile < t_end && slab < slabs;
     const auto rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<bf16_t *>(plain + ((int64_t)b * A + a0) * N), (short)0,
-        (int)(plain_rows * (unsigned)N * 2u), 0x00020000);
-    const unsigned off = (si < MH && sj < MW && tile < t_end)
-                             ? ((unsigned)(tid >> 4) * (unsigned)N + (unsigned)(si * MW + sj)) * 2u
-                             : 0xffffff00u;
+        const_cast<bf16_t *>(plain + ((int64_t)min(tile, t_end - 1) * slabs + min(slab, slabs - 1)) * 4096),
+        (short)0, live ? 8192 : 0, 0x00020000);
 #pragma unroll
-    for (int r = 0; r < kSteps; r++)
-      raw[r] = __builtin_bit_cast(
-          uint4, __builtin_amdgcn_raw_buffer_load_b128(
-                     rsrc, (int)off, (int)((unsigned)(r * kRowsPerStep) * (unsigned)N * 2u), 0));
-  };
-  auto fetch_coords = [&](int tile) __attribute__((always_inline)) {
-    int b, i0, j0;
-    tile_origin(tile, b, i0, j0);
-    const int gi = min(i0 + (p >> tw_shift), MH - 1), gj = min(j0 + (p & tw_mask), MW - 1);
-    const int64_t n_g = (int64_t)gi * MW + gj;
+    for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-    for (int t = 0; t < kTapsPerThread; t++) {
-      const int k = min(k_base + half + 2 * t, K - 1);
-      mxy[t] = *reinterpret_cast<const float2 *>(map + (n_g * K + k) * 2);
-    }
+      for (int s4 = 0; s4 < 4; s4++)
+        aregb[SET][mb][s4] = __builtin_bit_cast(
+            bf16x8, __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane * 16, (mb * 4 + s4) * 1024, 0));
   };
-  // taps of `tile`, from the coordinates fetch_coords(tile) brought, into half `par` of the
-  // tap cache: byte offsets into a channel block (16 bytes per pixel) and weights; pixels
-  // outside the image and taps past the last one weigh zero
-  auto resolve_taps = [&](int tile, int par) __attribute__((always_inline)) {
-    int b, i0, j0;
-    tile_origin(tile, b, i0, j0);
-    const bool live = i0 + (p >> tw_shift) < MH && j0 + (p & tw_mask) < MW && tile < t_end;
+  // Entries of `tile` from the table resolve_tap_table_kernel made, into registers: the taps
+  // of this pass as a buffer, so that taps past the map's last one and tiles past the range's
+  // end read as zeros (offset 0, weight 0).
+  auto fetch_taps = [&](int tile) __attribute__((always_inline)) {
+    const int taps = tile < t_end ? min(kRgKT, K - k_base) : 0;
+    const int t_in = min(tile, t_end - 1) % tiles_per_img;
+    const auto rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<unsigned *>(table + ((int64_t)t_in * K + k_base) * kTilePx * 2 * NA),
+        (short)0, taps * kTilePx * 8 * NA, 0x00020000);
+#pragma unroll
+    for (int t = 0; t < kTapsPerThread; t++)
+#pragma unroll
+      for (int h = 0; h < NA / 2; h++)
+        tapreg[t][h] = __builtin_bit_cast(
+            uint4, __builtin_amdgcn_raw_buffer_load_b128(
+                       rsrc, ((half + 2 * t) * kTilePx + p) * 8 * NA + 16 * h, 0, 0));
+  };
+  // what fetch_taps brought, into half `par` of the tap cache
+  auto store_taps = [&](int par) __attribute__((always_inline)) {
 #pragma unroll
     for (int t = 0; t < kTapsPerThread; t++) {
       const int k = half + 2 * t;
       if (k < kRgKT) {
-        PairTap<4> tp;
-        resolve_pairs<4, 16>(mxy[t].x, mxy[t].y, GH, GW, wrap != 0,
-                             (live && k_base + k < K) ? 1.f : 0.f, tp);
-        // (weights are kept as bf16 in the low half of a word, the high half zero: the form
-        // v_dot2_f32_bf16 multiplies a word of two channels by to get the even one)
-        auto wbits = [](float w) {
-          return __builtin_bit_cast(
-              float, __builtin_bit_cast(unsigned,
-                                        __builtin_convertvector(floatx2{w, 0.f}, bf16x2)));
-        };
         if constexpr (NA == 2) {
-          *reinterpret_cast<uint2 *>(&TapOff[par][k][p][0]) = make_uint2(tp.off[0], tp.off[1]);
-          *reinterpret_cast<float2 *>(&TapWt[par][k][p][0]) =
-              make_float2(wbits(tp.wt[0]), wbits(tp.wt[1]));
+          const uint4 e = tapreg[t][0];
+          *reinterpret_cast<uint2 *>(&TapOff[par][k][p][0]) = make_uint2(e.x, e.y);
+          *reinterpret_cast<uint2 *>(&TapWt[par][k][p][0]) = make_uint2(e.z, e.w);
         } else {
-          *reinterpret_cast<uint4 *>(&TapOff[par][k][p][0]) =
-              make_uint4(tp.off[0], tp.off[1], tp.off[2], tp.off[3]);
-          *reinterpret_cast<float4 *>(&TapWt[par][k][p][0]) =
-              make_float4(wbits(tp.wt[0]), wbits(tp.wt[1]), wbits(tp.wt[2]), wbits(tp.wt[3]));
+          *reinterpret_cast<uint4 *>(&TapOff[par][k][p][0]) = tapreg[t][0];
+          *reinterpret_cast<uint4 *>(&TapWt[par][k][p][0]) = tapreg[t][1];
         }
       }
     }
@@ -1675,33 +1729,25 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_bf16_ring_kernel(
     constexpr int PHASE = decltype(phase_tag)::value;
     // (kCross: `mxy` holds the coordinates of the next tile, whose taps go to the other half
     // of the cache; else those of this tile, resolved now)
+    constexpr int SET = PHASE & 1;
     const int par = kCross ? (tile - t_begin) & 1 : 0;
-    __syncthreads();  // the previous tile's plain operand and the tap cache to be written are free
-#pragma unroll
-    for (int r = 0; r < kSteps; r++)
-      *reinterpret_cast<uint4 *>(&PtB[(tid >> 4) + r * kRowsPerStep][px0]) = raw[r];
-    if constexpr (kCross)
-      resolve_taps(tile + 1, par ^ 1);
-    else
-      resolve_taps(tile, 0);
-    __syncthreads();
-    bf16x8 aregb[MB][4];
-#pragma unroll
-    for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-      for (int s4 = 0; s4 < 4; s4++)
-        aregb[mb][s4] = __builtin_bit_cast(
-            bf16x8, *reinterpret_cast<const uint4 *>(
-                        &PtB[(wave * MB + mb) * 16 + l15][32 * s4 + 8 * lq]));
-    if (sum_plain) {  // thread (row tid/4 of each 64, quarter tid%4) adds 32 pixels of its row
+    if constexpr (kCross) {
+      // (`tapreg` holds the next tile's taps; the half of the tap cache written here was last
+      // read before the previous tile's last barrier, and is first read after this tile's
+      // next one)
+      store_taps(par ^ 1);
+    } else {
+      __syncthreads();  // the tap cache is free
+      store_taps(0);  // (`tapreg` holds this tile's taps)
+      __syncthreads();
+    }
+    if (sum_plain) {  // the lane adds the 32 pixels it holds of each of its rows
 #pragma unroll
       for (int mb = 0; mb < MB; mb++) {
-        const uint4 *row =
-            reinterpret_cast<const uint4 *>(&PtB[64 * mb + (tid >> 2)][(tid & 3) * 32]);
         float t = 0.f;
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-          const uint4 v = row[r];
+        for (int s4 = 0; s4 < 4; s4++) {
+          const uint4 v = __builtin_bit_cast(uint4, aregb[SET][mb][s4]);
           const unsigned w4[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
           for (int j = 0; j < 4; j++)
@@ -1713,8 +1759,8 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_bf16_ring_kernel(
     }
     const auto base = gather_base(tile), base_next = gather_base(tile + 1);
     if constexpr (!kCross) issue(base, 0, 0, 0);  // (before the prefetches: it is waited for first)
-    fetch_plain(tile + 1);
-    fetch_coords(kCross ? tile + 2 : tile + 1);
+    fetch_plain(tile + 1, SET ^ 1);
+    fetch_taps(kCross ? tile + 2 : tile + 1);
 #pragma unroll
     for (int k = 0; k < kRgKT; k++) {
       const int slot_k = (PHASE * kRgKT + k) % kDepth;
@@ -1734,7 +1780,7 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_bf16_ring_kernel(
               *reinterpret_cast<const uint4 *>(&SB[buf][nb * 16 + l15][32 * s4 + 8 * lq]));
 #pragma unroll
           for (int mb = 0; mb < MB; mb++)
-            acc[k][nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aregb[mb][s4], bq,
+            acc[k][nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aregb[SET][mb][s4], bq,
                                                                      acc[k][nb][mb], 0, 0, 0);
         }
     }
@@ -1742,13 +1788,13 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_bf16_ring_kernel(
 
   // prologue: taps of the first tile, its plain operand, coordinates of the second, and the
   // gathers of the first kRgDepth units (a range without tiles stores its zeros)
-  static_assert(kRgDepth == 2 || kRgDepth == 3, "run_tile is instantiated per phase below");
+  static_assert(kRgDepth == 2, "run_tile is instantiated per phase below");
   if (t_begin < t_end) {
-    fetch_coords(t_begin);
+    fetch_taps(t_begin);
     if constexpr (kCross) {
-      resolve_taps(t_begin, 0);
-      fetch_plain(t_begin);
-      fetch_coords(t_begin + 1);
+      store_taps(0);
+      fetch_plain(t_begin, 0);
+      fetch_taps(t_begin + 1);
       __syncthreads();
       const auto base0 = gather_base(t_begin);
 #pragma unroll
@@ -1756,23 +1802,25 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_bf16_ring_kernel(
       for (int tile = t_begin; tile < t_end; tile += kDepth) {
         run_tile(std::integral_constant<int, 0>(), tile);
         run_tile(std::integral_constant<int, 1>(), tile + 1);
-        if constexpr (kDepth == 3) run_tile(std::integral_constant<int, 2>(), tile + 2);
       }
     } else {
-      fetch_plain(t_begin);
-      for (int tile = t_begin; tile < t_end; ++tile)
+      // (two tiles per turn for the two sets of plain operands; a tile past the end weighs zero)
+      fetch_plain(t_begin, 0);
+      for (int tile = t_begin; tile < t_end; tile += 2) {
         run_tile(std::integral_constant<int, 0>(), tile);
+        run_tile(std::integral_constant<int, 1>(), tile + 1);
+      }
     }
   }
 
-  if (sum_plain) {  // the four quarters of a row sit in neighbouring lanes
+  if (sum_plain) {  // the four quarters of a row sit 16 lanes apart
 #pragma unroll
     for (int mb = 0; mb < MB; mb++) {
       float t = plain_sum[mb];
-      t += __shfl_xor(t, 1);
-      t += __shfl_xor(t, 2);
-      const int a = a0 + 64 * mb + (tid >> 2);
-      if ((tid & 3) == 0 && a < A) plain_sum_part[(int64_t)range * A + a] = t;
+      t += __shfl_xor(t, 16);
+      t += __shfl_xor(t, 32);
+      const int a = a0 + (wave * MB + mb) * 16 + l15;
+      if (lq == 0 && a < A) plain_sum_part[(int64_t)range * A + a] = t;
     }
   }
   const int A4 = (A + 3) & ~3;
@@ -2502,6 +2550,14 @@ size_t mfma_weight_grad_bytes(int64_t B, int64_t A, int64_t G, int64_t MH, int64
     n += align256((size_t)(B * GH * GW * round_up(G, kGC)) * sizeof(float));
   else if (elem == 2)
     n += align256((size_t)(B * GH * GW * round_up(G, kGC)) * elem);
+  // bf16 images: the plain operand as MFMA fragments per pixel tile (to_plain_fragments_kernel)
+  // and the table of resolved taps (resolve_tap_table_kernel, four pairs per tap at most)
+  if (GH > 1 && elem == 2) {
+    const size_t tiles = (size_t)make_tiling(B, MH, MW, 2).total;
+    n += align256(tiles * (size_t)round_up(A, 32) * kTilePx * elem);
+    n += align256((size_t)make_tiling(B, MH, MW, 2).tiles_per_img * (size_t)K * kTilePx * 8 *
+                  sizeof(unsigned));
+  }
   return n;
 }
 
@@ -2527,10 +2583,10 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
   // lets one of the two launches run)
   // (its 16-byte pieces of the plain operand want rows that are a multiple of 8 pixels, and
   // an image of either operand is addressed as a buffer of less than 4 GiB)
-  const bool ring = sizeof(TD) == 2 && !cl && m.np == 1 && m.mode != kInterpNearest &&
+  const bool ring = sizeof(TD) == 2 && !cl && GH > 1 && m.np == 1 && m.mode != kInterpNearest &&
                     GH * GW * 16 < 0xffffff00LL && MW % 8 == 0 &&
-                    (reinterpret_cast<uintptr_t>(plain) & 15) == 0 &&
-                    (int64_t)kRgA * MH * MW * 2 < 0xffffff00LL;
+                    (reinterpret_cast<uintptr_t>(plain) & 15) == 0 && B <= 65535 &&
+                    A <= 32 * 65535;
   const int ranges = ring ? ring_weight_grad_ranges(t.total, A, G, K)
                           : weight_grad_ranges<TD>(t.total, A, G, K);
   float *sum_part = reinterpret_cast<float *>(
@@ -2586,6 +2642,25 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
     if (ring) {
       TD *stage = reinterpret_cast<TD *>((char *)pair_mask_ws + 256);
       if (int rc = launch_channel_blocks<TD>(gath, stage, B, G, GH * GW, s)) return rc;
+      // the plain operand tile by tile, after the blocks of the gathered one
+      bf16_t *tiles = reinterpret_cast<bf16_t *>(
+          (char *)stage + align256((size_t)(B * GH * GW * Gpad) * sizeof(TD)));
+      hipLaunchKernelGGL(to_plain_fragments_kernel,
+                         dim3((unsigned)t.tiles_per_img, (unsigned)((A + 31) / 32), (unsigned)B),
+                         dim3(256), 0, s, reinterpret_cast<const bf16_t *>(plain), tiles, (int)A,
+                         (int)MH, (int)MW, t.tiles_x, t.tiles_per_img, t.tw_shift);
+      MCX_HIP_CHECK_LAUNCH();
+      // the taps, resolved once for all workgroups (two or four pairs: the mask decides)
+      unsigned *table = reinterpret_cast<unsigned *>(
+          (char *)tiles + align256((size_t)t.total * (size_t)round_up(A, 32) * kTilePx * sizeof(TD)));
+      const dim3 rgrid((unsigned)t.tiles_per_img);
+      hipLaunchKernelGGL(resolve_tap_table_kernel<2>, rgrid, dim3(256), 0, s, map, table, (int)GH,
+                         (int)GW, (int)MH, (int)MW, (int)K, m.wrap, t.tiles_x, t.tw_shift,
+                         pair_mask);
+      hipLaunchKernelGGL(resolve_tap_table_kernel<4>, rgrid, dim3(256), 0, s, map, table, (int)GH,
+                         (int)GW, (int)MH, (int)MW, (int)K, m.wrap, t.tiles_x, t.tw_shift,
+                         pair_mask);
+      MCX_HIP_CHECK_LAUNCH();
     }
   }
   profile_begin(s);
@@ -2596,11 +2671,19 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
   hipLaunchKernelGGL(weight_grad_bf16_ring_kernel<NA>,                                            \
                      dim3((unsigned)(ranges * rg_groups * rg_passes),                             \
                           (unsigned)((A + kRgA - 1) / kRgA)),                                     \
-                     dim3(kThreads), 0, s, plain,                                                 \
-                     reinterpret_cast<const TD *>((char *)pair_mask_ws + 256), map, part, (int)A, \
-                     (int)G, (int)Gpad, (int)GH, (int)GW, (int)MH, (int)MW, (int)K, m.wrap,       \
-                     t.tiles_x, t.tiles_per_img, t.tw_shift, (int)t.total, ranges, rg_groups,     \
-                     rg_passes, plain_sum ? sum_part : (float *)nullptr, pair_mask)
+                     dim3(kThreads), 0, s,                                                        \
+                     reinterpret_cast<const TD *>(                                                \
+                         (char *)pair_mask_ws + 256 +                                             \
+                         align256((size_t)(B * GH * GW * Gpad) * sizeof(TD))),                    \
+                     reinterpret_cast<const TD *>((char *)pair_mask_ws + 256),                    \
+                     reinterpret_cast<const unsigned *>(                                          \
+                         (char *)pair_mask_ws + 256 +                                             \
+                         align256((size_t)(B * GH * GW * Gpad) * sizeof(TD)) +                    \
+                         align256((size_t)t.total * (size_t)round_up(A, 32) * kTilePx *           \
+                                  sizeof(TD))),                                                   \
+                     part, (int)A, (int)G, (int)Gpad, (int)GH, (int)GW, (int)K, t.tiles_per_img,  \
+                     (int)t.total, ranges, rg_groups, rg_passes,                                  \
+                     plain_sum ? sum_part : (float *)nullptr, pair_mask)
       MCX_LAUNCH_RING(2);
       MCX_LAUNCH_RING(4);
 #undef MCX_LAUNCH_RING
