@@ -35,7 +35,7 @@ int fill_bias(T *y, const T *bias, int64_t B, int64_t C, int64_t N, hipStream_t 
 struct bf16_t;
 bool mfma_supported(int64_t P);
 size_t mfma_gather_product_bytes(int64_t O, int64_t G, int64_t K, int64_t B, int64_t SH,
-                                 int64_t SW, int elem);
+                                 int64_t SW, int elem, int64_t MH, int64_t MW);
 template <typename TD>
 int mfma_gather_product(const TD *src, const float *map, const float *iw, const TD *w,
                         const TD *bias, TD *y, void *scratch, int64_t B, int64_t G, int64_t O,

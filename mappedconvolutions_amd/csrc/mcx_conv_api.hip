@@ -98,9 +98,12 @@ template <>
 int fill_zero<double>(double *p, int64_t n, hipStream_t s) { return fill_f64(p, n, 0.0, s); }
 
 // ---- scratch sizes of the three operators -------------------------------------------
+// SH x SW: the image sampled; MH x MW: the map
 size_t gather_product_ws(int dtype, int64_t G, int64_t O, int64_t K, int64_t P, int64_t B,
-                         int64_t SH, int64_t SW) {
-  return use_mfma(dtype, P) ? mfma_gather_product_bytes(O, G, K, B, SH, SW, (int)elem_size(dtype)) : 0;
+                         int64_t SH, int64_t SW, int64_t MH, int64_t MW) {
+  return use_mfma(dtype, P)
+             ? mfma_gather_product_bytes(O, G, K, B, SH, SW, (int)elem_size(dtype), MH, MW)
+             : 0;
 }
 size_t weight_grad_ws(int dtype, int64_t B, int64_t A, int64_t G, int64_t MH, int64_t MW,
                       int64_t K, int64_t P, int64_t GH, int64_t GW) {
@@ -199,7 +202,8 @@ int gather_product<float>(bool mfma, const void *src, const void *map, const voi
     return generic_gather_product<float>((const float *)src, (const float *)map,
                                          (const float *)iw, (const float *)w, (const float *)bias,
                                          (float *)y, B, G, O, SH, SW, MH * MW, K, P, interp, s);
-  if (!ws || ws_bytes < mfma_gather_product_bytes(O, G, K, B, SH, SW, 4)) return MCX_E_WORKSPACE;
+  if (!ws || ws_bytes < mfma_gather_product_bytes(O, G, K, B, SH, SW, 4, MH, MW))
+    return MCX_E_WORKSPACE;
   return mfma_gather_product<float>((const float *)src, (const float *)map, (const float *)iw,
                                     (const float *)w, (const float *)bias, (float *)y, ws, B, G, O,
                                     SH, SW, MH, MW, K, P, interp, s, plan);
@@ -258,7 +262,8 @@ int gather_product<bf16_t>(bool mfma, const void *src, const void *map, const vo
                            int64_t MW, int64_t K, int64_t P, int interp, hipStream_t s,
                            const void *plan) {
   if (!mfma) return MCX_E_DTYPE;
-  if (!ws || ws_bytes < mfma_gather_product_bytes(O, G, K, B, SH, SW, 2)) return MCX_E_WORKSPACE;
+  if (!ws || ws_bytes < mfma_gather_product_bytes(O, G, K, B, SH, SW, 2, MH, MW))
+    return MCX_E_WORKSPACE;
   return mfma_gather_product<bf16_t>((const bf16_t *)src, (const float *)map, (const float *)iw,
                                      (const bf16_t *)w, (const bf16_t *)bias, (bf16_t *)y, ws, B,
                                      G, O, SH, SW, MH, MW, K, P, interp, s, plan);
@@ -362,9 +367,9 @@ int tconv_backward_t(bool mfma, const void *gy, const void *map, const void *iw,
 }  // namespace
 
 extern "C" size_t mcx_conv_forward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t IH,
-                                             int64_t IW, int64_t, int64_t, int64_t K, int64_t P,
-                                             int dtype) {
-  return gather_product_ws(dtype, Ci, Co, K, P, B, IH, IW);
+                                             int64_t IW, int64_t OH, int64_t OW, int64_t K,
+                                             int64_t P, int dtype) {
+  return gather_product_ws(dtype, Ci, Co, K, P, B, IH, IW, OH, OW);
 }
 
 extern "C" int mcx_conv_forward(const void *x, const void *map, const void *iw, const void *w,
@@ -394,7 +399,7 @@ extern "C" int mcx_conv_forward_static(const void *x, const void *map, const voi
   if (int rc = check_ptrs(x, map, iw, w, P)) return rc;
   if (!bias || !y) return MCX_E_NULL;
   if (dtype != MCX_F32 && dtype != MCX_F64 && dtype != MCX_BF16) return MCX_E_DTYPE;
-  const size_t need = gather_product_ws(dtype, Ci, Co, K, P, B, IH, IW);
+  const size_t need = gather_product_ws(dtype, Ci, Co, K, P, B, IH, IW, OH, OW);
   if (need > kStaticScratchBytes) return MCX_E_STATIC_LIMIT;
   int rc = 0;
   void *ws = static_scratch_of_current_device(&rc);
@@ -581,7 +586,7 @@ extern "C" size_t mcx_tconv_backward_workspace(int64_t B, int64_t Ci, int64_t Co
                                                int64_t P, int dtype) {
   // backward-input is a gather-product with the channel roles swapped; the
   // gradients run one after the other and share the scratch
-  return std::max({gather_product_ws(dtype, Co, Ci, K, P, B, OH, OW),
+  return std::max({gather_product_ws(dtype, Co, Ci, K, P, B, OH, OW, IH, IW),
                    weight_grad_ws(dtype, B, Ci, Co, IH, IW, K, P, OH, OW),
                    bias_grad_ws(dtype, B, Co, OH * OW)});
 }

@@ -2451,6 +2451,19 @@ int launch_pair_mask(const float *map, const float *iw, int *mask, const ModeArg
 namespace {
 constexpr int kPlanSlots = 4;  // resolved entries per (location, tap) of a plan's gather part
 bool gather_plan_applies(int interp, int64_t P);
+template <int NCORN>
+__global__ void build_gather_plan_kernel(const float *__restrict__ map,
+                                         const float *__restrict__ iw, float2 *__restrict__ gmap,
+                                         int np, int weighted, int wrap, int SH, int SW, int K,
+                                         int64_t total);
+// bf16 images under single-point bilinear taps: a forward call without a plan resolves the
+// taps once into the same form before its product (a tenth of a millisecond where the product
+// kernel would spend four resolving them tile by tile)
+inline bool resolves_per_call(size_t elem, int64_t SH, int interp, int64_t P, int64_t MH,
+                              int64_t MW, int64_t K) {
+  return elem == 2 && SH > 1 && canonical_interp(interp) != kInterpNearest && P <= 1 &&
+         MH * MW * K * kPlanSlots * 2 <= 0x7fffffffLL;
+}
 }  // namespace
 size_t mfma_gather_plan_offset(int64_t DH, int64_t DW, int64_t MH, int64_t MW, int64_t K,
                                int64_t P);
@@ -2459,11 +2472,14 @@ size_t mfma_gather_plan_offset(int64_t DH, int64_t DW, int64_t MH, int64_t MW, i
 // Packed weights, then (single-row sources) the channel-last copy of the source, sized
 // for 4-byte elements.
 size_t mfma_gather_product_bytes(int64_t O, int64_t G, int64_t K, int64_t B, int64_t SH,
-                                 int64_t SW, int elem) {
+                                 int64_t SW, int elem, int64_t MH, int64_t MW) {
   size_t n = align256((size_t)(K * round_up(G, kGC) * round_up(O, kOT)) * sizeof(float));
   n += 256;  // the map's pair mask
   if (SH == 1 || elem == 2)
     n += align256((size_t)(B * SH * SW * round_up(G, kGC)) * sizeof(float));
+  // the taps resolved per call (whatever the interpolation will be: it is not known here)
+  if (resolves_per_call((size_t)elem, SH, kInterpBilinear, 1, MH, MW, K))
+    n += align256((size_t)(MH * MW * K) * kPlanSlots * sizeof(float2));
   return n;
 }
 
@@ -2478,9 +2494,8 @@ int mfma_gather_product(const TD *src, const float *map, const float *iw, const 
   // resolved measured the same within 1 %, so there only the plan's pair mask is used and the
   // 32 bytes per tap of the resolved form are not read; single-row sources and bf16 storage
   // gain from the resolved form)
-  // (bf16 images under single-point bilinear taps read pair words, which beats both)
   const bool resolved_pays =
-      !(SH > 1 && canonical_interp(interp) != kInterpNearest && (sizeof(TD) == 4 || P <= 1));
+      !(SH > 1 && canonical_interp(interp) != kInterpNearest && sizeof(TD) == 4);
   if (plan && resolved_pays && gather_plan_applies(interp, P) &&
       OH * OW * K * kPlanSlots * 2 <= 0x7fffffffLL) {
     // the map's taps were resolved when the plan was built: read them as four pre-resolved
@@ -2506,6 +2521,22 @@ int mfma_gather_product(const TD *src, const float *map, const float *iw, const 
                                            : nullptr;
   const ModeArgs m = mode_args(interp, P);
   const bool four_pairs = m.np * (m.mode == kInterpNearest ? 1 : 4) == 4;
+  if (!plan && resolves_per_call(sizeof(TD), SH, interp, P, OH, OW, K)) {
+    float2 *gmap = reinterpret_cast<float2 *>(
+        (char *)stage + align256((size_t)(B * SH * SW * round_up(G, kGC)) * sizeof(float)));
+    if (int rc = launch_pack_weights<TD>(w, wp, O, G, K, 0, s, pair_mask)) return rc;
+    if (int rc = launch_pair_mask(map, iw, pair_mask, m, SH, SW, OH * OW * K, s, true)) return rc;
+    const int64_t total = OH * OW * K;
+    hipLaunchKernelGGL(build_gather_plan_kernel<4>,
+                       dim3((unsigned)(((OH * OW + 63) / 64 * 64 * K + 255) / 256)), dim3(256), 0,
+                       s, map, iw, gmap, m.np, m.weighted, m.wrap, (int)SH, (int)SW, (int)K,
+                       total);
+    MCX_HIP_CHECK_LAUNCH();
+    return launch_gather_product<TD>(src, reinterpret_cast<const float *>(gmap), nullptr, wp, bias,
+                                     y, stage, B, G, O, SH, SW, OH, OW, K, kPlanSlots,
+                                     kInterpNearest, nullptr, 0, s, nullptr, false, pair_mask,
+                                     true);
+  }
   const int *mask = pair_mask;
   // the pair mask of a small map is made by the last block of the packing launch
   const bool mask_on_pack = four_pairs && !plan && OH * OW * K <= kSmallMapEntries;
@@ -2915,8 +2946,14 @@ __global__ void build_gather_plan_kernel(const float *__restrict__ map,
                                          const float *__restrict__ iw, float2 *__restrict__ gmap,
                                          int np, int weighted, int wrap, int SH, int SW, int K,
                                          int64_t total) {
-  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // (location, tap)
-  if (e >= total) return;
+  // (a wave takes 64 consecutive locations of one tap: its stores are 512-byte runs)
+  const int64_t t0 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t run = t0 / (64 * (int64_t)K), pixels = total / K;
+  const int r = (int)(t0 - run * 64 * K);
+  const int64_t n = run * 64 + (r & 63);
+  const int k = r >> 6;
+  if (n >= pixels) return;
+  const int64_t e = n * K + k;  // (location, tap)
   float2 out[kTransSlotsConst];
 #pragma unroll
   for (int i = 0; i < kTransSlotsConst; i++) out[i] = make_float2(0.f, 0.f);
@@ -2930,9 +2967,9 @@ __global__ void build_gather_plan_kernel(const float *__restrict__ map,
       if (sp * NCORN + i < kTransSlotsConst)
         out[sp * NCORN + i] = make_float2(__builtin_bit_cast(float, t.off[i]), t.wt[i]);
   }
-  const int64_t n = e / K, k = e % K, pixels = total / K;  // stored [tap][slot][location]
 #pragma unroll
-  for (int i = 0; i < kTransSlotsConst; i++) gmap[(k * kTransSlotsConst + i) * pixels + n] = out[i];
+  for (int i = 0; i < kTransSlotsConst; i++)  // stored [tap][slot][location]
+    gmap[((int64_t)k * kTransSlotsConst + i) * pixels + n] = out[i];
 }
 
 // A map has a gather part when a tap is at most four (offset, weight) pairs.
@@ -3070,7 +3107,7 @@ int mfma_scatter_plan_build(const float *map, const float *iw, void *plan, int64
   if (gather_plan_applies(interp, P) && MH * MW * K * kTransSlots * 2 <= 0x7fffffffLL) {
     float2 *gmap = (float2 *)((char *)plan + mfma_gather_plan_offset(DH, DW, MH, MW, K, P));
     const int64_t total = MH * MW * K;
-    const dim3 grid((unsigned)((total + 255) / 256));
+    const dim3 grid((unsigned)(((MH * MW + 63) / 64 * 64 * K + 255) / 256));
     if (m.mode == kInterpNearest)
       hipLaunchKernelGGL(build_gather_plan_kernel<1>, grid, dim3(256), 0, s, map, iw, gmap, m.np,
                          m.weighted, m.wrap, (int)DH, (int)DW, (int)K, total);
