@@ -122,6 +122,15 @@ __device__ inline float dot_bf16(unsigned word, unsigned w, float acc) {
                                          __builtin_bit_cast(bf16x2, w), acc, false);
 }
 
+// w.lo * word.lo + w.hi * word.hi, the head of such a sum.  (Written out because the compiler
+// renders dot_bf16(word, w, 0) as the accumulating two-operand form behind a move of zero:
+// one instruction in three of an interpolation.)
+__device__ inline float dot_bf16_first(unsigned word, unsigned w) {
+  float r;
+  asm("v_dot2_f32_bf16 %0, %1, %2, 0" : "=v"(r) : "v"(word), "v"(w));
+  return r;
+}
+
 template <typename TD>
 __global__ __launch_bounds__(256) void pack_weights_kernel(
     const TD *__restrict__ w, void *__restrict__ packed_out, int O, int G, int K, int Opad,
@@ -882,8 +891,6 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_bf16_direct_kernel
       for (int q = 0; q < 2; q++) {
         float sv[8];
 #pragma unroll
-        for (int ch = 0; ch < 8; ch++) sv[ch] = 0.f;
-#pragma unroll
         for (int r = 0; r < NPR; r++) {
           // a word of an entry holds channels 2j (low half) and 2j + 1 of its pixel: against
           // {w, 0} the dot product weighs the even channel, against {0, w} the odd one
@@ -895,8 +902,13 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_bf16_direct_kernel
 #pragma unroll
             for (int j = 0; j < 4; j++) {
               const unsigned word = ring[d][q][2 * r + e][j];
-              sv[2 * j] = dot_bf16(word, w_even[e], sv[2 * j]);
-              sv[2 * j + 1] = dot_bf16(word, w_odd[e], sv[2 * j + 1]);
+              if (r == 0 && e == 0) {
+                sv[2 * j] = dot_bf16_first(word, w_even[e]);
+                sv[2 * j + 1] = dot_bf16_first(word, w_odd[e]);
+              } else {
+                sv[2 * j] = dot_bf16(word, w_even[e], sv[2 * j]);
+                sv[2 * j + 1] = dot_bf16(word, w_odd[e], sv[2 * j + 1]);
+              }
             }
         }
         u32x4 pk;
@@ -1702,15 +1714,20 @@ __global__ __launch_bounds__(kThreads, 2) void weight_grad_bf16_ring_kernel(
     }
 #pragma unroll
     for (int j = 0; j < 4; j++) {  // channels 2j and 2j + 1 of the wave's eight
-      float e[2] = {0.f, 0.f}, o[2] = {0.f, 0.f};  // [pixel of the pair]
+      float e[2], o[2];  // [pixel of the pair]
 #pragma unroll
       for (int px = 0; px < 2; px++)
 #pragma unroll
         for (int i = 0; i < NA; i++) {  // in the order of the pairs, like every other kernel
           const uint4 t = q[SLOT][px * NA + i];
           const unsigned word = j == 0 ? t.x : j == 1 ? t.y : j == 2 ? t.z : t.w;
-          e[px] = dot_bf16(word, w_even[px * NA + i], e[px]);
-          o[px] = dot_bf16(word, w_odd[px * NA + i], o[px]);
+          if (i == 0) {
+            e[px] = dot_bf16_first(word, w_even[px * NA]);
+            o[px] = dot_bf16_first(word, w_odd[px * NA]);
+          } else {
+            e[px] = dot_bf16(word, w_even[px * NA + i], e[px]);
+            o[px] = dot_bf16(word, w_odd[px * NA + i], o[px]);
+          }
         }
       // (hardware round-to-nearest-even, the two pixels of a channel in one word)
       *reinterpret_cast<unsigned *>(&SB[buf][wave * 8 + 2 * j][2 * pp]) =
