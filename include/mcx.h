@@ -156,8 +156,8 @@ int mcx_conv_forward_static(const void *x, const void *map, const void *iw, cons
                             int interp, int dtype, void *stream);
 
 /* Bytes of device scratch the matching call needs for these sizes (may be 0).
- * The scratch holds repacked weights and partial sums; its contents need not
- * survive the call.  It must be 256-byte aligned. */
+ * The scratch holds repacked weights, partial sums, staging copies of operands and
+ * resolved taps; its contents need not survive the call.  It must be 256-byte aligned. */
 size_t mcx_conv_forward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t IH, int64_t IW,
                                   int64_t OH, int64_t OW, int64_t K, int64_t P, int dtype);
 size_t mcx_conv_backward_workspace(int64_t B, int64_t Ci, int64_t Co, int64_t IH, int64_t IW,

@@ -1490,20 +1490,27 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(
 //     four lanes per clock whatever the width), and a channel's two pixels leave as one
 //     32-bit LDS store, consecutive lanes to consecutive banks;
 //   * NA == 2: the loads of kRgDepth units are in flight, across tile boundaries: the taps of
-//     the next tile are resolved (into the other half of a double-buffered tap cache) and the
-//     next plain tile is fetched into registers while this tile's units are multiplied, so
-//     that in the steady state no wave waits for memory at a tile's start.  NA == 4 has twice
-//     the loads per unit and the same registers: one unit in flight (the next unit's loads are
-//     issued before this unit's products), a single tap cache, the first unit of a tile waited
-//     for;
+//     the next tile go into the other half of a double-buffered tap cache and the next tile's
+//     plain operand is fetched into a second set of registers while this tile's units are
+//     multiplied, so that in the steady state no wave waits for memory at a tile's start.
+//     NA == 4 has twice the loads per unit and the same registers: one unit in flight (the
+//     next unit's loads are issued before this unit's products), a single tap cache, the first
+//     unit of a tile waited for;
 //   * every load and store is unconditional (past the range's last tile the last one is
 //     fetched again, padded taps weigh zero), so the compiler's waits count exactly;
 //   * five taps per pass keep the accumulators at 80 registers, which leaves room for the
-//     rings at two workgroups per CU.
+//     rings at two workgroups per CU;
+//   * what every workgroup of a pixel range would do again is done once, before the launch:
+//     the taps are resolved into a table in tile order (resolve_tap_table_kernel) and only
+//     copied into the tap cache here, and the plain operand is cut into the MFMA fragments of
+//     each tile (to_plain_fragments_kernel), which a wave loads as contiguous kilobytes
+//     straight into its operand registers: no LDS tile, no barrier at a tile's start.
 // Partial sums leave in the layout of weight_grad_mfma_kernel.
+
 // The taps of a bilinear map resolved once for weight_grad_bf16_ring_kernel, in the order its
-// workgroups read them: table[tile of an image][tap][pixel of the tile][NA words of byte offsets into a
-// channel block (16 bytes per pixel), then NA words of weights as bf16 in the low half].  Every
+// workgroups read them: table[tile of an image][tap][pixel of the tile][NA words of byte
+// offsets into a channel block (16 bytes per pixel), then NA words of weights as bf16 in the
+// low half].  Every
 // workgroup of a pixel range (channel groups x tap passes) would otherwise resolve the same
 // taps from the map again, about a hundred instructions per tap, which is as much as its
 // products need.  Pixels outside the image weigh zero.  One workgroup per tile: its threads
