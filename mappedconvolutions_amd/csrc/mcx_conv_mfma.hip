@@ -1073,7 +1073,8 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
     const float *__restrict__ map, const float *__restrict__ iw, float *__restrict__ part, int A,
     int G, int GH, int GW, int MH, int MW, int K, int weighted, int wrap, int tiles_x,
     int tiles_per_img, int tw_shift, int total_tiles, int ranges, int cgroups,
-    float *__restrict__ plain_sum_part, const int *__restrict__ pair_mask, int run_if_leading) {
+    float *__restrict__ plain_sum_part, const int *__restrict__ pair_mask, int run_if_leading,
+    const uint4 *__restrict__ tap_table) {
   constexpr int NE = NP * NCORN;  // (offset, weight) pairs per pixel and tap
   static_assert(NA >= 1 && NA <= NE, "NA counts leading pairs");
   // two variants are launched, with NA == 2 (run_if_leading) and NA == NE; the map's mask of
@@ -1330,20 +1331,47 @@ __global__ __launch_bounds__(kThreads, NP * NCORN <= 4 ? 3 : 2) void weight_grad
       }
     };
 
+    // (two-pair taps of an image under fp32: resolved before the launch into a table in tile
+    // order, resolve_tap_table_kernel<2, 4, false>, and only copied into the tap cache)
+    constexpr bool kTable = sizeof(TD) == 4 && !CL && NA == 2 && NE == 4 && kCacheTaps;
     if (kCacheTaps) {
       // every wave has its A operands in registers: reuse the plain tile's LDS for the
       // resolved taps of this tile (thread (p, half) takes every other tap of pixel p)
       __syncthreads();
-      for (int k = half; k < ktaps; k += 2) {
-        unsigned o[NE];
-        float w_[NE];
-        resolve_tap(k_base + k, o, w_);
+      bool from_table = false;
+      if constexpr (kTable) {
+        if (tap_table) {
+          // (fetched only here: held across the plain tile's copy, the entries spill)
+          from_table = true;
+          const uint4 *te = tap_table + ((int64_t)t_in * K + k_base) * kTilePx + p;
+          constexpr int kTapsPerThread = (kWgKT + 1) / 2;
+          uint4 tap_entry[kTapsPerThread];
 #pragma unroll
-        for (int i = 0; i < NA; i++) {
-          TapOff[k][p][i] = o[i];
-          TapWt[k][p][i] = w_[i];
+          for (int t = 0; t < kTapsPerThread; t++)
+            tap_entry[t] = te[(int64_t)min(half + 2 * t, ktaps - 1) * kTilePx];
+#pragma unroll
+          for (int t = 0; t < kTapsPerThread; t++) {
+            const int k = half + 2 * t;
+            if (k < ktaps) {
+              *reinterpret_cast<uint2 *>(&TapOff[k][p][0]) =
+                  make_uint2(tap_entry[t].x, tap_entry[t].y);
+              *reinterpret_cast<uint2 *>(&TapWt[k][p][0]) =
+                  make_uint2(tap_entry[t].z, tap_entry[t].w);
+            }
+          }
         }
       }
+      if (!from_table)
+        for (int k = half; k < ktaps; k += 2) {
+          unsigned o[NE];
+          float w_[NE];
+          resolve_tap(k_base + k, o, w_);
+#pragma unroll
+          for (int i = 0; i < NA; i++) {
+            TapOff[k][p][i] = o[i];
+            TapWt[k][p][i] = w_[i];
+          }
+        }
       __syncthreads();
     }
 
@@ -1507,15 +1535,16 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(
 //     straight into its operand registers: no LDS tile, no barrier at a tile's start.
 // Partial sums leave in the layout of weight_grad_mfma_kernel.
 
-// The taps of a bilinear map resolved once for weight_grad_bf16_ring_kernel, in the order its
+// The taps of a bilinear map resolved once for a weight-gradient kernel, in the order its
 // workgroups read them: table[tile of an image][tap][pixel of the tile][NA words of byte
-// offsets into a channel block (16 bytes per pixel), then NA words of weights as bf16 in the
-// low half].  Every
+// offsets, then NA words of weights].  ESZ: bytes between neighbouring pixels of the gathered
+// operand (16 in a channel block, the element size in a plane); WBF: weights as bf16 in the low
+// half of the word (what weight_grad_bf16_ring_kernel multiplies by), else as fp32.  Every
 // workgroup of a pixel range (channel groups x tap passes) would otherwise resolve the same
-// taps from the map again, about a hundred instructions per tap, which is as much as its
-// products need.  Pixels outside the image weigh zero.  One workgroup per tile: its threads
-// walk the taps of their pixel two apart, so the tile's piece of the map stays in cache.
-template <int NA>
+// taps from the map again, about sixty instructions per tap, which is as much as its products
+// need.  Pixels outside the image weigh zero.  One workgroup per tile: its threads walk the
+// taps of their pixel two apart, so the tile's piece of the map stays in cache.
+template <int NA, int ESZ, bool WBF>
 __global__ __launch_bounds__(256) void resolve_tap_table_kernel(
     const float *__restrict__ map, unsigned *__restrict__ table, int GH, int GW, int MH, int MW,
     int K, int wrap, int tiles_x, int tw_shift, const int *__restrict__ pair_mask) {
@@ -1531,12 +1560,13 @@ __global__ __launch_bounds__(256) void resolve_tap_table_kernel(
   // (a weight as bf16 in the low half of a word, the high half zero: the form
   // v_dot2_f32_bf16 multiplies a word of two channels by to get the even one)
   auto wbits = [](float w) {
-    return __builtin_bit_cast(unsigned, __builtin_convertvector(floatx2{w, 0.f}, bf16x2));
+    return WBF ? __builtin_bit_cast(unsigned, __builtin_convertvector(floatx2{w, 0.f}, bf16x2))
+               : __builtin_bit_cast(unsigned, w);
   };
   for (int k = threadIdx.x >> 7; k < K; k += 2) {
     const float2 xy = entry[k];
     PairTap<4> t;
-    resolve_pairs<4, 16>(xy.x, xy.y, GH, GW, wrap != 0, live ? 1.f : 0.f, t);
+    resolve_pairs<4, ESZ>(xy.x, xy.y, GH, GW, wrap != 0, live ? 1.f : 0.f, t);
     uint4 *e = out + (int64_t)k * kTilePx * (NA / 2);
     if constexpr (NA == 2) {
       e[0] = make_uint4(t.off[0], t.off[1], wbits(t.wt[0]), wbits(t.wt[1]));
@@ -2605,6 +2635,8 @@ size_t mfma_weight_grad_bytes(int64_t B, int64_t A, int64_t G, int64_t MH, int64
     n += align256((size_t)(B * GH * GW * round_up(G, kGC)) * sizeof(float));
   else if (elem == 2)
     n += align256((size_t)(B * GH * GW * round_up(G, kGC)) * elem);
+  else  // fp32 images: the table of resolved two-pair taps (resolve_tap_table_kernel)
+    n += align256((size_t)make_tiling(B, MH, MW, 4).tiles_per_img * (size_t)K * kTilePx * 16);
   // bf16 images: the plain operand as MFMA fragments per pixel tile (to_plain_fragments_kernel)
   // and the table of resolved taps (resolve_tap_table_kernel, four pairs per tap at most)
   if (GH > 1 && elem == 2) {
@@ -2668,12 +2700,23 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
     else if (int rc = launch_pair_mask(map, iw, pair_mask, m, GH, GW, MH * MW * K, s))
       return rc;
   }
+  // fp32 images under single-point bilinear taps: the taps of the two-pair form resolved once
+  // (the table follows the pair mask in the scratch)
+  const uint4 *tap_table = nullptr;
+  if (sizeof(TD) == 4 && !cl && GH > 1 && m.np == 1 && m.mode != kInterpNearest && two_variants) {
+    unsigned *table = reinterpret_cast<unsigned *>((char *)pair_mask_ws + 256);
+    hipLaunchKernelGGL((resolve_tap_table_kernel<2, 4, false>), dim3((unsigned)t.tiles_per_img),
+                       dim3(256), 0, s, map, table, (int)GH, (int)GW, (int)MH, (int)MW, (int)K,
+                       m.wrap, t.tiles_x, t.tw_shift, pair_mask);
+    MCX_HIP_CHECK_LAUNCH();
+    tap_table = reinterpret_cast<const uint4 *>(table);
+  }
 #define MCX_LAUNCH_NA(NCORN, NP, CL, NA, MASK, LEAD)                                             \
   hipLaunchKernelGGL((weight_grad_mfma_kernel<TD, NCORN, NP, CL, NA>), grid, dim3(kThreads), 0,  \
                      s, plain, gath, map, iw, part, (int)A, (int)G, (int)GH, (int)GW, (int)MH,   \
                      (int)MW, (int)K, m.weighted, m.wrap, t.tiles_x, t.tiles_per_img,            \
                      t.tw_shift, (int)t.total, ranges, cgroups,                                  \
-                     plain_sum ? sum_part : (float *)nullptr, MASK, LEAD)
+                     plain_sum ? sum_part : (float *)nullptr, MASK, LEAD, tap_table)
 #define MCX_LAUNCH_CL(NCORN, NP, CL)                                          \
   if constexpr (NCORN * NP == 4) {                                            \
     if (!ring) {                                                              \
@@ -2709,10 +2752,10 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
       unsigned *table = reinterpret_cast<unsigned *>(
           (char *)tiles + align256((size_t)t.total * (size_t)round_up(A, 32) * kTilePx * sizeof(TD)));
       const dim3 rgrid((unsigned)t.tiles_per_img);
-      hipLaunchKernelGGL(resolve_tap_table_kernel<2>, rgrid, dim3(256), 0, s, map, table, (int)GH,
+      hipLaunchKernelGGL((resolve_tap_table_kernel<2, 16, true>), rgrid, dim3(256), 0, s, map, table, (int)GH,
                          (int)GW, (int)MH, (int)MW, (int)K, m.wrap, t.tiles_x, t.tw_shift,
                          pair_mask);
-      hipLaunchKernelGGL(resolve_tap_table_kernel<4>, rgrid, dim3(256), 0, s, map, table, (int)GH,
+      hipLaunchKernelGGL((resolve_tap_table_kernel<4, 16, true>), rgrid, dim3(256), 0, s, map, table, (int)GH,
                          (int)GW, (int)MH, (int)MW, (int)K, m.wrap, t.tiles_x, t.tw_shift,
                          pair_mask);
       MCX_HIP_CHECK_LAUNCH();
