@@ -757,7 +757,7 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_bf16_direct_kernel
   constexpr int kDepth = NA <= 2 ? 3 : 2;  // units whose loads are in flight
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
   __shared__ __attribute__((aligned(16))) unsigned TapOff[TG][kDgPx][NA];
-  __shared__ __attribute__((aligned(16))) unsigned TapW[TG][kDgPx][NPR];  // bf16 weights, two per word
+  __shared__ __attribute__((aligned(16))) unsigned TapW[TG][kDgPx][NA];  // bf16 weights as {w, 0}
   __shared__ __attribute__((aligned(16))) uint4 Wt[2][2][kOT * OG];
   if (gate && ((*gate == 0) != (run_if_zero != 0))) return;  // device-side path selection
   const int tid = threadIdx.x;
@@ -836,12 +836,13 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_bf16_direct_kernel
         }
 #pragma unroll
         for (int r = 0; r < NA; r++) TapOff[kl][tid][r] = off[r];
-        // entry r weighs w[r] (rounded to bf16, the precision of the samples themselves): the
-        // word of entries 2r and 2r + 1 holds both, lane-side shifts make {w, 0} and {0, w}
+        // entry r weighs w[r] (rounded to bf16, the precision of the samples themselves), kept
+        // as the word {w, 0} that weighs the even channel of a sample word; a lane-side shift
+        // makes the {0, w} of the odd one
 #pragma unroll
-        for (int r = 0; r < NPR; r++)
+        for (int r = 0; r < NA; r++)
           TapW[kl][tid][r] = __builtin_bit_cast(
-              unsigned, __builtin_convertvector(floatx2{wgt[2 * r], wgt[2 * r + 1]}, bf16x2));
+              unsigned, __builtin_convertvector(floatx2{wgt[r], 0.f}, bf16x2));
       }
     }
     __syncthreads();
@@ -853,7 +854,7 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_bf16_direct_kernel
     int ki = 0, ci = 0, ks = 0;
     // `offn`: the offsets of the unit whose loads are issued next; `wnext`: the packed weights
     // of the unit that is interpolated next (both read from LDS a step ahead)
-    unsigned offn[2][NA], wnext[2][NPR];
+    unsigned offn[2][NA], wnext[2][NA];
     auto fetch_offsets = [&]() __attribute__((always_inline)) {
 #pragma unroll
       for (int q = 0; q < 2; q++)
@@ -864,7 +865,7 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_bf16_direct_kernel
 #pragma unroll
       for (int q = 0; q < 2; q++)
 #pragma unroll
-        for (int r = 0; r < NPR; r++) wnext[q][r] = TapW[ks][px[q]][r];
+        for (int r = 0; r < NA; r++) wnext[q][r] = TapW[ks][px[q]][r];
     };
     auto issue_slot = [&](int d) __attribute__((always_inline)) {
       // (wave-uniform by construction; said so explicitly, or the loads get a loop over lanes)
@@ -894,9 +895,8 @@ __global__ __launch_bounds__(kThreads, 2) void gather_product_bf16_direct_kernel
         for (int r = 0; r < NPR; r++) {
           // a word of an entry holds channels 2j (low half) and 2j + 1 of its pixel: against
           // {w, 0} the dot product weighs the even channel, against {0, w} the odd one
-          const unsigned wp2 = wnext[q][r];
-          const unsigned w_even[2] = {wp2 & 0xffffu, wp2 >> 16};
-          const unsigned w_odd[2] = {wp2 << 16, wp2 & 0xffff0000u};
+          const unsigned w_even[2] = {wnext[q][2 * r], wnext[q][2 * r + 1]};
+          const unsigned w_odd[2] = {w_even[0] << 16, w_even[1] << 16};
 #pragma unroll
           for (int e = 0; e < 2; e++)
 #pragma unroll
