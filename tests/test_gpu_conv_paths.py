@@ -340,6 +340,33 @@ def test_bf16_backward_under_a_map_with_fractional_rows(radius, interp, device):
     assert_close_elementwise(gr[1].float(), g_o[1], 2e-2, "grad_weight")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("row_shift", [0.0, 0.37])
+def test_weight_gradient_with_staged_operands_over_ragged_channel_groups(row_shift, dtype, device):
+    """More plain channels than one workgroup takes (136 = 128 + 8: the second group's staged
+    fragments end after one slab), gathered channels that do not fill their last group, 25 taps
+    (three passes over a resolved-tap table, the last one short) and image sizes that leave
+    ragged pixel tiles, with integral map rows (two-pair forms, which read the tap tables) and
+    with fractional ones (four-pair forms): all three gradients against the oracle."""
+    B, Ci, Co, H, W, radius = 2, 40, 136, 14, 136, 2
+    K = (2 * radius + 1) ** 2
+    g = torch.Generator().manual_seed(99)
+    cast = lambda t: t.to(dtype)
+    x, gy = cast(torch.randn(B, Ci, H, W, generator=g)), cast(torch.randn(B, Co, H, W, generator=g))
+    w = cast(torch.randn(Co, Ci, K, generator=g) / (Ci * K) ** 0.5)
+    b = cast(torch.randn(Co, generator=g))
+    smap = synthetic.latitude_map(H, W, radius)
+    if row_shift:
+        smap[..., 1] = (smap[..., 1] + row_shift).clamp(0, H - 1)
+    g_o = O.mapped_conv_backward(gy.float(), smap, x.float(), w.float(), b.float(), K, 1)
+    xd, sd, wd_, bd, gyd = dev(x, smap, w, b, gy)
+    gr = _C.mapped_conv_backward(gyd, sd, xd, wd_, bd, K, 1)
+    tol = 2e-2 if dtype == torch.bfloat16 else 1e-5
+    for a, r, nm in zip(gr, g_o, ("grad_input", "grad_weight", "grad_bias")):
+        assert rel_err(a.float(), r) < tol, nm
+    assert_close_elementwise(gr[1].float(), g_o[1], tol, "grad_weight")
+
+
 @pytest.mark.parametrize("row_shift", [0.0, 0.5])
 @pytest.mark.parametrize("shape", [(1, 3, 5, 6, 16), (2, 1, 2, 3, 8), (1, 9, 17, 5, 264)])
 def test_bf16_backward_with_very_few_channels(shape, row_shift, device):
