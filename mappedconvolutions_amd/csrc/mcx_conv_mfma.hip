@@ -232,36 +232,54 @@ __global__ __launch_bounds__(256) void to_channel_blocks_kernel(const TD *__rest
 // fragment (mb, s4) holds, for lane (l15 = lane & 15, lq = lane >> 4), pixels 32 * s4 + 8 * lq
 // .. + 7 of channel 16 * mb + l15 of the slab.  A wave of that kernel then loads a fragment as
 // one contiguous kilobyte straight into its operand registers.
-// One workgroup: one slab of one tile through LDS (reads: 256-byte runs of a channel's row;
-// writes: the slab's 8 KB in one piece).  MW is a multiple of 8.
+// One workgroup: one slab of kFragTiles consecutive tiles through LDS (reads: runs of up to a
+// kilobyte of a channel's row; writes: each tile's slab, 8 KB, in one piece).  MW is a multiple
+// of 8.
+constexpr int kFragTiles = 4;
 __global__ __launch_bounds__(256) void to_plain_fragments_kernel(const bf16_t *__restrict__ y,
                                                                  bf16_t *__restrict__ yt, int A,
                                                                  int MH, int MW, int tiles_x,
                                                                  int tiles_per_img, int tw_shift) {
-  __shared__ __attribute__((aligned(16))) uint16_t T[32][kTilePx + 8];
-  const int tile = blockIdx.x, slab = blockIdx.y, b = blockIdx.z;
-  const int tile_y = tile / tiles_x, tile_x = tile - tile_y * tiles_x;
+  __shared__ __attribute__((aligned(16))) uint16_t T[kFragTiles][32][kTilePx + 8];
+  const int slab = blockIdx.y, b = blockIdx.z;
   const int px = (threadIdx.x & 15) * 8;
-  const int si = tile_y * (kTilePx >> tw_shift) + (px >> tw_shift);
-  const int sj = (tile_x << tw_shift) + (px & ((1 << tw_shift) - 1));
-  const bool inside = si < MH && sj < MW;
   const int64_t N = (int64_t)MH * MW;
+  uint4 v[kFragTiles][2];
 #pragma unroll
-  for (int h = 0; h < 2; h++) {
-    const int row = h * 16 + (threadIdx.x >> 4), a = slab * 32 + row;
-    uint4 v = make_uint4(0u, 0u, 0u, 0u);
-    if (inside && a < A)
-      v = *reinterpret_cast<const uint4 *>(y + ((int64_t)b * A + a) * N + (int64_t)si * MW + sj);
-    *reinterpret_cast<uint4 *>(&T[row][px]) = v;
+  for (int i = 0; i < kFragTiles; i++) {
+    const int tile = min((int)blockIdx.x * kFragTiles + i, tiles_per_img - 1);
+    const int tile_y = tile / tiles_x, tile_x = tile - tile_y * tiles_x;
+    const int si = tile_y * (kTilePx >> tw_shift) + (px >> tw_shift);
+    const int sj = (tile_x << tw_shift) + (px & ((1 << tw_shift) - 1));
+    const bool inside = si < MH && sj < MW;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      const int a = slab * 32 + h * 16 + (threadIdx.x >> 4);
+      v[i][h] = make_uint4(0u, 0u, 0u, 0u);
+      if (inside && a < A)
+        v[i][h] = *reinterpret_cast<const uint4 *>(y + ((int64_t)b * A + a) * N +
+                                                   (int64_t)si * MW + sj);
+    }
   }
-  __syncthreads();
-  uint4 *dst = reinterpret_cast<uint4 *>(yt) +
-               (((int64_t)b * tiles_per_img + tile) * gridDim.y + slab) * 512;
 #pragma unroll
-  for (int h = 0; h < 2; h++) {
-    const int o = h * 256 + threadIdx.x;  // (mb, s4, lane)
-    const int mb = o >> 8, s4 = (o >> 6) & 3, lane = o & 63;
-    dst[o] = *reinterpret_cast<const uint4 *>(&T[mb * 16 + (lane & 15)][32 * s4 + 8 * (lane >> 4)]);
+  for (int i = 0; i < kFragTiles; i++)
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+      *reinterpret_cast<uint4 *>(&T[i][h * 16 + (threadIdx.x >> 4)][px]) = v[i][h];
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < kFragTiles; i++) {
+    const int tile = blockIdx.x * kFragTiles + i;
+    if (tile >= tiles_per_img) break;
+    uint4 *dst = reinterpret_cast<uint4 *>(yt) +
+                 (((int64_t)b * tiles_per_img + tile) * gridDim.y + slab) * 512;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      const int o = h * 256 + threadIdx.x;  // (mb, s4, lane)
+      const int mb = o >> 8, s4 = (o >> 6) & 3, lane = o & 63;
+      dst[o] = *reinterpret_cast<const uint4 *>(
+          &T[i][mb * 16 + (lane & 15)][32 * s4 + 8 * (lane >> 4)]);
+    }
   }
 }
 
@@ -2744,7 +2762,8 @@ int mfma_weight_grad(const TD *plain, const TD *gath, const float *map, const fl
       bf16_t *tiles = reinterpret_cast<bf16_t *>(
           (char *)stage + align256((size_t)(B * GH * GW * Gpad) * sizeof(TD)));
       hipLaunchKernelGGL(to_plain_fragments_kernel,
-                         dim3((unsigned)t.tiles_per_img, (unsigned)((A + 31) / 32), (unsigned)B),
+                         dim3((unsigned)((t.tiles_per_img + kFragTiles - 1) / kFragTiles),
+                              (unsigned)((A + 31) / 32), (unsigned)B),
                          dim3(256), 0, s, reinterpret_cast<const bf16_t *>(plain), tiles, (int)A,
                          (int)MH, (int)MW, t.tiles_x, t.tiles_per_img, t.tw_shift);
       MCX_HIP_CHECK_LAUNCH();
