@@ -227,6 +227,22 @@ def plans(dev):
           flops=2 * flop)
     _line("unplanned headline conv backward fp32",
           _time(lambda: _C.mapped_conv_backward(gy, smap, x, w, b, K, 1)), flops=2 * flop)
+    del x, gy, w, b, smap, cplan
+    B, C, H, W, K = 16, 128, 512, 1024, 25
+    bf = torch.bfloat16
+    x = torch.randn(B, C, H, W, generator=g, dtype=bf).to(dev)
+    gy = torch.randn(B, C, H, W, generator=g, dtype=bf).to(dev)
+    w = (torch.randn(C, C, K, generator=g) / (C * K) ** 0.5).to(dev, bf)
+    b = torch.zeros(C, device=dev, dtype=bf)
+    smap = synthetic.latitude_map(H, W, 2).to(dev)
+    cplan = _C.conv_map_plan(smap, None, H, W, 1, bf)
+    flop = 2.0 * B * H * W * C * C * K
+    _line("planned config5 bf16 conv forward",
+          _time(lambda: _C.mapped_conv_forward(x, smap, w, b, K, 1, plan=cplan)),
+          flops=flop, peak_tflops=BF16_MFMA_TFLOPS)
+    _line("planned config5 bf16 conv backward",
+          _time(lambda: _C.mapped_conv_backward(gy, smap, x, w, b, K, 1, plan=cplan)),
+          flops=2 * flop, peak_tflops=BF16_MFMA_TFLOPS)
 
 
 def _launches(fn):
