@@ -566,6 +566,34 @@ def _picks(OH, OW, count, seed):
     return torch.tensor(sorted(set(p for p in fixed + rnd if p < n)), dtype=torch.int64)
 
 
+def test_config5_full_size_weight_gradient_two_ways(device):
+    """Configuration 5 at full size, weight gradient element by element: the fast form (staged
+    operands, tap table, 5 120 workgroups, images beyond 2^31 bytes) against the general kernel,
+    which the same call takes when grad_output is not 16-byte aligned.  The two differ in where
+    they round (bf16 interpolation weights in the fast form) and in the order of their fp32
+    sums, nothing else."""
+    B, C, H, W, K = 16, 128, 512, 1024, 25
+    smap = synthetic.latitude_map(H, W, 2).cuda()
+    torch.manual_seed(58)
+    x = torch.randn(B, C, H, W, device=device, dtype=torch.bfloat16)
+    w = (torch.randn(C, C, K, device=device) / (C * K) ** 0.5).bfloat16()
+    b = torch.zeros(C, device=device, dtype=torch.bfloat16)
+    n = B * C * H * W
+    buf = torch.empty(n + 8, device=device, dtype=torch.bfloat16)
+    buf[:n].copy_(torch.randn(n // 64, device=device).bfloat16().repeat(64))
+    gy = buf[:n].view(B, C, H, W)
+    assert gy.data_ptr() % 16 == 0
+    needs = (False, True, True)
+    _, gw_fast, gb_fast = _C.mapped_conv_backward(gy, smap, x, w, b, K, 1, needs=needs)
+    buf[1:n + 1].copy_(buf[:n].clone())
+    gy_off = buf[1:n + 1].view(B, C, H, W)
+    assert gy_off.data_ptr() % 16 != 0 and gy_off.is_contiguous()
+    _, gw_gen, gb_gen = _C.mapped_conv_backward(gy_off, smap, x, w, b, K, 1, needs=needs)
+    assert rel_err(gw_fast.float(), gw_gen.float()) < 2e-2
+    assert_close_elementwise(gw_fast.float(), gw_gen.float(), 2e-2, "grad_weight")
+    assert rel_err(gb_fast.float(), gb_gen.float()) < 2e-2
+
+
 @pytest.mark.parametrize("interp", [0, 1])
 def test_config2_full_size(interp, device):
     """The headline shape: B=8, 64 -> 64 channels, 256 x 512, 3 x 3 latitude map, fp32, nearest
